@@ -1,0 +1,236 @@
+"""Pins the oracle's group quantizer.
+
+Checks are chosen so that a plausible slip (wrong rounding mode, eps applied in the input
+dtype, a scale written to the wrong slot, an off-by-one exponent) fails at least one:
+  * torch's own CPU fp32 divide / multiply / float8 cast as an independent routine,
+    arranged like the reference's torch-native test helper
+    (python/sglang/test/test_block_fp8.py:23-48);
+  * the known-answer construction of test/srt/quant/test_fp8_kernel.py:24-45;
+  * closed forms and invariants (|q| <= 448, the amax element maps to +-448, zero groups);
+  * power-of-two scales: fp64 ceil(log2), exact powers of two and their 1-ulp neighbours;
+  * layout algebra: every layout unpacks to the same row-major scales, padding is zero.
+"""
+import math
+
+import pytest
+import torch
+
+from sglang_amd.workloads import make_activation
+
+FP8 = torch.float8_e4m3fn
+
+
+def _torch_group_quant(x, group, mode):
+    """fp32 torch restatement; eps clamp done in fp32 (both real kernels do that)."""
+    M, K = x.shape
+    xf = x.to(torch.float32).view(M, K // group, group)
+    amax = xf.abs().amax(-1, keepdim=True).clamp(min=1e-10)
+    if mode == "div":
+        s = amax / 448.0
+        t = xf / s
+    elif mode == "rcp":
+        s = amax / 448.0
+        t = xf * (1.0 / s)
+    else:
+        s = amax * torch.tensor(1.0 / 448.0, dtype=torch.float32)
+        t = xf * (torch.full_like(amax, 448.0) / amax)  # true division; `448.0 / t` is reciprocal()*448 in torch
+    q = t.clamp(-448.0, 448.0).to(FP8).view(M, K)
+    return q, s.view(M, K // group)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("mode", ["div", "rcp", "mul"])
+@pytest.mark.parametrize("group", [16, 64, 128, 256])
+def test_matches_torch_fp32_arithmetic(oracle, dtype, mode, group):
+    x = make_activation(37, 1024, seed=group + 7, dtype=dtype, zero_group_frac=0.02, group=group)
+    q, s = oracle.group_quant(x, group, mode=mode)
+    q_t, s_t = _torch_group_quant(x, group, mode)
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32))
+    assert torch.equal(q.view(torch.uint8), q_t.view(torch.uint8))
+
+
+def test_modes_differ_somewhere_but_only_by_one_code(oracle):
+    # guards against the three modes being wired to the same arithmetic
+    x = make_activation(256, 2048, seed=3)
+    q = {m: oracle.group_quant(x, 128, mode=m)[0].view(torch.uint8).to(torch.int16) for m in ("div", "rcp", "mul")}
+    for a, b in (("div", "rcp"), ("div", "mul")):
+        d = (q[a] - q[b]).abs()
+        assert 0 < int((d != 0).sum()) < 0.005 * d.numel()
+        assert int(d.max()) == 1
+
+
+def _known_answer(M, K, group, seed):
+    """q_gt on the fp8 grid with |max| = 448 per group; scale with a short mantissa so that
+    q_gt * scale, 448 * scale and (448 * scale) / 448 are all exact in fp32."""
+    g = torch.Generator().manual_seed(seed)
+    qa = torch.rand(M, K // group, group, generator=g) * 2 - 1
+    qa = qa * (448.0 / qa.abs().amax(-1, keepdim=True))
+    q_gt = qa.clamp(-448, 448).to(FP8)
+    # make sure each group really contains +-448
+    assert bool((q_gt.to(torch.float32).abs().amax(-1) == 448).all())
+    mant = torch.randint(1, 1 << 11, (M, K // group), generator=g).to(torch.float32)
+    expo = torch.randint(-20, 4, (M, K // group), generator=g).to(torch.float32)
+    scale = mant * torch.exp2(expo)
+    x = (q_gt.to(torch.float32) * scale[..., None]).view(M, K)
+    return x, q_gt.view(M, K), scale
+
+
+@pytest.mark.parametrize("mode", ["div", "rcp", "mul"])
+def test_known_answer_construction(oracle, mode):
+    x, q_gt, scale = _known_answer(64, 512, 128, seed=11)
+    q, s = oracle.group_quant(x, 128, mode=mode)
+    if mode == "mul":  # amax * (1/448f) is rounded twice; the reference's own test allows 1.3e-6 relative
+        torch.testing.assert_close(s, scale)
+    else:
+        assert torch.equal(s, scale)
+    assert torch.equal(q.view(torch.uint8), q_gt.view(torch.uint8))
+
+
+def test_invariants_and_zero_groups(oracle):
+    x = make_activation(128, 1024, seed=5, zero_group_frac=0.05)
+    xf = x.to(torch.float32).view(128, 8, 128)
+    zero = xf.abs().amax(-1) == 0
+    assert zero.any()
+    for mode in ("div", "rcp", "mul"):
+        q, s = oracle.group_quant(x, 128, mode=mode)
+        qf = q.to(torch.float32).view(128, 8, 128)
+        assert not torch.isnan(qf).any() and float(qf.abs().max()) <= 448.0
+        # zero groups: q == 0 and the scale is eps/448 (mode mul: eps * (1/448))
+        assert bool((qf[zero] == 0).all())
+        want = (torch.tensor(1e-10) / 448.0) if mode != "mul" else torch.tensor(1e-10) * torch.tensor(1.0 / 448.0)
+        assert bool((s[zero] == want).all())
+        # scale closed form on the other groups
+        amax = xf.abs().amax(-1)
+        want_s = amax / 448.0 if mode != "mul" else amax * torch.tensor(1.0 / 448.0)
+        assert torch.equal(s[~zero], want_s[~zero])
+    # in DIV mode the element that attains amax is exactly +-448
+    q, _ = oracle.group_quant(x, 128, mode="div")
+    qf = q.to(torch.float32).view(128, 8, 128)
+    idx = xf.abs().argmax(-1, keepdim=True)
+    top = qf.gather(-1, idx).squeeze(-1).abs()
+    assert bool((top[~zero] == 448).all())
+
+
+def test_eps_is_applied_in_fp32_not_in_the_input_dtype(oracle):
+    # bf16(1e-10) != 1e-10f; a group whose amax is below eps must give exactly 1e-10f/448
+    x = torch.full((1, 128), 3e-11, dtype=torch.bfloat16)
+    _, s = oracle.group_quant(x, 128, mode="div")
+    assert float(s[0, 0]) == float(torch.tensor(1e-10) / 448.0)
+
+
+def test_int8_destination_truncates(oracle):
+    x = make_activation(32, 512, seed=9)
+    q, s = oracle.group_quant(x, 128, mode="div", dst_dtype=torch.int8)
+    xf = x.to(torch.float32).view(32, 4, 128)
+    amax = xf.abs().amax(-1, keepdim=True).clamp(min=1e-10)
+    s_t = amax / 127.0
+    q_t = (xf / s_t).clamp(-128, 127).to(torch.int8).view(32, 512)  # torch's float->int8 cast truncates toward zero
+    assert torch.equal(s, s_t.view(32, 4)) and torch.equal(q, q_t)
+    frac = (xf / s_t).view(32, 512)
+    assert bool((q.to(torch.float32).abs() <= frac.abs()).all())  # never rounds away from zero
+
+
+# ---------------------------------------------------------------- power-of-two scales
+
+def _positive_normal_bf16():
+    bits = torch.arange(0x0080, 0x7F80, dtype=torch.int32).to(torch.int16)
+    return bits.view(torch.bfloat16)
+
+
+def test_ue8m0_exponent_for_every_positive_normal_bf16_amax(oracle):
+    amax = _positive_normal_bf16()
+    amax = amax[amax.to(torch.float32) >= 1e-10]  # below eps the group behaves like a zero group
+    M = amax.numel()
+    x = torch.zeros(M, 128, dtype=torch.bfloat16)
+    x[:, 5] = amax
+    want = torch.ceil(torch.log2(amax.to(torch.float64) / 448.0)).to(torch.int64) + 127
+    for mode in ("mul", "div", "rcp"):
+        _, s = oracle.group_quant(x, 128, mode=mode, layout="ue8m0")
+        got = oracle.unpack_ue8m0(s, 1).view(-1).to(torch.int64)
+        assert torch.equal(got, want), mode
+
+
+def test_ue8m0_powers_of_two_and_neighbours(oracle):
+    # amax = 448 * 2^k (fp32 input so that 1-ulp neighbours exist) -> exactly 2^k; one ulp above -> 2^(k+1)
+    ks = torch.arange(-30, 30)
+    amax = 448.0 * torch.exp2(ks.to(torch.float32))
+    up = torch.nextafter(amax, torch.tensor(float("inf")))
+    dn = torch.nextafter(amax, torch.tensor(0.0))
+    for vals, want in ((amax, ks + 127), (up, ks + 128), (dn, ks + 127)):
+        x = torch.zeros(len(ks), 128, dtype=torch.float32)
+        x[:, 0] = -vals
+        for mode in ("div", "mul"):
+            _, s = oracle.group_quant(x, 128, mode=mode, layout="ue8m0")
+            got = oracle.unpack_ue8m0(s, 1).view(-1).to(torch.int64)
+            if mode == "mul" and vals is dn:
+                # amax*(1/448f) rounds; the reference's v2 kernel has the same property, so only bound it
+                assert bool(((got - want).abs() <= 1).all())
+            else:
+                assert torch.equal(got, want), (mode,)
+
+
+def test_ue8m0_zero_group_bytes(oracle):
+    x = torch.zeros(4, 512, dtype=torch.bfloat16)
+    _, s = oracle.group_quant(x, 128, mode="mul", layout="ue8m0")
+    assert set(oracle.unpack_ue8m0(s, 4).view(-1).tolist()) == {85}  # 1e-10/448 = 2^-42.03 -> 2^-42
+    _, s = oracle.group_quant(x, 128, mode="div", layout="ue8m0", pow2_floor=1e-10)
+    assert set(oracle.unpack_ue8m0(s, 4).view(-1).tolist()) == {94}  # ceil(log2(1e-10)) = -33
+    assert math.ceil(math.log2(1e-10 / 448)) + 127 == 85 and math.ceil(math.log2(1e-10)) + 127 == 94
+
+
+def test_pow2_scales_make_all_modes_identical(oracle):
+    x = make_activation(64, 1024, seed=21, zero_group_frac=0.05)
+    outs = [oracle.group_quant(x, 128, mode=m, layout="ue8m0") for m in ("div", "rcp", "mul")]
+    for q, s in outs[1:]:
+        assert torch.equal(q.view(torch.uint8), outs[0][0].view(torch.uint8))
+        assert torch.equal(s, outs[0][1])
+    # and q equals x / 2^e computed independently
+    e = oracle.unpack_ue8m0(outs[0][1], 8).to(torch.float32) - 127
+    t = (x.to(torch.float32).view(64, 8, 128) / torch.exp2(e)[..., None]).clamp(-448, 448)
+    assert torch.equal(outs[0][0].view(torch.uint8), t.to(FP8).view(64, 1024).view(torch.uint8))
+
+
+# ---------------------------------------------------------------- scale layouts
+
+@pytest.mark.parametrize("M,K", [(1, 128), (5, 640), (16, 7168), (127, 384), (130, 1664)])
+def test_layouts_hold_the_same_scales(oracle, M, K):
+    x = make_activation(M, K, seed=M + K)
+    q0, s_row = oracle.group_quant(x, 128, mode="div", layout="row")
+    assert s_row.is_contiguous() and tuple(s_row.shape) == (M, K // 128)
+    for layout in ("col", "col_aligned"):
+        q, s = oracle.group_quant(x, 128, mode="div", layout=layout)
+        assert tuple(s.shape) == (M, K // 128)
+        assert s.stride(0) == 1 and s.stride(1) == (M if layout == "col" else (M + 3) // 4 * 4)
+        assert torch.equal(s, s_row) and torch.equal(q.view(torch.uint8), q0.view(torch.uint8))
+
+
+@pytest.mark.parametrize("M,K", [(1, 128), (5, 640), (16, 7168), (127, 384), (130, 1664)])
+def test_packed_layout_algebra(oracle, M, K):
+    G = K // 128
+    x = make_activation(M, K, seed=M * 3 + K)
+    _, s = oracle.group_quant(x, 128, mode="mul", layout="ue8m0")
+    assert s.dtype == torch.int32 and tuple(s.shape) == (M, (G + 3) // 4)
+    assert s.stride(0) == 1 and s.stride(1) == (M + 3) // 4 * 4
+    # bytes -> exponents -> the same power-of-two scales as the unpacked computation
+    xf = x.to(torch.float32).view(M, G, 128)
+    t = xf.abs().amax(-1).clamp(min=1e-10) * torch.tensor(1.0 / 448.0)
+    want = torch.ceil(torch.log2(t.to(torch.float64))).to(torch.int64) + 127
+    assert torch.equal(oracle.unpack_ue8m0(s, G).to(torch.int64), want)
+    by = oracle.unpack_ue8m0(s, 4 * s.shape[1])
+    assert bool((by[:, G:] == 0).all())  # padding bytes of the last word are zero
+    # word w of row m sits at element offset w * align4(M) + m of the underlying storage
+    base = s.as_strided((s.stride(1) * s.shape[1],), (1,))
+    for m in (0, M - 1):
+        for w in (0, s.shape[1] - 1):
+            assert int(base[w * s.stride(1) + m]) == int(s[m, w])
+
+
+def test_per_token_quant_int8(oracle):
+    x = make_activation(64, 4096, seed=31)
+    q, s = oracle.per_token_quant_int8(x)
+    xf = x.to(torch.float32)
+    amax = xf.abs().amax(1, keepdim=True).clamp(min=1e-10)
+    t = xf * (torch.full_like(amax, 127.0) / amax)
+    want = (torch.sign(t) * torch.floor(t.abs() + 0.5)).to(torch.int8)  # round half away from zero
+    assert torch.equal(q, want) and torch.equal(s, amax / 127.0)
+    assert int(q.abs().max()) == 127
