@@ -1,0 +1,138 @@
+/*
+ * mi355_qlinear -- C ABI of the MI355X (gfx950) quantized-linear kernels.
+ *
+ * One shared library, plain pointers and sizes, no framework types.  Every pointer
+ * is a device pointer unless stated otherwise; every call only enqueues work on
+ * `stream` (a hipStream_t passed as void*, NULL = the default stream) and returns
+ * without synchronizing, so all entry points are usable inside HIP graph capture.
+ * The library never allocates or frees device memory: outputs and workspaces are
+ * the caller's.
+ *
+ * Return value: 0 on success, otherwise one of the MI355_ERR_* codes; the message
+ * for the calling thread is available from mi355_last_error().
+ *
+ * Each entry point names the reference interface it stands in for (paths relative
+ * to the SGLang source tree).
+ */
+#ifndef MI355_QLINEAR_H
+#define MI355_QLINEAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_QLINEAR_ABI_VERSION 1
+
+/* Element types (values are part of the ABI). */
+enum {
+  MI355_F32 = 0,
+  MI355_F16 = 1,
+  MI355_BF16 = 2,
+  MI355_FP8_E4M3FN = 3, /* OCP E4M3: max 448, no infinity, 0x7f/0xff NaN */
+  MI355_I8 = 4,
+  MI355_I32 = 5
+};
+
+/* How the group quantizer scales an element once the group's amax is known. */
+enum {
+  MI355_QUANT_DIV = 0, /* s = amax / qmax;          q = x / s           (per_token_group_quant_8bit.cu:86,:110) */
+  MI355_QUANT_RCP = 1, /* s = amax / qmax;          q = x * (1.0f / s)  (fp8_kernel.py:156-158)                */
+  MI355_QUANT_MUL = 2  /* s = amax * (1.0f / qmax); q = x * (qmax/amax) (per_token_group_quant_8bit_v2.cu:77-78) */
+};
+
+/* What is stored per group. */
+enum {
+  MI355_SCALE_F32 = 0,         /* float at s[row * s_stride_row + kgroup * s_stride_col]                       */
+  MI355_SCALE_UE8M0_PACKED = 1 /* biased exponent byte of a power-of-two scale, four consecutive k-groups per
+                                  32-bit word, words column-major: byte address
+                                  (kgroup/4) * s_stride_col * 4 + row * 4 + kgroup % 4; the unused bytes of a
+                                  row's last word are written as zero
+                                  (per_token_group_quant_8bit.cu:54-61, per_token_group_quant_8bit_v2.cu:305-329) */
+};
+
+enum {
+  MI355_OK = 0,
+  MI355_ERR_INVALID_ARGUMENT = 1, /* a shape, stride, alignment or enum the contract excludes */
+  MI355_ERR_UNSUPPORTED = 2,      /* valid in the reference, not implemented here             */
+  MI355_ERR_LAUNCH = 3,           /* the HIP runtime refused the launch                       */
+  MI355_ERR_WORKSPACE = 4         /* workspace missing or smaller than *_workspace_bytes()     */
+};
+
+int mi355_qlinear_abi_version(void);
+
+/* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the next call. */
+const char* mi355_last_error(void);
+
+/*
+ * Per-token-group 8-bit quantization.
+ * Replaces sgl_per_token_group_quant_8bit    (sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:116-217),
+ *          sgl_per_token_group_quant_8bit_v2 (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:394-514,
+ *                                             without its MoE-only silu/masked variants),
+ *          and the Triton kernels behind per_token_group_quant_fp8
+ *                                            (python/sglang/srt/layers/quantization/fp8_kernel.py:121-323).
+ *
+ *   x        [M, K] contiguous, x_dtype in {F32, F16, BF16}
+ *   q        [M, K] contiguous, q_dtype FP8_E4M3FN (round to nearest even) or I8 (truncation toward zero)
+ *   s        scales, see scale_kind; caller-allocated, written in place
+ *   group    elements per scale along K; a power of two with group * sizeof(x element) in [16, 2048] bytes,
+ *            dividing K
+ *   amax = max(eps, max |x|) in fp32; q is clamped to [qmin, qmax] before conversion
+ *   pow2_floor  only for UE8M0 with DIV/RCP: lower bound on amax/qmax before rounding up to a power of two
+ *            (1e-10f reproduces per_token_group_quant_8bit.cu:88; 0 reproduces fp8_kernel.py:207-208)
+ */
+int mi355_group_quant_8bit(const void* x, int x_dtype, void* q, int q_dtype, void* s, int64_t M, int64_t K,
+                           int group, float eps, float qmin, float qmax, int mode, int scale_kind,
+                           float pow2_floor, int64_t s_stride_row, int64_t s_stride_col, void* stream);
+
+/*
+ * Blockwise-scaled FP8 GEMM:  out[m,n] = cast( sum_kb (sum_{k in kb} a[m,k] * b[n,k]) * sa[m,kb] * sb[n/128,kb] ).
+ * Replaces fp8_blockwise_scaled_mm (sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:368-465) and
+ *          w8a8_block_fp8_matmul   (python/sglang/srt/layers/quantization/fp8_kernel.py:691-773, :1068-1164).
+ *
+ *   a   [M, K] e4m3fn, K contiguous, row stride lda (bytes == elements)
+ *   b   [N, K] e4m3fn, K contiguous, row stride ldb: the weight as stored.  The reference's column-major
+ *       `mat_b [K, N]` (stride(0) == 1) is this same memory with ldb = mat_b.stride(1).
+ *   sa  fp32, element (m, kb) at sa[m * sa_sm + kb * sa_sk], kb < ceil(K/128)
+ *   sb  fp32, element (nb, kb) at sb[nb * sb_sn + kb * sb_sk], nb < ceil(N/128)
+ *   out [M, N] BF16, F16 or F32, row stride ldo
+ *   K and N need not be multiples of 128 (ragged last blocks are masked like fp8_kernel.py:738-751).
+ *   workspace: at least mi355_fp8_blockwise_mm_workspace_bytes(M, N, K) bytes of device memory (may be NULL
+ *   when that is 0); used for split-K partial sums, contents undefined afterwards.
+ */
+size_t mi355_fp8_blockwise_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const float* sb, void* out, int out_dtype,
+                           int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t sa_sm, int64_t sa_sk,
+                           int64_t sb_sn, int64_t sb_sk, int64_t ldo, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/*
+ * Per-token x per-channel INT8 GEMM:  acc = sum_k a[m,k] * b[n,k] exactly in int32;
+ *   out[m,n] = cast( f32(acc) * (sb[n] * sa[m]) + f32(bias[n]) ).
+ * Replaces int8_scaled_mm (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; epilogue order of
+ *          sgl-kernel/csrc/cutlass_extensions/epilogue/epilogue_per_row_per_col_scale.h:273-303).
+ *
+ *   a [M, K] int8 row stride lda;  b [N, K] int8 row stride ldb (the reference's column-major mat_b [K, N]);
+ *   sa [M], sb [N] fp32 contiguous; bias NULL or [N] in the output dtype; out [M, N] BF16/F16 row stride ldo.
+ *   out_dtype MI355_I32 writes the raw accumulators instead (sa, sb, bias ignored): the hook that lets a
+ *   test prove the accumulation exact before any rounding.
+ */
+size_t mi355_int8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_int8_scaled_mm(const void* a, const void* b, const float* sa, const float* sb, const void* bias, void* out,
+                         int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldo,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Per-token INT8 activation quantization: absmax = max(1e-10, max |x[m,:]|), s[m] = absmax / 127,
+ * q = round-half-away-from-zero(x * (127 / absmax)).
+ * Replaces per_token_quant_int8 (python/sglang/srt/layers/quantization/int8_kernel.py:28-89, without cal_sum).
+ *   x [M, K] contiguous F32/F16/BF16; q [M, K] int8 contiguous; s [M] fp32.  K * sizeof(x element) % 16 == 0.
+ */
+int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_QLINEAR_H */

@@ -1,0 +1,86 @@
+"""Loader of ``libmi355_qlinear.so`` and typed ctypes prototypes of its C ABI.
+
+There is no fallback: if the library is missing the import of any operator fails with a
+clear message.  ``include/mi355_qlinear.h`` is the authoritative declaration; the prototypes
+below mirror it one to one.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(_CSRC, "libmi355_qlinear.so")
+ABI_VERSION = 1
+
+# enum values of include/mi355_qlinear.h
+F32, F16, BF16, FP8_E4M3FN, I8, I32 = range(6)
+QUANT_DIV, QUANT_RCP, QUANT_MUL = range(3)
+SCALE_F32, SCALE_UE8M0_PACKED = range(2)
+
+EXPORTS = (
+    "mi355_qlinear_abi_version",
+    "mi355_last_error",
+    "mi355_group_quant_8bit",
+    "mi355_fp8_blockwise_mm_workspace_bytes",
+    "mi355_fp8_blockwise_mm",
+    "mi355_int8_scaled_mm_workspace_bytes",
+    "mi355_int8_scaled_mm",
+    "mi355_per_token_quant_int8",
+)
+
+_lib = None
+
+
+class Mi355Error(RuntimeError):
+    """A C-ABI call returned a non-zero status; the message is the library's own."""
+
+
+def build() -> str:
+    """Compile the library in-tree with the Makefile beside the sources (cross-compiles without a GPU)."""
+    import subprocess
+
+    subprocess.run(["make", "-C", _CSRC, "-B", "-j8", "libmi355_qlinear.so"], check=True)
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C {_CSRC}` (or __graft_entry__.build()). "
+            "The quantized-linear operators have no other implementation."
+        )
+    L = ctypes.CDLL(LIB_PATH)
+    i64, i32, f32, vp, sz = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+    L.mi355_qlinear_abi_version.restype = i32
+    L.mi355_last_error.restype = ctypes.c_char_p
+    L.mi355_group_quant_8bit.argtypes = [vp, i32, vp, i32, vp, i64, i64, i32, f32, f32, f32, i32, i32, f32, i64, i64, vp]
+    L.mi355_group_quant_8bit.restype = i32
+    L.mi355_fp8_blockwise_mm_workspace_bytes.argtypes = [i64, i64, i64]
+    L.mi355_fp8_blockwise_mm_workspace_bytes.restype = sz
+    L.mi355_fp8_blockwise_mm.argtypes = [vp, vp, vp, vp, vp, i32] + [i64] * 10 + [vp, sz, vp]
+    L.mi355_fp8_blockwise_mm.restype = i32
+    L.mi355_int8_scaled_mm_workspace_bytes.argtypes = [i64, i64, i64]
+    L.mi355_int8_scaled_mm_workspace_bytes.restype = sz
+    L.mi355_int8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32] + [i64] * 6 + [vp, sz, vp]
+    L.mi355_int8_scaled_mm.restype = i32
+    L.mi355_per_token_quant_int8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
+    L.mi355_per_token_quant_int8.restype = i32
+    got = L.mi355_qlinear_abi_version()
+    if got != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}: rebuild it")
+    _lib = L
+    return L
+
+
+def check(status: int) -> None:
+    """Raise the library's message as RuntimeError (NotImplementedError for unsupported cases)."""
+    if status == 0:
+        return
+    msg = lib().mi355_last_error().decode("utf-8", "replace")
+    if status == 2:
+        raise NotImplementedError(msg)
+    raise Mi355Error(msg)

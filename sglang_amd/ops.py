@@ -1,0 +1,279 @@
+"""PyTorch-ROCm custom operators ``torch.ops.sgl_kernel.*`` backed by the gfx950 C ABI.
+
+The operator names and schema strings are the reference's own
+(sgl-kernel/csrc/common_extension.cc:158-181); the implementations are registered for the
+``CUDA`` dispatch key, which is the HIP device under PyTorch-ROCm.  Each implementation
+checks its arguments the way the reference's host function does (same conditions, same
+wording, RuntimeError), allocates outputs and workspaces through torch's caching allocator
+(so nothing here breaks HIP graph capture) and passes raw device pointers plus the current
+stream to ``libmi355_qlinear.so``.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+
+_DT = {
+    torch.float32: _lib.F32,
+    torch.float16: _lib.F16,
+    torch.bfloat16: _lib.BF16,
+    torch.float8_e4m3fn: _lib.FP8_E4M3FN,
+    torch.int8: _lib.I8,
+    torch.int32: _lib.I32,
+}
+
+SCHEMAS = {
+    "int8_scaled_mm": "int8_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, "
+    "ScalarType out_dtype, Tensor? bias) -> Tensor",
+    "fp8_blockwise_scaled_mm": "fp8_blockwise_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, "
+    "Tensor scales_b, ScalarType out_dtype) -> Tensor",
+    "sgl_per_token_group_quant_8bit": "sgl_per_token_group_quant_8bit(Tensor input, Tensor output_q, "
+    "Tensor output_s, int group_size, float eps, float fp8_min, float fp8_max, bool scale_ue8m0) -> ()",
+    "sgl_per_token_group_quant_8bit_v2": "sgl_per_token_group_quant_8bit_v2(Tensor input, Tensor output_q, "
+    "Tensor output_s, int group_size, float eps, float fp8_min, float fp8_max, bool scale_ue8m0, "
+    "bool fuse_silu_and_mul, Tensor? masked_m) -> ()",
+}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_input(t: torch.Tensor, name: str) -> None:
+    # CHECK_INPUT of sgl-kernel/include/utils.h:193-212
+    _require(t.is_cuda, f"{name} must be a CUDA tensor")
+    _require(t.is_contiguous(), f"{name} must be contiguous")
+
+
+# ---------------------------------------------------------------- group quantizer
+
+def _group_quant(input, output_q, output_s, group_size, eps, qmin, qmax, scale_ue8m0, mode, pow2_floor, op):
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _require(input.numel() % group_size == 0, f"CHECK_EQ(input.numel() % group_size, 0) failed in {op}")
+    _require(output_s.dim() == 2, f"CHECK_EQ(output_s.dim(), 2) failed in {op}")
+    _require(input.dtype in (torch.float32, torch.float16, torch.bfloat16), f"{op}: unsupported input dtype {input.dtype}")
+    _require(output_q.dtype in (torch.float8_e4m3fn, torch.int8), f"{op}: unsupported output dtype {output_q.dtype}")
+    _require(output_q.numel() == input.numel(), f"{op}: output_q must have as many elements as input")
+    if input.numel() == 0:
+        return
+    K = input.size(-1)
+    M = input.numel() // K
+    _require(K % group_size == 0, f"{op}: the last dimension must be divisible by group_size")
+    # same test as per_token_group_quant_8bit.cu:153 / per_token_group_quant_8bit_v2.cu:426
+    column_major = output_s.stride(0) < output_s.stride(1)
+    if scale_ue8m0:
+        _require(column_major, f"{op}: scale_ue8m0 needs column-major scales")
+        _require(output_s.dtype == torch.int32, f"{op}: packed UE8M0 scales are stored in an int32 tensor")
+        kind, s_row, s_col = _lib.SCALE_UE8M0_PACKED, 1, output_s.stride(1)
+    else:
+        _require(output_s.dtype == torch.float32, f"{op}: output_s must be float32")
+        kind = _lib.SCALE_F32
+        # row-major scales are addressed by the flat group index, as in the reference kernels
+        s_row, s_col = (1, output_s.stride(1)) if column_major else (K // group_size, 1)
+    check(
+        lib().mi355_group_quant_8bit(
+            input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), _DT[output_q.dtype], output_s.data_ptr(),
+            M, K, group_size, eps, qmin, qmax, mode, kind, pow2_floor, s_row, s_col, _stream(),
+        )
+    )
+
+
+def sgl_per_token_group_quant_8bit(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0):
+    """sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:116-217: q = x / (amax / max)."""
+    _group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0,
+                 _lib.QUANT_DIV, 1e-10, "sgl_per_token_group_quant_8bit")
+
+
+def sgl_per_token_group_quant_8bit_v2(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0,
+                                      fuse_silu_and_mul, masked_m):
+    """sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:394-514: q = x * (max / amax)."""
+    op = "sgl_per_token_group_quant_8bit_v2"
+    if fuse_silu_and_mul or masked_m is not None:
+        raise NotImplementedError(f"{op}: fuse_silu_and_mul / masked_m (expert-parallel MoE layouts) are not built")
+    _require(input.numel() > 0, f"{op}: input.numel() > 0")
+    _require(abs(1e-10 - eps) < 1e-13, f"{op}: eps must be 1e-10")
+    _require(group_size in (16, 32, 64, 128), "Unsupported group_size")
+    _require(input.dtype in (torch.float16, torch.bfloat16), f"{op}: input must be float16 or bfloat16")
+    want = (-448.0, 448.0) if output_q.dtype == torch.float8_e4m3fn else (-128.0, 127.0)
+    _require((fp8_min, fp8_max) == want, f"{op}: CHECK_EQ(dst_dtype_info::MIN/MAX, min_8bit/max_8bit) failed")
+    _group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, _lib.QUANT_MUL, 0.0, op)
+
+
+# ---------------------------------------------------------------- blockwise FP8 GEMM
+
+def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
+    """sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:368-465."""
+    _require(mat_a.is_cuda, "mat_a must be a CUDA tensor")
+    _require(mat_b.is_cuda, "mat_b must be a CUDA tensor")
+    _require(mat_a.dim() == 2, "mat_a must be a 2D tensor")
+    _require(mat_b.dim() == 2, "mat_b must be a 2D tensor")
+    _require(mat_a.stride(1) == 1, "mat_a must be a row major tensor")
+    _require(mat_b.stride(0) == 1, "mat_b must be a column major tensor")
+    _require(mat_a.size(1) == mat_b.size(0), "mat_a and mat_b shapes cannot be multiplied")
+    _require((mat_a.size(1) * mat_a.element_size()) % 16 == 0, "mat_a must be multiple of 16 bytes for memory alignment")
+    _require((mat_b.size(0) * mat_b.element_size()) % 16 == 0, "mat_b must be multiple of 16 bytes for memory alignment")
+    _require(mat_a.dtype == torch.float8_e4m3fn, "mat_a must be Float8_e4m3fn")
+    _require(mat_b.dtype == torch.float8_e4m3fn, "mat_b must be Float8_e4m3fn")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be Half or BFloat16")
+
+    def is_contiguous_vector(t):
+        return t.is_contiguous() and (t.dim() == 1 or (t.dim() == 2 and min(t.shape) == 1))
+
+    M, K = mat_a.shape
+    N = mat_b.size(1)
+    _require(scales_a.dim() == 2 and scales_b.dim() == 2, "scales must be 2D tensors")
+    _require(M == scales_a.size(0), "size of scales_a is not matched")
+    _require(K // 128 == scales_a.size(1), "size of scales_a is not matched")
+    _require(scales_a.stride(0) == 1 or is_contiguous_vector(scales_a), "scales_a must be M major")
+    _require(K // 128 == scales_b.size(0), "size of scales_b is not matched")
+    _require(N // 128 == scales_b.size(1), "size of scales_b is not matched")
+    _require(scales_b.stride(0) == 1 or is_contiguous_vector(scales_b), "scales_b must be K major")
+    _require(scales_a.dtype == torch.float32, "scales_a must be Float32")
+    _require(scales_b.dtype == torch.float32, "scales_b must be Float32")
+    _require((N * torch.empty((), dtype=out_dtype).element_size()) % 16 == 0,
+             "out must be multiple of 16 bytes for memory alignment")
+    # the integer divisions above accept ragged K or N but leave the tail without scales
+    _require(K % 128 == 0 and N % 128 == 0, "fp8_blockwise_scaled_mm needs K and N to be multiples of 128")
+    out = torch.empty((M, N), dtype=out_dtype, device=mat_a.device)
+    if M == 0:
+        return out
+    _launch_fp8_mm(mat_a, mat_b.data_ptr(), mat_b.stride(1), scales_a, scales_b.data_ptr(),
+                   scales_b.stride(1), scales_b.stride(0), out, M, N, K)
+    return out
+
+
+def _launch_fp8_mm(a, b_ptr, ldb, sa, sb_ptr, sb_sn, sb_sk, out, M, N, K):
+    L = lib()
+    ws_bytes = L.mi355_fp8_blockwise_mm_workspace_bytes(M, N, K)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+    check(
+        L.mi355_fp8_blockwise_mm(
+            a.data_ptr(), b_ptr, sa.data_ptr(), sb_ptr, out.data_ptr(), _DT[out.dtype], M, N, K,
+            a.stride(0), ldb, sa.stride(0), sa.stride(1), sb_sn, sb_sk, out.stride(0),
+            ws.data_ptr() if ws is not None else None, ws_bytes, _stream(),
+        )
+    )
+
+
+def block_fp8_matmul(A2d, B, As2d, Bs, out2d):
+    """The ``w8a8_block_fp8_matmul`` contract on flattened operands: B [N, K] row-major weight,
+    Bs [ceil(N/128), ceil(K/128)], As2d [M, ceil(K/128)] any strides, ragged N and K allowed."""
+    M, K = A2d.shape
+    N = B.shape[0]
+    if M == 0:
+        return out2d
+    _launch_fp8_mm(A2d, B.data_ptr(), B.stride(0), As2d, Bs.data_ptr(), Bs.stride(0), Bs.stride(1), out2d, M, N, K)
+    return out2d
+
+
+# ---------------------------------------------------------------- INT8 GEMM
+
+def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[torch.Tensor] = None):
+    """sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747."""
+    _require(mat_a.is_cuda, "mat_a must be a CUDA tensor")
+    _require(mat_b.is_cuda, "mat_b must be a CUDA tensor")
+    _require(mat_a.dim() == 2, "mat_a must be a 2D tensor")
+    _require(mat_b.dim() == 2, "mat_b must be a 2D tensor")
+    _require(mat_a.stride(1) == 1, "mat_a must be a row major tensor")
+    _require(mat_b.stride(0) == 1, "mat_b must be a column major tensor")
+    _require(mat_a.size(1) == mat_b.size(0), "mat_a and mat_b shapes cannot be multiplied")
+    _require(mat_a.size(1) % 16 == 0, "mat_a.size(1) must be multiple of 16 for memory alignment")
+    _require(mat_b.size(0) % 16 == 0, "mat_b.size(0) must be multiple of 16 for memory alignment")
+    _require(mat_b.size(1) % 8 == 0, "mat_b.size(1) must be multiple of 8 for memory alignment")
+    _require(mat_a.dtype == torch.int8, "mat_a must be Int8")
+    _require(mat_b.dtype == torch.int8, "mat_b must be Int8")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be Half or BFloat16")
+    M, K = mat_a.shape
+    N = mat_b.size(1)
+    _require(scales_a.numel() == M, "size of scales_a is not matched")
+    _require(scales_b.numel() == N, "size of scales_b is not matched")
+    _require(scales_a.is_contiguous(), "scales_a must be contiguous")
+    _require(scales_b.is_contiguous(), "scales_b msut be contiguous")
+    _require(scales_a.dtype == torch.float32, "scales_a must be Float32")
+    _require(scales_b.dtype == torch.float32, "scales_b must be Float32")
+    if bias is not None:
+        _require(bias.numel() == N, "size of bias is not matched")
+        _require(bias.is_contiguous(), "bias must be contiguous")
+        _require(bias.dtype == out_dtype, "bias dtype must match output dtype")
+    out = torch.empty((M, N), dtype=out_dtype, device=mat_a.device)
+    if M == 0:
+        return out
+    _launch_int8_mm(mat_a, mat_b, scales_a, scales_b, bias, out)
+    return out
+
+
+def _launch_int8_mm(mat_a, mat_b, scales_a, scales_b, bias, out):
+    M, K = mat_a.shape
+    N = mat_b.size(1)
+    L = lib()
+    ws_bytes = L.mi355_int8_scaled_mm_workspace_bytes(M, N, K)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=mat_a.device) if ws_bytes else None
+    check(
+        L.mi355_int8_scaled_mm(
+            mat_a.data_ptr(), mat_b.data_ptr(),
+            scales_a.data_ptr() if scales_a is not None else None,
+            scales_b.data_ptr() if scales_b is not None else None,
+            bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out.dtype], M, N, K,
+            mat_a.stride(0), mat_b.stride(1), out.stride(0),
+            ws.data_ptr() if ws is not None else None, ws_bytes, _stream(),
+        )
+    )
+
+
+def int8_mm_raw_accumulators(mat_a: torch.Tensor, mat_b: torch.Tensor) -> torch.Tensor:
+    """int32 accumulators of ``int8_scaled_mm`` before its epilogue (same kernel, epilogue skipped)."""
+    out = torch.empty((mat_a.size(0), mat_b.size(1)), dtype=torch.int32, device=mat_a.device)
+    if mat_a.size(0):
+        _launch_int8_mm(mat_a, mat_b, None, None, None, out)
+    return out
+
+
+def per_token_quant_int8(x2d: torch.Tensor, q: torch.Tensor, s: torch.Tensor) -> None:
+    M, K = x2d.shape
+    if M:
+        check(lib().mi355_per_token_quant_int8(x2d.data_ptr(), _DT[x2d.dtype], q.data_ptr(), s.data_ptr(), M, K, _stream()))
+
+
+# ---------------------------------------------------------------- registration
+
+_registered = False
+_torch_lib = None
+
+
+def register() -> None:
+    """Define the ``sgl_kernel`` operators (unless an installed sgl_kernel already did) and attach
+    the gfx950 implementations to the CUDA (= HIP) dispatch key.  Idempotent."""
+    global _registered, _torch_lib
+    if _registered:
+        return
+    lib()  # fail now, loudly, if the native library is missing
+    _torch_lib = torch.library.Library("sgl_kernel", "FRAGMENT")
+    impls = {
+        "int8_scaled_mm": int8_scaled_mm,
+        "fp8_blockwise_scaled_mm": fp8_blockwise_scaled_mm,
+        "sgl_per_token_group_quant_8bit": sgl_per_token_group_quant_8bit,
+        "sgl_per_token_group_quant_8bit_v2": sgl_per_token_group_quant_8bit_v2,
+    }
+    for name, fn in impls.items():
+        if not hasattr(torch.ops.sgl_kernel, name):
+            _torch_lib.define(SCHEMAS[name])
+        _torch_lib.impl(name, fn, "CUDA")
+
+    def _fake_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+        return mat_a.new_empty((mat_a.size(0), mat_b.size(1)), dtype=out_dtype)
+
+    torch.library.register_fake("sgl_kernel::int8_scaled_mm", _fake_mm, lib=_torch_lib)
+    torch.library.register_fake("sgl_kernel::fp8_blockwise_scaled_mm", _fake_mm, lib=_torch_lib)
+    torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit", lambda *a: None, lib=_torch_lib)
+    torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit_v2", lambda *a: None, lib=_torch_lib)
+    _registered = True

@@ -1,0 +1,126 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads, exports every symbol the
+header declares, validates arguments before touching the device, and the Python operator
+layer carries the reference's names, schemas and error wording.  No kernel is launched."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mi355_qlinear.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from sglang_amd import _lib
+
+    L = _lib.lib()
+    declared = _declared_symbols()
+    assert len(declared) >= 8
+    for name in declared:
+        assert getattr(L, name) is not None, name
+    assert sorted(_lib.EXPORTS) == declared
+    assert L.mi355_qlinear_abi_version() == _lib.ABI_VERSION == 1
+
+
+def test_argument_validation_happens_before_any_device_work():
+    from sglang_amd import _lib
+
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    # K not divisible by group
+    rc = L.mi355_group_quant_8bit(p, _lib.BF16, p, _lib.FP8_E4M3FN, p, 4, 100, 128, 1e-10, -448.0, 448.0,
+                                  _lib.QUANT_DIV, _lib.SCALE_F32, 0.0, 1, 1, None)
+    assert rc == 1 and b"divisible by group" in L.mi355_last_error()
+    with pytest.raises(_lib.Mi355Error, match="divisible"):
+        _lib.check(rc)
+    # unsupported dtype / mode / group size
+    assert L.mi355_group_quant_8bit(p, _lib.I8, p, _lib.FP8_E4M3FN, p, 4, 128, 128, 1e-10, -448.0, 448.0, 0, 0, 0.0, 1, 1, None) == 1
+    assert L.mi355_group_quant_8bit(p, _lib.BF16, p, _lib.F16, p, 4, 128, 128, 1e-10, -448.0, 448.0, 0, 0, 0.0, 1, 1, None) == 1
+    assert L.mi355_group_quant_8bit(p, _lib.BF16, p, _lib.FP8_E4M3FN, p, 4, 128, 128, 1e-10, -448.0, 448.0, 7, 0, 0.0, 1, 1, None) == 1
+    rc = L.mi355_group_quant_8bit(p, _lib.BF16, p, _lib.FP8_E4M3FN, p, 4, 96, 24, 1e-10, -448.0, 448.0, 0, 0, 0.0, 1, 1, None)
+    assert rc == 2
+    with pytest.raises(NotImplementedError):
+        _lib.check(rc)
+    # empty problem is a successful no-op and clears the message
+    assert L.mi355_group_quant_8bit(None, _lib.BF16, None, _lib.FP8_E4M3FN, None, 0, 128, 128, 1e-10, -448.0, 448.0, 0, 0, 0.0, 1, 1, None) == 0
+    assert L.mi355_last_error() == b""
+
+
+def test_operator_schemas_are_the_reference_ones():
+    from sglang_amd import ops
+
+    ops.register()
+    ops.register()  # idempotent
+    for name in ("int8_scaled_mm", "fp8_blockwise_scaled_mm", "sgl_per_token_group_quant_8bit",
+                 "sgl_per_token_group_quant_8bit_v2"):
+        op = getattr(torch.ops.sgl_kernel, name).default
+        got = str(op._schema)
+        want = "sgl_kernel::" + ops.SCHEMAS[name]
+        assert got.replace(" ", "") == want.replace(" ", ""), (got, want)
+
+
+def test_python_surface_matches_reference_signatures():
+    from sglang_amd import fp8_kernel, sgl_kernel
+
+    sig = inspect.signature(sgl_kernel.sgl_per_token_group_quant_8bit)
+    assert list(sig.parameters) == ["input", "output_q", "output_s", "group_size", "eps", "fp8_min", "fp8_max",
+                                    "scale_ue8m0", "fuse_silu_and_mul", "masked_m", "enable_v2"]
+    assert sgl_kernel.sgl_per_token_group_quant_fp8 is sgl_kernel.sgl_per_token_group_quant_8bit
+    assert list(inspect.signature(sgl_kernel.fp8_blockwise_scaled_mm).parameters) == [
+        "mat_a", "mat_b", "scales_a", "scales_b", "out_dtype"]
+    assert list(inspect.signature(sgl_kernel.int8_scaled_mm).parameters) == [
+        "mat_a", "mat_b", "scales_a", "scales_b", "out_dtype", "bias"]
+    sig = inspect.signature(fp8_kernel.per_token_group_quant_fp8)
+    assert list(sig.parameters) == ["x", "group_size", "eps", "dtype", "column_major_scales", "scale_tma_aligned",
+                                    "scale_ue8m0"]
+    assert sig.parameters["eps"].default == 1e-10 and sig.parameters["dtype"].default == torch.float8_e4m3fn
+    sig = inspect.signature(fp8_kernel.w8a8_block_fp8_matmul)
+    assert list(sig.parameters) == ["A", "B", "As", "Bs", "block_size", "output_dtype"]
+    assert sig.parameters["output_dtype"].default == torch.float16
+    assert fp8_kernel.fp8_max == 448.0 and fp8_kernel.fp8_min == -448.0
+
+
+def test_scale_allocator_shapes_and_strides():
+    from sglang_amd.fp8_kernel import create_per_token_group_quant_fp8_output_scale as mk
+
+    s = mk((130, 1664), "cpu", 128, False, False, False)
+    assert s.shape == (130, 13) and s.is_contiguous() and s.dtype == torch.float32
+    s = mk((130, 1664), "cpu", 128, True, False, False)
+    assert s.shape == (130, 13) and s.stride() == (1, 130)
+    s = mk((130, 1664), "cpu", 128, True, True, False)
+    assert s.shape == (130, 13) and s.stride() == (1, 132)
+    s = mk((130, 1664), "cpu", 128, True, True, True)
+    assert s.shape == (130, 4) and s.stride() == (1, 132) and s.dtype == torch.int32
+    s = mk((3, 7, 256), "cpu", 64, False, False, False)
+    assert s.shape == (3, 7, 4)
+
+
+def test_host_checks_reject_bad_operands_with_reference_wording():
+    from sglang_amd import ops, sgl_kernel
+
+    a = torch.zeros(4, 256, dtype=torch.float8_e4m3fn)
+    # through the dispatcher a CPU tensor finds no kernel, exactly as with the reference's CUDA-only registration
+    with pytest.raises(NotImplementedError, match="CPU"):
+        sgl_kernel.fp8_blockwise_scaled_mm(a, a.t(), torch.zeros(4, 2), torch.zeros(2, 2), torch.bfloat16)
+    # the registered host functions themselves speak the reference's TORCH_CHECK wording
+    with pytest.raises(RuntimeError, match="mat_a must be a CUDA tensor"):
+        ops.fp8_blockwise_scaled_mm(a, a.t(), torch.zeros(4, 2), torch.zeros(2, 2), torch.bfloat16)
+    with pytest.raises(RuntimeError, match="mat_a must be a CUDA tensor"):
+        ops.int8_scaled_mm(a.view(torch.int8), a.view(torch.int8).t(), torch.zeros(4), torch.zeros(4), torch.bfloat16)
+    with pytest.raises(RuntimeError, match="input must be a CUDA tensor"):
+        ops.sgl_per_token_group_quant_8bit(torch.zeros(4, 256), a, torch.zeros(4, 2), 128, 1e-10, -448.0, 448.0, False)
+    with pytest.raises(AssertionError, match="only v2 support"):
+        sgl_kernel.sgl_per_token_group_quant_8bit(torch.zeros(4, 256), a, torch.zeros(4, 2), 128, 1e-10, -448.0, 448.0,
+                                                  fuse_silu_and_mul=True, enable_v2=False)
+    with pytest.raises(NotImplementedError):
+        ops.sgl_per_token_group_quant_8bit_v2(torch.zeros(4, 256), a, torch.zeros(4, 2), 128, 1e-10, -448.0, 448.0,
+                                              False, True, None)
