@@ -1,0 +1,536 @@
+// Blockwise-scaled FP8 GEMM and per-token/per-channel INT8 GEMM for gfx950 (MI355X).
+//
+// One LDS-staged MFMA skeleton serves both:
+//   * 256 threads = 4 waves per workgroup, macro tile BM (tokens) x BN (output channels) x 128 (K bytes);
+//   * both operands are K-contiguous bytes; a K step of 128 bytes per row is staged through LDS in a
+//     double buffer: global_load_dwordx4 -> registers -> ds_write_b128, the loads for step k+1 are in
+//     flight while step k is multiplied;
+//   * LDS rows are 128 bytes, the eight 16-byte chunks of a row are XOR-swizzled with (row & 7) so both
+//     the cooperative writes and the MFMA operand reads (16 rows x one chunk per ds_read_b128) are free
+//     of bank conflicts;
+//   * the weight tile is the MFMA "A" operand and the token tile the "B" operand, so a lane's four
+//     accumulator registers are four consecutive output channels of ONE token: the per-token scale is a
+//     single value per lane and M-tile, and the output store is 4 contiguous elements;
+//   * FP8: v_mfma_f32_16x16x128_f8f6f4 consumes exactly one 128-wide scale block, its result is promoted
+//     into the fp32 accumulator with one FMA per element: acc += part * (sa[m,kb] * sb[nb,kb])
+//     (python/sglang/srt/layers/quantization/fp8_kernel.py:749-758);
+//   * INT8: two v_mfma_i32_16x16x64_i8 per K step accumulate exactly in int32; the epilogue is
+//     f32(acc) * (sb[n] * sa[m]) + bias (epilogue_per_row_per_col_scale.h:280-303);
+//   * small token counts stream the weight once with a split along K: partial tiles go to a caller
+//     workspace and a second kernel adds them in a fixed order (deterministic, no atomics);
+//   * workgroups are renumbered so that each of the 8 XCDs (own L2) works on a contiguous, M-grouped
+//     patch of output tiles.
+#include <type_traits>
+
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int KSTEP = 128;   // bytes of K per row and stage
+constexpr int THREADS = 256;
+
+struct GemmParams {
+  const uint8_t* a;  // tokens   [M, K], row stride lda
+  const uint8_t* b;  // channels [N, K], row stride ldb
+  const float* sa;
+  const float* sb;
+  const void* bias;
+  void* out;
+  void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
+  int M, N, K;
+  int64_t lda, ldb, ldo;
+  int64_t sa_sm, sa_sk, sb_sn, sb_sk;
+  int kb_total, kb_per_split, splits;
+  int tiles_m, tiles_n;
+  int out_dtype;
+};
+
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off, const float* r, int nvalid,
+                                           bool vec_ok) {
+  if (out_dtype == MI355_F32) {
+    float* o = reinterpret_cast<float*>(out) + off;
+    if (nvalid == 4 && vec_ok) {
+      *reinterpret_cast<v4f*>(o) = v4f{r[0], r[1], r[2], r[3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i < nvalid) o[i] = r[i];
+    }
+    return;
+  }
+  uint32_t h[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) h[i] = (out_dtype == MI355_BF16) ? f32_to_bf16_bits(r[i]) : f32_to_f16_bits(r[i]);
+  uint16_t* o = reinterpret_cast<uint16_t*>(out) + off;
+  if (nvalid == 4 && vec_ok) {
+    *reinterpret_cast<u32x2*>(o) = u32x2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < nvalid) o[i] = (uint16_t)h[i];
+  }
+}
+
+// IS_FP8: blockwise-scaled fp8 (fp32 accumulators) or int8 (int32 accumulators).
+// BM x BN macro tile, WGM x WGN waves (WGM * WGN == 4).
+// ALIGNED: rows of both operands start on 16-byte boundaries and K % 16 == 0, so 16-byte loads are legal.
+// SPLIT: write raw partial accumulators to the workspace instead of the epilogue.
+template <bool IS_FP8, int BM, int BN, int WGM, int WGN, bool ALIGNED, bool SPLIT>
+__global__ __launch_bounds__(THREADS) void gemm_kernel(const GemmParams p) {
+  static_assert(WGM * WGN == 4, "four waves per workgroup");
+  constexpr int WM = BM / WGM, WN = BN / WGN;
+  constexpr int MT = WM / 16, NT = WN / 16;
+  static_assert(MT >= 1 && NT >= 1 && 128 % WN == 0, "a wave's channels must lie inside one 128-wide scale block");
+  constexpr int ROWS = BM + BN;
+  constexpr int LOADS = (ROWS + 31) / 32;  // 16-byte chunks per thread and stage
+  constexpr bool LAST_PARTIAL = (ROWS % 32) != 0;  // the last pass covers fewer than 32 rows
+  constexpr int STAGE_BYTES = ROWS * KSTEP;
+  using AccT = typename std::conditional<IS_FP8, float, int>::type;
+
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  uint8_t* tiles = smem;                                                 // [2][ROWS][128]
+  float* s_scale = reinterpret_cast<float*>(smem + 2 * STAGE_BYTES);     // [2][BM] (fp8 only)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave / WGN, wave_n = wave % WGN;
+  const int l16 = lane & 15, q = lane >> 4;
+
+  // ---- which tile: XCD-contiguous, M-grouped order
+  int bid = blockIdx.x;
+  {
+    const int total = gridDim.x;
+    const int per = total >> 3;
+    if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
+  }
+  const int tiles_mn = p.tiles_m * p.tiles_n;
+  const int split = bid / tiles_mn;
+  const int lid = bid - split * tiles_mn;
+  constexpr int GROUP_M = 8;
+  const int per_group = GROUP_M * p.tiles_n;
+  const int group = lid / per_group;
+  const int first_m = group * GROUP_M;
+  const int gm = min(p.tiles_m - first_m, GROUP_M);
+  const int in_group = lid - group * per_group;
+  const int tile_m = first_m + in_group % gm;
+  const int tile_n = in_group / gm;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int kb_begin = split * p.kb_per_split;
+  const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
+
+  // ---- loader set-up: thread owns chunk (tid & 7) of rows (tid >> 3) + 32 * i
+  const int chunk = tid & 7;
+  const uint8_t* gptr[LOADS];
+  uint32_t lds_off[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int row = min((tid >> 3) + 32 * i, ROWS - 1);  // rows < BM are tokens, the rest channels
+    if (row < BM) {
+      const int m = min(m0 + row, p.M - 1);  // rows past the edge re-read the last valid row; never stored
+      gptr[i] = p.a + (int64_t)m * p.lda + chunk * 16;
+    } else {
+      const int n = min(n0 + row - BM, p.N - 1);
+      gptr[i] = p.b + (int64_t)n * p.ldb + chunk * 16;
+    }
+    lds_off[i] = row * KSTEP + ((chunk ^ (row & 7)) << 4);
+  }
+  const float* sa_ptr = nullptr;
+  if constexpr (IS_FP8) {
+    if (tid < BM) sa_ptr = p.sa + (int64_t)min(m0 + tid, p.M - 1) * p.sa_sm;
+  }
+
+  u32x4 stage_regs[LOADS];
+  float stage_scale = 0.f;
+
+  auto load_global = [&](int kb) {
+    const int kbyte = kb * KSTEP + chunk * 16;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const uint8_t* src = gptr[i] + (int64_t)kb * KSTEP;
+      if constexpr (ALIGNED) {
+        stage_regs[i] = (kbyte < p.K) ? *reinterpret_cast<const u32x4*>(src) : u32x4{0, 0, 0, 0};
+      } else {
+        // arbitrary K and row strides: byte loads with a bound on every byte
+        uint32_t w[4] = {0, 0, 0, 0};
+        for (int j = 0; j < 16; ++j)
+          if (kbyte + j < p.K) w[j >> 2] |= (uint32_t)src[j] << (8 * (j & 3));
+        stage_regs[i] = u32x4{w[0], w[1], w[2], w[3]};
+      }
+    }
+    if constexpr (IS_FP8) {
+      if (tid < BM) stage_scale = sa_ptr[(int64_t)kb * p.sa_sk];
+    }
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      if (LAST_PARTIAL && i == LOADS - 1 && (tid >> 3) + 32 * i >= ROWS) continue;
+      *reinterpret_cast<u32x4*>(tiles + buf * STAGE_BYTES + lds_off[i]) = stage_regs[i];
+    }
+    if constexpr (IS_FP8) {
+      if (tid < BM) s_scale[buf * BM + tid] = stage_scale;
+    }
+  };
+
+  AccT acc[NT][MT][4];
+#pragma unroll
+  for (int i = 0; i < NT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0;
+
+  // operand fragment addresses inside a stage (swizzled); constant over K
+  uint32_t tok_off[MT][2], ch_off[NT][2];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int row = wave_m * WM + j * 16 + l16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) tok_off[j][h] = row * KSTEP + (((2 * q + h) ^ (row & 7)) << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    const int row = BM + wave_n * WN + i * 16 + l16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) ch_off[i][h] = row * KSTEP + (((2 * q + h) ^ (row & 7)) << 4);
+  }
+  // one 128x128 weight block holds all of this wave's channels
+  const int nb = min(n0 + wave_n * WN, p.N - 1) / 128;
+
+  if (kb_begin < kb_end) {
+    load_global(kb_begin);
+    store_lds(0);
+  }
+  __syncthreads();
+
+  for (int kb = kb_begin; kb < kb_end; ++kb) {
+    const int buf = (kb - kb_begin) & 1;
+    const bool more = kb + 1 < kb_end;
+    if (more) load_global(kb + 1);
+
+    const uint8_t* st = tiles + buf * STAGE_BYTES;
+    u32x4 tok[MT][2];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      tok[j][0] = *reinterpret_cast<const u32x4*>(st + tok_off[j][0]);
+      tok[j][1] = *reinterpret_cast<const u32x4*>(st + tok_off[j][1]);
+    }
+    if constexpr (IS_FP8) {
+      const float sbv = p.sb[(int64_t)nb * p.sb_sn + (int64_t)kb * p.sb_sk];
+      float sc[MT];
+#pragma unroll
+      for (int j = 0; j < MT; ++j) sc[j] = s_scale[buf * BM + wave_m * WM + j * 16 + l16] * sbv;
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const u32x4 c0 = *reinterpret_cast<const u32x4*>(st + ch_off[i][0]);
+        const u32x4 c1 = *reinterpret_cast<const u32x4*>(st + ch_off[i][1]);
+        const v8i wfrag = {(int)c0.x, (int)c0.y, (int)c0.z, (int)c0.w, (int)c1.x, (int)c1.y, (int)c1.z, (int)c1.w};
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          const v8i tfrag = {(int)tok[j][0].x, (int)tok[j][0].y, (int)tok[j][0].z, (int)tok[j][0].w,
+                             (int)tok[j][1].x, (int)tok[j][1].y, (int)tok[j][1].z, (int)tok[j][1].w};
+          const v4f part =
+              __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wfrag, tfrag, v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[i][j][v] = fmaf(part[v], sc[j], acc[i][j][v]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const u32x4 c0 = *reinterpret_cast<const u32x4*>(st + ch_off[i][0]);
+        const u32x4 c1 = *reinterpret_cast<const u32x4*>(st + ch_off[i][1]);
+        const v4i w0 = {(int)c0.x, (int)c0.y, (int)c0.z, (int)c0.w};
+        const v4i w1 = {(int)c1.x, (int)c1.y, (int)c1.z, (int)c1.w};
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          v4i c = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+          const v4i t0 = {(int)tok[j][0].x, (int)tok[j][0].y, (int)tok[j][0].z, (int)tok[j][0].w};
+          const v4i t1 = {(int)tok[j][1].x, (int)tok[j][1].y, (int)tok[j][1].z, (int)tok[j][1].w};
+          c = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, t0, c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, t1, c, 0, 0, 0);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[i][j][v] = c[v];
+        }
+      }
+    }
+
+    if (more) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds channels n = nbase + 4q .. +3 of token m = mbase + l16
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = m0 + wave_m * WM + j * 16 + l16;
+    if (m >= p.M) continue;
+    float sa_m = 1.f;
+    if constexpr (!IS_FP8 && !SPLIT) {
+      if (p.out_dtype != MI355_I32) sa_m = p.sa[m];
+    }
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      const int n = n0 + wave_n * WN + i * 16 + 4 * q;
+      if (n >= p.N) continue;
+      const int nvalid = min(4, p.N - n);
+      if constexpr (SPLIT) {
+        AccT* w = reinterpret_cast<AccT*>(p.ws) + ((int64_t)split * p.M + m) * p.N + n;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (v < nvalid) w[v] = acc[i][j][v];
+      } else if constexpr (IS_FP8) {
+        store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
+      } else {
+        if (p.out_dtype == MI355_I32) {
+          int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (v < nvalid) o[v] = acc[i][j][v];
+        } else {
+          float r[4];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int nn = min(n + v, p.N - 1);
+            // separately rounded multiply and add: the contract is mul, mul, add, not a fused multiply-add
+            float t = __fmul_rn((float)acc[i][j][v], __fmul_rn(p.sb[nn], sa_m));
+            if (p.bias) {
+              const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[nn];
+              t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+            }
+            r[v] = t;
+          }
+          store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, nvalid, vec_ok);
+        }
+      }
+    }
+  }
+}
+
+// Sums the split-K partial tiles in ascending split order and applies the epilogue.
+template <bool IS_FP8>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) {
+  const int64_t total = (int64_t)p.M * p.N;
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= total) return;
+  // N % 4 == 0 is required for the split path, so the four elements share a row
+  const int m = (int)(idx / p.N);
+  const int n = (int)(idx - (int64_t)m * p.N);
+  if constexpr (IS_FP8) {
+    const float* w = reinterpret_cast<const float*>(p.ws) + idx;
+    v4f s = *reinterpret_cast<const v4f*>(w);
+    for (int k = 1; k < p.splits; ++k) {
+      const v4f t = *reinterpret_cast<const v4f*>(w + (int64_t)k * total);
+      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
+    }
+    const float r[4] = {s[0], s[1], s[2], s[3]};
+    const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+    store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
+  } else {
+    const int* w = reinterpret_cast<const int*>(p.ws) + idx;
+    v4i s = *reinterpret_cast<const v4i*>(w);
+    for (int k = 1; k < p.splits; ++k) {
+      const v4i t = *reinterpret_cast<const v4i*>(w + (int64_t)k * total);
+      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
+    }
+    if (p.out_dtype == MI355_I32) {
+      int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
+      for (int v = 0; v < 4; ++v) o[v] = s[v];
+      return;
+    }
+    const float sa_m = p.sa[m];
+    float r[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float t = __fmul_rn((float)s[v], __fmul_rn(p.sb[n + v], sa_m));
+      if (p.bias) {
+        const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
+        t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+      }
+      r[v] = t;
+    }
+    const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+    store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+struct Plan {
+  int bm, bn, splits, kb_per_split;
+};
+
+constexpr int NUM_CUS = 256;
+
+// Tile and split selection.  Large token counts are MFMA-bound and want the biggest tile; small ones
+// stream the weight once and want enough workgroups in flight to cover HBM latency.
+Plan make_plan(int64_t M, int64_t N, int64_t K) {
+  Plan pl;
+  pl.bn = 128;
+  if (M <= 16) pl.bm = 16;
+  else if (M <= 32) pl.bm = 32;
+  else if (M <= 64) pl.bm = 64;
+  else if (M <= 1024) pl.bm = 128;
+  else pl.bm = 256;
+  const int64_t kb_total = (K + KSTEP - 1) / KSTEP;
+  const int64_t tiles = ((M + pl.bm - 1) / pl.bm) * ((N + pl.bn - 1) / pl.bn);
+  int splits = 1;
+  if (N % 4 == 0 && tiles < 2 * NUM_CUS) {
+    // aim at ~4 workgroups per CU, keep at least 4 K steps per split
+    int64_t want = (4 * NUM_CUS + tiles - 1) / tiles;
+    int64_t max_by_k = kb_total / 4 > 0 ? kb_total / 4 : 1;
+    splits = (int)(want < max_by_k ? want : max_by_k);
+    if (splits < 1) splits = 1;
+    if (splits > 32) splits = 32;
+  }
+  pl.kb_per_split = (int)((kb_total + splits - 1) / splits);
+  pl.splits = (int)((kb_total + pl.kb_per_split - 1) / pl.kb_per_split);
+  if (pl.splits < 1) pl.splits = 1;
+  return pl;
+}
+
+size_t workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const Plan pl = make_plan(M, N, K);
+  return pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
+}
+
+template <bool IS_FP8, int BM, int BN, int WGM, int WGN>
+int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* what) {
+  p.tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + BN - 1) / BN;
+  const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * p.splits);
+  const size_t lds = 2 * (size_t)(BM + BN) * KSTEP + (IS_FP8 ? 2 * BM * sizeof(float) : 0);
+  const bool split = p.splits > 1;
+#define MI355_LAUNCH(AL, SP)                                                                                   \
+  do {                                                                                                         \
+    auto kfn = gemm_kernel<IS_FP8, BM, BN, WGM, WGN, AL, SP>;                                                  \
+    static bool lds_reserved = false;                                                                          \
+    if (lds > 64 * 1024 && !lds_reserved) {                                                                    \
+      lds_reserved = true;                                                                                     \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                                   \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                \
+      if (e != hipSuccess) {                                                                                   \
+        set_error("%s: cannot reserve %zu bytes of LDS: %s", what, lds, hipGetErrorString(e));                 \
+        return MI355_ERR_LAUNCH;                                                                               \
+      }                                                                                                        \
+    }                                                                                                          \
+    hipLaunchKernelGGL(kfn, dim3(grid), dim3(THREADS), lds, stream, p);                                        \
+  } while (0)
+  if (aligned) {
+    if (split) MI355_LAUNCH(true, true); else MI355_LAUNCH(true, false);
+  } else {
+    if (split) MI355_LAUNCH(false, true); else MI355_LAUNCH(false, false);
+  }
+#undef MI355_LAUNCH
+  int rc = check_launch(what);
+  if (rc != MI355_OK) return rc;
+  if (split) {
+    const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
+    hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
+    rc = check_launch(what);
+  }
+  return rc;
+}
+
+template <bool IS_FP8>
+int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipStream_t stream, const char* what) {
+  const Plan pl = make_plan(p.M, p.N, p.K);
+  p.kb_total = (p.K + KSTEP - 1) / KSTEP;
+  p.splits = pl.splits;
+  p.kb_per_split = pl.kb_per_split;
+  if (pl.splits > 1) {
+    const size_t need = (size_t)pl.splits * (size_t)p.M * (size_t)p.N * 4u;
+    MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
+                  "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
+    MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
+                  "%s: workspace must be 16-byte aligned", what);
+    p.ws = workspace;
+  }
+  const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
+                       ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
+  switch (pl.bm) {
+    case 16: return launch_tile<IS_FP8, 16, 128, 1, 4>(p, aligned, stream, what);
+    case 32: return launch_tile<IS_FP8, 32, 128, 1, 4>(p, aligned, stream, what);
+    case 64: return launch_tile<IS_FP8, 64, 128, 1, 4>(p, aligned, stream, what);
+    case 128: return launch_tile<IS_FP8, 128, 128, 2, 2>(p, aligned, stream, what);
+    default: return launch_tile<IS_FP8, 256, 128, 2, 2>(p, aligned, stream, what);
+  }
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" size_t mi355_fp8_blockwise_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return workspace_bytes(M, N, K);
+}
+
+extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                      int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                      int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo,
+                                      void* workspace, size_t workspace_bytes_given, void* stream) {
+  const char* what = "mi355_fp8_blockwise_mm";
+  clear_error();
+  MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
+  MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16 || out_dtype == MI355_F32,
+                MI355_ERR_INVALID_ARGUMENT, "%s: out_dtype must be bfloat16, float16 or float32", what);
+  if (M == 0 || N == 0) return MI355_OK;
+  MI355_REQUIRE(K > 0, MI355_ERR_INVALID_ARGUMENT, "%s: K must be positive", what);
+  MI355_REQUIRE(a && b && sa && sb && out, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  MI355_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MI355_ERR_INVALID_ARGUMENT,
+                "%s: dimensions must fit in 31 bits", what);
+  MI355_REQUIRE(lda >= K && ldb >= K && ldo >= N, MI355_ERR_INVALID_ARGUMENT,
+                "%s: row strides smaller than the row length", what);
+  GemmParams p{};
+  p.a = static_cast<const uint8_t*>(a);
+  p.b = static_cast<const uint8_t*>(b);
+  p.sa = sa, p.sb = sb, p.bias = nullptr, p.out = out, p.ws = nullptr;
+  p.M = (int)M, p.N = (int)N, p.K = (int)K;
+  p.lda = lda, p.ldb = ldb, p.ldo = ldo;
+  p.sa_sm = sa_sm, p.sa_sk = sa_sk, p.sb_sn = sb_sn, p.sb_sk = sb_sk;
+  p.out_dtype = out_dtype;
+  return run_gemm<true>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
+}
+
+extern "C" size_t mi355_int8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return workspace_bytes(M, N, K);
+}
+
+extern "C" int mi355_int8_scaled_mm(const void* a, const void* b, const float* sa, const float* sb, const void* bias,
+                                    void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                    int64_t ldb, int64_t ldo, void* workspace, size_t workspace_bytes_given,
+                                    void* stream) {
+  const char* what = "mi355_int8_scaled_mm";
+  clear_error();
+  MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
+  MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16 || out_dtype == MI355_I32,
+                MI355_ERR_INVALID_ARGUMENT, "%s: out_dtype must be bfloat16 or float16 (int32 for raw accumulators)",
+                what);
+  if (M == 0 || N == 0) return MI355_OK;
+  MI355_REQUIRE(K > 0, MI355_ERR_INVALID_ARGUMENT, "%s: K must be positive", what);
+  MI355_REQUIRE(a && b && out, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  MI355_REQUIRE(out_dtype == MI355_I32 || (sa && sb), MI355_ERR_INVALID_ARGUMENT, "%s: scales missing", what);
+  MI355_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 17), MI355_ERR_INVALID_ARGUMENT,
+                "%s: K must stay below 131072 so that int32 accumulation cannot overflow", what);
+  MI355_REQUIRE(lda >= K && ldb >= K && ldo >= N, MI355_ERR_INVALID_ARGUMENT,
+                "%s: row strides smaller than the row length", what);
+  GemmParams p{};
+  p.a = static_cast<const uint8_t*>(a);
+  p.b = static_cast<const uint8_t*>(b);
+  p.sa = sa, p.sb = sb, p.bias = bias, p.out = out, p.ws = nullptr;
+  p.M = (int)M, p.N = (int)N, p.K = (int)K;
+  p.lda = lda, p.ldb = ldb, p.ldo = ldo;
+  p.out_dtype = out_dtype;
+  return run_gemm<false>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
+}

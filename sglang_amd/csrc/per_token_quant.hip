@@ -1,0 +1,138 @@
+// Per-token (per-row) symmetric INT8 quantizer for gfx950.
+//
+// One workgroup per row: 16-byte loads, |x| max over the row (DPP inside a wave, LDS across the four
+// waves), then q = round-half-away(x * (127 / absmax)) with absmax floored at 1e-10 and
+// scale = absmax / 127, as in python/sglang/srt/layers/quantization/int8_kernel.py:47-50.
+// Rows of up to 8192 two-byte elements stay in registers between the two phases; longer rows are
+// re-read (from L2).
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int DT>
+__device__ __forceinline__ void unpack16(const u32x4& r, float* f) {
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+  if constexpr (DT == MI355_F32) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(w[i]);
+  } else if constexpr (DT == MI355_BF16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = f16_bits_to_f32(w[i] & 0xffffu);
+      f[2 * i + 1] = f16_bits_to_f32(w[i] >> 16);
+    }
+  }
+}
+
+__device__ __forceinline__ float wave_allreduce_max(float v) {
+  // row_shr-free butterfly inside 16-lane rows, then across rows with ds_swizzle-free readlane
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
+  float r = fmaxf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)),
+                  __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16)));
+  r = fmaxf(r, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)));
+  r = fmaxf(r, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48)));
+  return r;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void per_token_quant_int8_kernel(const void* x, int8_t* q, float* s, int64_t K) {
+  constexpr int VEC = (DT == MI355_F32) ? 4 : 8;
+  constexpr int KEEP = 4;  // vectors per thread kept in registers
+  __shared__ float wave_max[4];
+  const int64_t row = blockIdx.x;
+  const int64_t nvec = K / VEC;
+  const u32x4* src = reinterpret_cast<const u32x4*>(x) + row * nvec;
+  u32x4 keep[KEEP];
+  float amax = 1e-10f;
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int64_t v = threadIdx.x + 256 * i;
+    keep[i] = (v < nvec) ? src[v] : u32x4{0, 0, 0, 0};
+    float f[VEC];
+    unpack16<DT>(keep[i], f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) amax = fmaxf(amax, fabsf(f[j]));
+  }
+  for (int64_t v = threadIdx.x + 256 * KEEP; v < nvec; v += 256) {
+    float f[VEC];
+    unpack16<DT>(src[v], f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) amax = fmaxf(amax, fabsf(f[j]));
+  }
+  amax = wave_allreduce_max(amax);
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+  if (threadIdx.x == 0) s[row] = amax / 127.0f;
+  const float mul = 127.0f / amax;
+
+  auto emit = [&](const u32x4& raw, int64_t v) {
+    float f[VEC];
+    unpack16<DT>(raw, f);
+    uint32_t w[VEC / 4];
+#pragma unroll
+    for (int j = 0; j < VEC / 4; ++j) {
+      uint32_t pk = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) pk |= ((uint32_t)(int)roundf(f[4 * j + b] * mul) & 0xffu) << (8 * b);
+      w[j] = pk;
+    }
+    int8_t* d = q + row * K + v * VEC;
+    if constexpr (VEC == 8)
+      *reinterpret_cast<u32x2*>(d) = u32x2{w[0], w[1]};
+    else
+      *reinterpret_cast<uint32_t*>(d) = w[0];
+  };
+#pragma unroll
+  for (int i = 0; i < KEEP; ++i) {
+    const int64_t v = threadIdx.x + 256 * i;
+    if (v < nvec) emit(keep[i], v);
+  }
+  for (int64_t v = threadIdx.x + 256 * KEEP; v < nvec; v += 256) emit(src[v], v);
+}
+
+}  // namespace
+}  // namespace mi355
+
+extern "C" int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K,
+                                          void* stream) {
+  using namespace mi355;
+  const char* what = "mi355_per_token_quant_int8";
+  clear_error();
+  MI355_REQUIRE(M >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
+  MI355_REQUIRE(x_dtype == MI355_F32 || x_dtype == MI355_F16 || x_dtype == MI355_BF16, MI355_ERR_INVALID_ARGUMENT,
+                "%s: input must be float32, float16 or bfloat16", what);
+  if (M == 0 || K == 0) return MI355_OK;
+  MI355_REQUIRE(x && q && s, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  MI355_REQUIRE((K * (int64_t)dtype_size(x_dtype)) % 16 == 0, MI355_ERR_UNSUPPORTED,
+                "%s: a row must span a multiple of 16 input bytes", what);
+  MI355_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)q % 8 == 0), MI355_ERR_INVALID_ARGUMENT,
+                "%s: input must be 16-byte and output 8-byte aligned", what);
+  MI355_REQUIRE(M < (1ll << 31), MI355_ERR_INVALID_ARGUMENT, "%s: too many rows", what);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int8_t* qq = static_cast<int8_t*>(q);
+  switch (x_dtype) {
+    case MI355_F32:
+      hipLaunchKernelGGL(per_token_quant_int8_kernel<MI355_F32>, dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      break;
+    case MI355_F16:
+      hipLaunchKernelGGL(per_token_quant_int8_kernel<MI355_F16>, dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      break;
+    default:
+      hipLaunchKernelGGL(per_token_quant_int8_kernel<MI355_BF16>, dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+  }
+  return check_launch(what);
+}
