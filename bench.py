@@ -1,22 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--quick]
 
-Prints ONE JSON line.  A "step" is one pass of the hot path over one batch of synthetic,
-seeded input that is already resident in HBM.  Inputs rotate over several buffers whose
-total size exceeds the 256 MB Infinity Cache, so every step streams from HBM.
+Prints ONE JSON line.  A "step" is one pass of the hot path over one batch of seeded synthetic
+input that is already resident in HBM; operands rotate over several buffers so that
+bandwidth-bound steps stream from HBM rather than from the 256 MB Infinity Cache.
 
-Workloads (``--workload``):
-  fp8_gemm   blockwise-FP8 GEMM, M=4096, DeepSeek-V3 gate_up (K=7168 -> N=36864)   [default, headline]
-  quant      per-token-group FP8 quantization, M=16384 K=7168 g=128, fp32 row-major scales
-  quant_ue8m0  same, column-major packed UE8M0 scales
-The default run reports the headline GEMM as ``value`` and carries the quantizer (both
-variants) and the other shapes of the named configurations under ``"also"``.
+--workload:
+  fp8_gemm   (headline, default) blockwise-FP8 GEMM, M=4096, DeepSeek-V3 gate_up K=7168 -> N=36864
+  quant      per-token-group FP8 quantization, M=16384 K=7168 g=128, row-major fp32 scales
+  quant_ue8m0  the same with column-major packed UE8M0 scales
+  all        (what the default run does) headline as `value`, every other configuration the
+             baseline names under "also": both quantizer variants, the M=4096 MLP/MLA shapes,
+             the decode shapes M in {1,8,32,128}, the single linear, and the INT8 GEMM shapes.
 
-``roofline.achieved`` is algorithmic bytes (or FLOPs) per launch divided by the average
-launch duration measured with HIP events on the launch stream; ``cpu_baseline`` times the CPU
-oracle on a bounded sample of the same workload on this host.
+`roofline.achieved` = algorithmic FLOPs (2*M*N*K) or bytes per launch / average launch duration
+measured with HIP events on the launch stream.  `cpu_baseline` times the CPU oracle on a bounded
+sample of the same workload on this host's cores.
 """
 from __future__ import annotations
 
@@ -31,16 +32,16 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
-FP8_PEAK_TFLOPS = 5000.0    # dense fp8 MFMA (no sparsity)
-INT8_PEAK_TOPS = 5000.0
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E
+FP8_PEAK_TFLOPS = 5000.0  # dense fp8 MFMA, no sparsity
+INT8_PEAK_TOPS = 5000.0   # dense int8 MFMA
 
 METRIC = "blockwise-FP8 GEMM TFLOPS & %MFMA peak; quant GB/s & %HBM peak (1 GPU)"
 
 
 def _time_launches(fn, nbuf, steps, warmup):
-    """Run fn(i % nbuf) warmup + steps times on the current stream; returns (wall seconds for the
-    timed steps, list of per-launch milliseconds from HIP events)."""
+    """fn(i % nbuf) is launched warmup + steps times on the current stream.  Returns the wall seconds of
+    the timed steps (synchronize on both sides) and the per-launch milliseconds from HIP events."""
     import torch
 
     for i in range(warmup):
@@ -57,10 +58,28 @@ def _time_launches(fn, nbuf, steps, warmup):
     return wall, [a.elapsed_time(b) for a, b in evs]
 
 
+def _stats(ms):
+    s = sorted(ms)
+    return {"avg": sum(ms) / len(ms), "median": statistics.median(ms), "p20_p80": [s[len(s) // 5], s[len(s) * 4 // 5]]}
+
+
+def _cpu_time_boxed(fn, seconds=10.0):
+    fn()  # page in, spin up the OpenMP team
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < seconds:
+        fn()
+        reps += 1
+    return (time.perf_counter() - t0) / reps, reps
+
+
+# ------------------------------------------------------------------------------------------ quantizer
+
 def bench_quant(steps, warmup, ue8m0, with_cpu):
     import torch
 
     from sglang_amd import fp8_kernel
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_fp8
     from sglang_amd.workloads import make_activation, quant_algorithmic_bytes
 
     dev = torch.device("cuda:0")
@@ -68,53 +87,164 @@ def bench_quant(steps, warmup, ue8m0, with_cpu):
     nbuf = 4
     base = make_activation(M, K, zero_group_frac=1e-4, zero_elem_frac=1e-4)
     xs = [base.to(dev)]
-    for i in range(1, nbuf):  # distinct buffers; rolling the rows keeps the distribution and costs no host time
+    for i in range(1, nbuf):  # distinct buffers; rolling the rows keeps the distribution
         xs.append(torch.roll(xs[0], shifts=i * 97, dims=0).contiguous())
     qs = [torch.empty(M, K, dtype=torch.float8_e4m3fn, device=dev) for _ in range(nbuf)]
     ss = [fp8_kernel.create_per_token_group_quant_fp8_output_scale((M, K), dev, G, ue8m0, ue8m0, ue8m0)
           for _ in range(nbuf)]
-    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_fp8
 
     def step(i):
         sgl_per_token_group_quant_fp8(xs[i], qs[i], ss[i], G, 1e-10, -448.0, 448.0, ue8m0, enable_v2=ue8m0)
 
     wall, ms = _time_launches(step, nbuf, steps, warmup)
     alg = quant_algorithmic_bytes(M, K, G, 2, ue8m0)
-    avg_ms = sum(ms) / len(ms)
+    st = _stats(ms)
     rec = {
-        "workload": ("quant_ue8m0" if ue8m0 else "quant") + f" M={M} K={K} g={G} bf16->e4m3fn "
-        + ("col-major packed UE8M0 scales (v2 arithmetic)" if ue8m0 else "row-major fp32 scales (v1 arithmetic)"),
-        "value": alg / (wall / steps) / 1e9,
-        "unit": "GB/s",
-        "ms_per_step": wall / steps * 1e3,
-        "kernel_ms_avg": avg_ms,
-        "kernel_ms_median": statistics.median(ms),
-        "kernel_ms_p20_p80": [sorted(ms)[len(ms) // 5], sorted(ms)[len(ms) * 4 // 5]],
-        "dtype": "bf16->fp8(e4m3fn), fp32 arithmetic",
-        "roofline": {
-            "bound": "hbm", "achieved": alg / (avg_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": alg / (avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": alg,
-        },
+        "workload": ("quant_ue8m0" if ue8m0 else "quant") + f" M={M} K={K} g={G} bf16->e4m3fn, "
+        + ("column-major packed UE8M0 scales (q = x * 448/amax)" if ue8m0 else "row-major fp32 scales (q = x / s)"),
+        "value": alg / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "f32 arithmetic on bf16 input, e4m3fn output",
+        "roofline": {"bound": "hbm", "achieved": alg / (st["avg"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg / (st["avg"] * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": alg},
     }
     if with_cpu:
         from oracle import oracle
 
-        rows = 2048  # 1/8 of the batch
-        xs_cpu = base[:rows].contiguous()
-        oracle.group_quant(xs_cpu[:64], G, mode="mul" if ue8m0 else "div", layout="ue8m0" if ue8m0 else "row")
-        t0 = time.perf_counter()
-        reps = 0
-        while time.perf_counter() - t0 < 10.0:
-            oracle.group_quant(xs_cpu, G, mode="mul" if ue8m0 else "div", layout="ue8m0" if ue8m0 else "row",
-                               pow2_floor=0.0 if ue8m0 else 1e-10)
-            reps += 1
-        dt = (time.perf_counter() - t0) / reps
+        rows = 2048
+        xc = base[:rows].contiguous()
+        kw = dict(mode="mul" if ue8m0 else "div", layout="ue8m0" if ue8m0 else "row", pow2_floor=0.0 if ue8m0 else 1e-10)
+        dt, reps = _cpu_time_boxed(lambda: oracle.group_quant(xc, G, **kw))
         rec["cpu_baseline"] = {
             "value": quant_algorithmic_bytes(rows, K, G, 2, ue8m0) / dt / 1e9, "unit": "GB/s",
             "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"first {rows} of {M} rows, {reps} repetitions (~10 s), C oracle with OpenMP",
+            "sample": f"first {rows} of {M} rows, {reps} repetitions in ~10 s, C oracle with OpenMP",
         }
     return rec
+
+
+# ------------------------------------------------------------------------------------------ FP8 GEMM
+
+def _device_fp8_codes(shape, gen, dev):
+    import torch
+
+    c = torch.randint(0, 256, shape, dtype=torch.uint8, device=dev, generator=gen)
+    return torch.where((c & 0x7F) == 0x7F, c & 0xF7, c).view(torch.float8_e4m3fn)  # no NaN codes
+
+
+def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
+    """One blockwise-FP8 linear through sgl_kernel.fp8_blockwise_scaled_mm (or, for N not a multiple of
+    128, through w8a8_block_fp8_matmul).  Activations are N(0,1)+outliers quantized by the GPU quantizer;
+    weights are random finite e4m3fn codes with block scales around 2e-4 (drawn on the device: the value
+    distribution does not change the timing, and drawing 2.6e8 Gaussians on the host would dominate the run)."""
+    import torch
+
+    from sglang_amd import fp8_kernel, sgl_kernel
+    from sglang_amd.workloads import cdiv, fp8_gemm_algorithmic_bytes, gemm_flops, make_activation
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(N * 10007 + K)
+    wbytes = N * K
+    nbuf = max(2, min(6, int(600e6 // wbytes) + 1))  # rotate through > 512 MB of weights when they are small
+    ws = [_device_fp8_codes((N, K), gen, dev) for _ in range(nbuf)]
+    wss = [(torch.rand(cdiv(N, 128), cdiv(K, 128), device=dev, generator=gen) + 0.5) * 2e-4 for _ in range(nbuf)]
+    x = make_activation(M, K).to(dev)
+    aligned = N % 128 == 0 and K % 128 == 0
+    x_q, x_s = fp8_kernel.per_token_group_quant_fp8(x, 128, column_major_scales=aligned)
+
+    if aligned:
+        def step(i):
+            return sgl_kernel.fp8_blockwise_scaled_mm(x_q, ws[i].t(), x_s, wss[i].t(), torch.bfloat16)
+    else:
+        def step(i):
+            return fp8_kernel.w8a8_block_fp8_matmul(x_q, ws[i], x_s, wss[i], [128, 128], torch.bfloat16)
+
+    wall, ms = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms)
+    flops = gemm_flops(M, N, K)
+    nbytes = fp8_gemm_algorithmic_bytes(M, N, K)
+    tflops_avg = flops / (st["avg"] * 1e-3) / 1e12
+    gbs_avg = nbytes / (st["avg"] * 1e-3) / 1e9
+    # which roof binds: time at peak MFMA rate vs time at peak HBM rate
+    mfma_bound = flops / (FP8_PEAK_TFLOPS * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9)
+    rec = {
+        "workload": f"fp8_gemm {name} M={M} K={K} N={N} (e4m3fn x e4m3fn, 1x128 / 128x128 fp32 scales, bf16 out)",
+        "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "gbytes_per_s": gbs_avg, "dtype": "fp8(e4m3fn) MFMA, f32 accumulate",
+        "roofline": ({"bound": "mfma", "achieved": tflops_avg, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                      "frac": tflops_avg / FP8_PEAK_TFLOPS, "traffic": None, "algorithmic_flops_per_launch": flops}
+                     if mfma_bound else
+                     {"bound": "hbm", "achieved": gbs_avg, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                      "frac": gbs_avg / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": nbytes}),
+    }
+    if with_cpu:
+        from oracle import oracle
+
+        ms_, ns_ = min(M, 64), min(N, 1024)
+        a_c, sa_c = x_q[:ms_].cpu().contiguous(), x_s[:ms_].cpu().contiguous()
+        w_c, sw_c = ws[0][:ns_].cpu().contiguous(), wss[0][: cdiv(ns_, 128)].cpu().contiguous()
+        dt, reps = _cpu_time_boxed(lambda: oracle.fp8_blockwise_mm(a_c, w_c, sa_c, sw_c, torch.bfloat16))
+        rec["cpu_baseline"] = {
+            "value": gemm_flops(ms_, ns_, K) / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(),
+            "kind": "port",
+            "sample": f"first {ms_} tokens x first {ns_} channels x full K={K}, {reps} repetitions in ~10 s, "
+                      "C oracle with OpenMP (fp64 block sums)",
+        }
+        # the reference's torch-native formulation (test_block_fp8.py:273-325) on the same sample, fp32 matmul per K block
+        A32, B32 = a_c.float(), w_c.float()
+
+        def native():
+            C = torch.zeros(ms_, ns_)
+            for kb in range(cdiv(K, 128)):
+                ks = slice(kb * 128, min((kb + 1) * 128, K))
+                C.add_((A32[:, ks] @ B32[:, ks].T) * (sa_c[:, kb:kb + 1] * sw_c[:, kb].repeat_interleave(128)[None, :ns_]))
+            return C.to(torch.bfloat16)
+
+        dt2, reps2 = _cpu_time_boxed(native, 5.0)
+        rec["cpu_baseline_torch_native"] = {
+            "value": gemm_flops(ms_, ns_, K) / dt2 / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "sample": f"same sample, {reps2} repetitions in ~5 s, torch fp32 matmul per K block",
+        }
+    return rec
+
+
+# ------------------------------------------------------------------------------------------ INT8 GEMM
+
+def bench_int8_gemm(name, M, K, N, steps, warmup):
+    import torch
+
+    from sglang_amd import sgl_kernel
+    from sglang_amd.workloads import gemm_flops, int8_gemm_algorithmic_bytes
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(N * 10009 + K)
+    nbuf = max(2, min(6, int(600e6 // (N * K)) + 1))
+    ws = [torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=gen) for _ in range(nbuf)]
+    a = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=gen)
+    sa = torch.rand(M, 1, device=dev, generator=gen) * 0.05
+    sb = torch.rand(N, device=dev, generator=gen) * 1e-3
+    bias = torch.randn(N, device=dev, generator=gen).to(torch.bfloat16)
+
+    def step(i):
+        return sgl_kernel.int8_scaled_mm(a, ws[i].t(), sa, sb, torch.bfloat16, bias)
+
+    wall, ms = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms)
+    ops_, nbytes = gemm_flops(M, N, K), int8_gemm_algorithmic_bytes(M, N, K)
+    tops, gbs = ops_ / (st["avg"] * 1e-3) / 1e12, nbytes / (st["avg"] * 1e-3) / 1e9
+    mfma_bound = ops_ / (INT8_PEAK_TOPS * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9)
+    return {
+        "workload": f"int8_gemm {name} M={M} K={K} N={N} (int8 x int8 -> int32, per-token x per-channel scales, bias, bf16 out)",
+        "value": ops_ / (wall / steps) / 1e12, "unit": "TOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "gbytes_per_s": gbs, "dtype": "int8 MFMA, int32 accumulate",
+        "roofline": ({"bound": "mfma", "achieved": tops, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                      "frac": tops / INT8_PEAK_TOPS, "traffic": None}
+                     if mfma_bound else
+                     {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                      "frac": gbs / HBM_PEAK_GBS, "traffic": None}),
+    }
 
 
 def main():
@@ -122,12 +252,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="default")
+    ap.add_argument("--workload", default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--quick", action="store_true", help="headline only (no 'also' list)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this path is measured on ONE GPU; it has no collectives and --gpus N>1 is not run "
-              "(see DESIGN.md, 'How the path shards').", file=sys.stderr)
+        print("bench.py: this path is measured on ONE GPU; it contains no collective, and a run with --gpus N>1 "
+              "is not provided (DESIGN.md, 'How the path would shard').", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -136,37 +267,43 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     from sglang_amd import _lib
+    from sglang_amd.workloads import DSV3_MLA, DSV3_MLP, LLAMA3_8B
 
     _lib.lib()  # fail loudly if the HIP library is missing
 
-    with_cpu = not args.no_cpu
+    S, W, cpu = args.steps, args.warmup, not args.no_cpu
+    also = []
     if args.workload in ("quant", "quant_ue8m0"):
-        rec = bench_quant(args.steps, args.warmup, args.workload == "quant_ue8m0", with_cpu)
-        also = []
+        rec = bench_quant(S, W, args.workload == "quant_ue8m0", cpu)
     else:
-        rec = bench_quant(args.steps, args.warmup, False, with_cpu)
-        also = [bench_quant(args.steps, args.warmup, True, False)]
+        K, N = DSV3_MLP["gate_up"]
+        rec = bench_fp8_gemm("gate_up", 4096, K, N, S, W, cpu)
+        if args.workload == "all" and not args.quick:
+            also.append(bench_quant(S, W, False, cpu))
+            also.append(bench_quant(S, W, True, False))
+            K, N = DSV3_MLP["down"]
+            also.append(bench_fp8_gemm("down", 4096, K, N, S, W, False))
+            for nm, (K, N) in DSV3_MLA.items():
+                also.append(bench_fp8_gemm(nm, 4096, K, N, S, W, False))
+            for M in (1, 8, 32, 128):
+                for nm, (K, N) in DSV3_MLP.items():
+                    also.append(bench_fp8_gemm(nm, M, K, N, S, W, False))
+            also.append(bench_fp8_gemm("single_linear", 16, 7168, 2048, S, W, cpu))
+            for M in (1, 256, 4096):
+                for nm, (K, N) in LLAMA3_8B.items():
+                    also.append(bench_int8_gemm(nm, M, K, N, S, W))
 
     line = {
-        "metric": METRIC,
-        "value": rec["value"],
-        "unit": rec["unit"],
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": rec["ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
+        "metric": METRIC, "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": S, "warmup": W,
+        "ms_per_step": rec["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": rec["dtype"],
-        "data": "synthetic (seeded torch.Generator on CPU, copied to HBM before timing)",
+        "data": "synthetic, seeded; resident in HBM before the timed region",
         "config": {"workload": rec["workload"]},
-        "roofline": rec["roofline"],
-        "kernel_ms": {"avg": rec["kernel_ms_avg"], "median": rec["kernel_ms_median"],
-                      "p20_p80": rec["kernel_ms_p20_p80"]},
+        "roofline": rec["roofline"], "kernel_ms": rec["kernel_ms"],
     }
-    if "cpu_baseline" in rec:
-        line["cpu_baseline"] = rec["cpu_baseline"]
+    for k in ("cpu_baseline", "cpu_baseline_torch_native", "gbytes_per_s"):
+        if k in rec:
+            line[k] = rec[k]
     if also:
         line["also"] = also
     print(json.dumps(line))
