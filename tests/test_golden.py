@@ -1,0 +1,97 @@
+"""Golden fixtures (tests/golden/qlinear_golden.npz, written by tests/golden/make_golden.py).
+
+CPU: the oracle must still reproduce them (guards the checker itself against regressions).
+GPU: the HIP kernels must reproduce them without the oracle in the loop."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "qlinear_golden.npz")
+FP8 = torch.float8_e4m3fn
+
+
+@pytest.fixture(scope="module")
+def gold():
+    z = np.load(GOLD, allow_pickle=False)
+    return {k: torch.from_numpy(z[k].copy()) for k in z.files}
+
+
+def _bf16(t):
+    return t.view(torch.bfloat16)
+
+
+def _f32(t):
+    return t.view(torch.float32)
+
+
+def test_oracle_reproduces_quant_fixtures(oracle, gold):
+    x = _bf16(gold["quant_x_bf16"])
+    for mode, floor in (("div", 1e-10), ("rcp", 0.0), ("mul", 0.0)):
+        q, s = oracle.group_quant(x, 128, mode=mode)
+        assert torch.equal(q.view(torch.uint8), gold[f"quant_{mode}_q"])
+        assert torch.equal(s.view(torch.int32), gold[f"quant_{mode}_s_f32"])
+        q, s = oracle.group_quant(x, 128, mode=mode, layout="ue8m0", pow2_floor=floor)
+        assert torch.equal(q.view(torch.uint8), gold[f"quant_{mode}_ue8m0_q"])
+        assert torch.equal(oracle.unpack_ue8m0(s, 4), gold[f"quant_{mode}_ue8m0_bytes"])
+    q, s = oracle.group_quant(x, 128, mode="div", dst_dtype=torch.int8)
+    assert torch.equal(q, gold["quant_div_int8_q"]) and torch.equal(s.view(torch.int32), gold["quant_div_int8_s_f32"])
+    pq, ps = oracle.per_token_quant_int8(x)
+    assert torch.equal(pq, gold["ptq_q"]) and torch.equal(ps.view(torch.int32), gold["ptq_s_f32"])
+
+
+def test_oracle_reproduces_gemm_fixtures(oracle, gold):
+    aq, asc = gold["gemm_a_q"].view(FP8), _f32(gold["gemm_a_s_f32"])
+    wq, ws = gold["gemm_w_q"].view(FP8), _f32(gold["gemm_w_s_f32"])
+    assert torch.equal(oracle.fp8_blockwise_mm(aq, wq, asc, ws, torch.float32).view(torch.int32), gold["gemm_out_f32"])
+    assert torch.equal(oracle.fp8_blockwise_mm(aq, wq, asc, ws, torch.bfloat16).view(torch.int16), gold["gemm_out_bf16"])
+    acc = oracle.int8_mm_acc(gold["int8_a"], gold["int8_w"])
+    assert torch.equal(acc, gold["int8_acc"])
+    out = oracle.int8_epilogue(acc, _f32(gold["int8_sa_f32"]), _f32(gold["int8_sb_f32"]), torch.bfloat16,
+                               _bf16(gold["int8_bias_bf16"]))
+    assert torch.equal(out.view(torch.int16), gold["int8_out_bf16"])
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_quant_fixtures(gpu, gold):
+    from sglang_amd.fp8_kernel import per_token_group_quant_fp8, sglang_per_token_group_quant_8bit
+    from sglang_amd.int8_kernel import per_token_quant_int8
+
+    x = _bf16(gold["quant_x_bf16"]).to(gpu)
+    q, s = per_token_group_quant_fp8(x, 128)  # Triton row-major arithmetic: x * (1/s)
+    assert torch.equal(q.cpu().view(torch.uint8), gold["quant_rcp_q"])
+    assert torch.equal(s.cpu().view(torch.int32), gold["quant_rcp_s_f32"])
+    for v2, mode in ((False, "div"), (True, "mul")):
+        q, s = sglang_per_token_group_quant_8bit(x, 128, FP8, enable_v2=v2)
+        assert torch.equal(q.cpu().view(torch.uint8), gold[f"quant_{mode}_q"])
+        assert torch.equal(s.cpu().view(torch.int32), gold[f"quant_{mode}_s_f32"])
+        q, s = sglang_per_token_group_quant_8bit(x, 128, FP8, column_major_scales=True, scale_tma_aligned=True,
+                                                 scale_ue8m0=True, enable_v2=v2)
+        assert torch.equal(q.cpu().view(torch.uint8), gold[f"quant_{mode}_ue8m0_q"])
+        dense = torch.empty(tuple(s.shape), dtype=torch.int32)
+        dense.copy_(s.cpu())
+        assert torch.equal(dense.view(torch.uint8).reshape(s.shape[0], -1)[:, :4], gold[f"quant_{mode}_ue8m0_bytes"])
+    q, s = sglang_per_token_group_quant_8bit(x, 128, torch.int8, enable_v2=False)
+    assert torch.equal(q.cpu(), gold["quant_div_int8_q"]) and torch.equal(s.cpu().view(torch.int32), gold["quant_div_int8_s_f32"])
+    pq, ps = per_token_quant_int8(x)
+    assert torch.equal(pq.cpu(), gold["ptq_q"]) and torch.equal(ps.cpu().view(torch.int32), gold["ptq_s_f32"])
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_gemm_fixtures(gpu, gold):
+    from sglang_amd import ops
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
+    from sglang_amd.sgl_kernel import int8_scaled_mm
+
+    aq, asc = gold["gemm_a_q"].view(FP8).to(gpu), _f32(gold["gemm_a_s_f32"]).to(gpu)
+    wq, ws = gold["gemm_w_q"].view(FP8).to(gpu), _f32(gold["gemm_w_s_f32"]).to(gpu)
+    ref = _f32(gold["gemm_out_f32"])
+    out = w8a8_block_fp8_matmul(aq, wq, asc, ws, [128, 128], torch.float32).cpu()
+    # floating point: |err| <= 1e-2 |ref| + 1e-4 * (sum of |terms|), here bounded by K * max|term| ~ row scale
+    assert bool(((out - ref).abs() <= 1e-2 * ref.abs() + 1e-4 * ref.abs().max()).all())
+    a, w = gold["int8_a"].to(gpu), gold["int8_w"].to(gpu)
+    assert torch.equal(ops.int8_mm_raw_accumulators(a, w.t()).cpu(), gold["int8_acc"])
+    out = int8_scaled_mm(a, w.t(), _f32(gold["int8_sa_f32"]).to(gpu), _f32(gold["int8_sb_f32"]).to(gpu), torch.bfloat16,
+                         _bf16(gold["int8_bias_bf16"]).to(gpu))
+    assert torch.equal(out.cpu().view(torch.int16), gold["int8_out_bf16"])
