@@ -1,0 +1,96 @@
+// Shared declarations of the gfx950 GEMM kernels: vector types, launch parameters, output store, tile order.
+#pragma once
+
+#include <type_traits>
+
+#include "common.h"
+
+namespace mi355 {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int KSTEP = 128;   // bytes of K per row and stage
+constexpr int THREADS = 256;
+constexpr int GROUP_M = 8;    // M-tiles per group in the tile order
+
+struct GemmParams {
+  const uint8_t* a;  // tokens   [M, K], row stride lda
+  const uint8_t* b;  // channels [N, K], row stride ldb
+  const float* sa;
+  const float* sb;
+  const void* bias;
+  void* out;
+  void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
+  int M, N, K;
+  int64_t lda, ldb, ldo;
+  int64_t sa_sm, sa_sk, sb_sn, sb_sk;
+  int kb_total, kb_per_split, splits;
+  int tiles_m, tiles_n;
+  int out_dtype;
+};
+
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off, const float* r, int nvalid,
+                                           bool vec_ok) {
+  if (out_dtype == MI355_F32) {
+    float* o = reinterpret_cast<float*>(out) + off;
+    if (nvalid == 4 && vec_ok) {
+      *reinterpret_cast<v4f*>(o) = v4f{r[0], r[1], r[2], r[3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i < nvalid) o[i] = r[i];
+    }
+    return;
+  }
+  uint32_t h[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) h[i] = (out_dtype == MI355_BF16) ? f32_to_bf16_bits(r[i]) : f32_to_f16_bits(r[i]);
+  uint16_t* o = reinterpret_cast<uint16_t*>(out) + off;
+  if (nvalid == 4 && vec_ok) {
+    *reinterpret_cast<u32x2*>(o) = u32x2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < nvalid) o[i] = (uint16_t)h[i];
+  }
+}
+
+
+struct TileCoord {
+  int tile_m, tile_n, split;
+};
+
+// Workgroup -> output tile.  Consecutive workgroup ids go round-robin to the 8 XCDs (each with its own L2), so
+// ids are first renumbered to give every XCD a contiguous range; inside a range tiles are walked GROUP_M
+// M-tiles at a time, so that the tiles an XCD works on concurrently share weight and token rows in its L2.
+__device__ __forceinline__ TileCoord tile_of_block(int bid, int total, int tiles_m, int tiles_n) {
+  const int per = total >> 3;
+  if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
+  const int tiles_mn = tiles_m * tiles_n;
+  TileCoord c;
+  c.split = bid / tiles_mn;
+  const int lid = bid - c.split * tiles_mn;
+  const int per_group = GROUP_M * tiles_n;
+  const int group = lid / per_group;
+  const int first_m = group * GROUP_M;
+  const int gm = min(tiles_m - first_m, GROUP_M);
+  const int in_group = lid - group * per_group;
+  c.tile_m = first_m + in_group % gm;
+  c.tile_n = in_group / gm;
+  return c;
+}
+
+// Large-M blockwise FP8 GEMM (256 x 128 tile, three LDS stages, software-pipelined); gemm_fp8_pipelined.hip.
+// Needs 16-byte aligned rows and K % 16 == 0.  Returns an MI355_* status.
+int launch_fp8_pipelined(GemmParams& p, hipStream_t stream, const char* what);
+
+// Large-M blockwise FP8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, two LDS stages); gemm_fp8_dma.hip.
+// Same requirements.
+int launch_fp8_dma(GemmParams& p, hipStream_t stream, const char* what);
+
+}  // namespace mi355

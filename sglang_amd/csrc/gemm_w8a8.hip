@@ -20,64 +20,10 @@
 //     workspace and a second kernel adds them in a fixed order (deterministic, no atomics);
 //   * workgroups are renumbered so that each of the 8 XCDs (own L2) works on a contiguous, M-grouped
 //     patch of output tiles.
-#include <type_traits>
-
-#include "common.h"
+#include "gemm_common.h"
 
 namespace mi355 {
 namespace {
-
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-constexpr int KSTEP = 128;   // bytes of K per row and stage
-constexpr int THREADS = 256;
-
-struct GemmParams {
-  const uint8_t* a;  // tokens   [M, K], row stride lda
-  const uint8_t* b;  // channels [N, K], row stride ldb
-  const float* sa;
-  const float* sb;
-  const void* bias;
-  void* out;
-  void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
-  int M, N, K;
-  int64_t lda, ldb, ldo;
-  int64_t sa_sm, sa_sk, sb_sn, sb_sk;
-  int kb_total, kb_per_split, splits;
-  int tiles_m, tiles_n;
-  int out_dtype;
-};
-
-// ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off, const float* r, int nvalid,
-                                           bool vec_ok) {
-  if (out_dtype == MI355_F32) {
-    float* o = reinterpret_cast<float*>(out) + off;
-    if (nvalid == 4 && vec_ok) {
-      *reinterpret_cast<v4f*>(o) = v4f{r[0], r[1], r[2], r[3]};
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (i < nvalid) o[i] = r[i];
-    }
-    return;
-  }
-  uint32_t h[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) h[i] = (out_dtype == MI355_BF16) ? f32_to_bf16_bits(r[i]) : f32_to_f16_bits(r[i]);
-  uint16_t* o = reinterpret_cast<uint16_t*>(out) + off;
-  if (nvalid == 4 && vec_ok) {
-    *reinterpret_cast<u32x2*>(o) = u32x2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
-  } else {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (i < nvalid) o[i] = (uint16_t)h[i];
-  }
-}
 
 // IS_FP8: blockwise-scaled fp8 (fp32 accumulators) or int8 (int32 accumulators).
 // BM x BN macro tile, WGM x WGN waves (WGM * WGN == 4).
@@ -105,24 +51,8 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const GemmParams p) {
   const int wave_m = wave / WGN, wave_n = wave % WGN;
   const int l16 = lane & 15, q = lane >> 4;
 
-  // ---- which tile: XCD-contiguous, M-grouped order
-  int bid = blockIdx.x;
-  {
-    const int total = gridDim.x;
-    const int per = total >> 3;
-    if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
-  }
-  const int tiles_mn = p.tiles_m * p.tiles_n;
-  const int split = bid / tiles_mn;
-  const int lid = bid - split * tiles_mn;
-  constexpr int GROUP_M = 8;
-  const int per_group = GROUP_M * p.tiles_n;
-  const int group = lid / per_group;
-  const int first_m = group * GROUP_M;
-  const int gm = min(p.tiles_m - first_m, GROUP_M);
-  const int in_group = lid - group * per_group;
-  const int tile_m = first_m + in_group % gm;
-  const int tile_n = in_group / gm;
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
+  const int tile_m = tc.tile_m, tile_n = tc.tile_n, split = tc.split;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int kb_begin = split * p.kb_per_split;
@@ -190,19 +120,21 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const GemmParams p) {
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[i][j][v] = 0;
 
-  // operand fragment addresses inside a stage (swizzled); constant over K
+  // operand fragment addresses inside a stage (swizzled); constant over K.  Lane quarter q takes the 16-byte
+  // chunks q and q + 4 of a row: with this mapping a ds_read_b128 runs at the full 256 B/clk of the gfx950 LDS
+  // (chunks 2q, 2q+1 measure at half of that).  Both operands use the same mapping, so the dot product is unchanged.
   uint32_t tok_off[MT][2], ch_off[NT][2];
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
     const int row = wave_m * WM + j * 16 + l16;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) tok_off[j][h] = row * KSTEP + (((2 * q + h) ^ (row & 7)) << 4);
+    for (int h = 0; h < 2; ++h) tok_off[j][h] = row * KSTEP + (((q + 4 * h) ^ (row & 7)) << 4);
   }
 #pragma unroll
   for (int i = 0; i < NT; ++i) {
     const int row = BM + wave_n * WN + i * 16 + l16;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) ch_off[i][h] = row * KSTEP + (((2 * q + h) ^ (row & 7)) << 4);
+    for (int h = 0; h < 2; ++h) ch_off[i][h] = row * KSTEP + (((q + 4 * h) ^ (row & 7)) << 4);
   }
   // one 128x128 weight block holds all of this wave's channels
   const int nb = min(n0 + wave_n * WN, p.N - 1) / 128;
@@ -458,7 +390,20 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
   }
   const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
                        ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
-  switch (pl.bm) {
+  if constexpr (IS_FP8) {
+    // the pipelined kernel addresses rows with 32-bit byte offsets from the matrix base
+    const bool small_offsets = (int64_t)p.M * p.lda < (1ll << 32) && (int64_t)p.N * p.ldb < (1ll << 32);
+    if (pl.bm == 256 && pl.splits == 1 && aligned && small_offsets) {
+      // 256 x 256 tiles (8 waves, direct-to-LDS) when they still give every CU a workgroup, else 256 x 128
+      const int64_t tiles_256 = ((int64_t)(p.M + 255) / 256) * ((p.N + 255) / 256);
+      const int64_t tiles_128 = ((int64_t)(p.M + 255) / 256) * ((p.N + 127) / 128);
+      if (tiles_256 >= NUM_CUS) return launch_fp8_dma(p, stream, what);
+      if (tiles_128 >= NUM_CUS) return launch_fp8_pipelined(p, stream, what);
+    }
+  }
+  int bm = pl.bm;
+  if (bm == 256 && ((int64_t)(p.M + 255) / 256) * ((p.N + 127) / 128) < NUM_CUS) bm = 128;  // too few 256-row tiles to fill the chip
+  switch (bm) {
     case 16: return launch_tile<IS_FP8, 16, 128, 1, 4>(p, aligned, stream, what);
     case 32: return launch_tile<IS_FP8, 32, 128, 1, 4>(p, aligned, stream, what);
     case 64: return launch_tile<IS_FP8, 64, 128, 1, 4>(p, aligned, stream, what);

@@ -185,3 +185,23 @@ def test_full_size_prefill_shape_properties(gpu, oracle):
     _check(out[rows.to(gpu)], ref, mag, "sampled rows")
     out2 = w8a8_block_fp8_matmul(ag, wg, Asg * 2, Bsg, [128, 128], torch.bfloat16)
     assert torch.equal(out2.float(), out.float() * 2)
+
+
+# Large-M kernels: 256x256 direct-to-LDS tiles (>= 256 such tiles) and 256x128 pipelined tiles, each with K a multiple of
+# 128 and not, and with ragged M and N edges.  The oracle checks a sample of rows (first, last, tile borders, random).
+@pytest.mark.parametrize("M,N,K", [(4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 512), (4000, 2100, 272),
+                                   (8192, 2048, 1024)])
+def test_large_m_kernels(gpu, oracle, M, N, K):
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
+
+    print(f"case M={M} N={N} K={K}", flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    a, w = _rand_fp8((M, K), g), _rand_fp8((N, K), g)
+    As = torch.rand(M, cdiv(K, 128), generator=g) * 1e-2
+    Bs = torch.rand(cdiv(N, 128), cdiv(K, 128), generator=g) * 1e-2
+    out = w8a8_block_fp8_matmul(a.to(gpu), w.to(gpu), As.to(gpu), Bs.to(gpu), [128, 128], torch.bfloat16)
+    rows = torch.cat([torch.tensor([0, 1, 127, 128, 255, 256, 257, M - 257, M - 256, M - 2, M - 1]),
+                      torch.randperm(M, generator=g)[:40]])
+    ref, mag = oracle.fp8_blockwise_mm(a[rows].contiguous(), w, As[rows].contiguous(), Bs, torch.float32, want_abs=True)
+    _check(out[rows.to(gpu)], ref, mag, f"M={M} N={N} K={K}")
+    assert bool(torch.isfinite(out).all())
