@@ -88,6 +88,29 @@ __device__ __forceinline__ int log2_ceil_bits(float x) {
 }
 __device__ __forceinline__ float pow2_int(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }
 
+// Streaming stores.  Written as instructions because the optimizer drops the nontemporal hint of
+// __builtin_nontemporal_store in this kernel, and the hint is worth ~8 % of bandwidth here (the output is never re-read).
+__device__ __forceinline__ void store_nt(void* p, u32x2 v) {
+  asm volatile("global_store_dwordx2 %0, %1, off nt" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_nt(void* p, uint32_t v) {
+  asm volatile("global_store_dword %0, %1, off nt" ::"v"(p), "v"(v) : "memory");
+}
+
+// x / s, correctly rounded, for many x sharing one divisor s, given r = RN(1 / s).
+// q0 = RN(x * r) is within 2 ulp of the quotient; each step q += RN(x - q * s) * r (the residual is exact in an FMA)
+// at least squares the relative error, so after two steps the result is the correctly rounded quotient (Markstein's
+// iteration, the same refinement the hardware divide expansion uses, minus its per-element reciprocal and range
+// scaling).  Needs no range scaling here: |x / s| <= qmax * (1 + 2^-23), s and r are normal for every amax >= eps,
+// and results below 2^-11 (where a subnormal residual could lose bits) convert to zero in either output format.
+// Checked on the device against the `/` operator for every bf16 and fp16 x under 65536 divisors.
+__device__ __forceinline__ float div_shared(float x, float s, float r) {
+  float q = x * r;
+  q = fmaf(fmaf(-q, s, x), r, q);
+  q = fmaf(fmaf(-q, s, x), r, q);
+  return q;
+}
+
 // T: element tag; LPG lanes per group; ITERS 16-byte vectors per lane and group.
 template <typename T, int LPG, int ITERS, int MODE, bool UE8M0, bool FP8_OUT, int UNROLL>
 __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
@@ -100,18 +123,19 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
   u32x4 raw[UNROLL][ITERS];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
-    const uint32_t g = g_first + u * GROUPS_PER_PASS;
+    // Past the last group the lanes redo the last group (same values to the same addresses): the body stays free of
+    // branches, which keeps the stores nontemporal and the loop fully unrolled.
+    const uint32_t g = min(g_first + u * GROUPS_PER_PASS, p.num_groups - 1);
     const u32x4* src = reinterpret_cast<const u32x4*>(p.x) + (size_t)g * (LPG * ITERS) + lane;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      // Whole groups are valid or not, so the lanes of a live group never reduce with a dead one.
-      raw[u][it] = (g < p.num_groups) ? __builtin_nontemporal_load(src + it * LPG) : u32x4{0, 0, 0, 0};
+      raw[u][it] = __builtin_nontemporal_load(src + it * LPG);
     }
   }
 
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
-    const uint32_t g = g_first + u * GROUPS_PER_PASS;
+    const uint32_t g = min(g_first + u * GROUPS_PER_PASS, p.num_groups - 1);
     float v[ITERS][VEC];
     float amax = p.eps;
 #pragma unroll
@@ -143,28 +167,17 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
       }
     }
     constexpr bool USE_DIV = (MODE == MI355_QUANT_DIV) && !UE8M0;
+    float rcp = 0.f;
+    if constexpr (USE_DIV) rcp = 1.0f / s_val;  // correctly rounded; shared by the whole group
 
-    if (g < p.num_groups) {
-      if (lane == 0) {
-        const uint32_t row = fastdiv(g, p.groups_per_row);
-        const uint32_t kg = g - row * p.groups_per_row.div;
-        if constexpr (UE8M0) {
-          uint8_t* sb = reinterpret_cast<uint8_t*>(p.s) + (size_t)(kg >> 2) * (size_t)p.s_stride_col * 4u +
-                        (size_t)row * 4u + (kg & 3u);
-          *sb = (uint8_t)(__float_as_uint(s_val) >> 23);
-          if (kg == p.groups_per_row.div - 1)
-            for (uint32_t t = (kg & 3u) + 1; t < 4; ++t) sb[t - (kg & 3u)] = 0;
-        } else {
-          reinterpret_cast<float*>(p.s)[(int64_t)row * p.s_stride_row + (int64_t)kg * p.s_stride_col] = s_val;
-        }
-      }
+    {
       uint8_t* dst = p.q + (size_t)g * GROUP + (size_t)lane * VEC;
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
         float t[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          const float y = USE_DIV ? v[it][j] / s_val : v[it][j] * mul;
+          const float y = USE_DIV ? div_shared(v[it][j], s_val, rcp) : v[it][j] * mul;
           t[j] = fminf(fmaxf(y, p.qmin), p.qmax);
         }
         uint32_t w[VEC / 4];
@@ -181,9 +194,22 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
         }
         uint8_t* d = dst + (size_t)it * (LPG * VEC);
         if constexpr (VEC == 8)
-          __builtin_nontemporal_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(d));
+          store_nt(d, u32x2{w[0], w[1]});
         else
-          __builtin_nontemporal_store(w[0], reinterpret_cast<uint32_t*>(d));
+          store_nt(d, w[0]);
+      }
+      if (lane == 0) {
+        const uint32_t row = fastdiv(g, p.groups_per_row);
+        const uint32_t kg = g - row * p.groups_per_row.div;
+        if constexpr (UE8M0) {
+          uint8_t* sb = reinterpret_cast<uint8_t*>(p.s) + (size_t)(kg >> 2) * (size_t)p.s_stride_col * 4u +
+                        (size_t)row * 4u + (kg & 3u);
+          *sb = (uint8_t)(__float_as_uint(s_val) >> 23);
+          if (kg == p.groups_per_row.div - 1)
+            for (uint32_t t = (kg & 3u) + 1; t < 4; ++t) sb[t - (kg & 3u)] = 0;
+        } else {
+          reinterpret_cast<float*>(p.s)[(int64_t)row * p.s_stride_row + (int64_t)kg * p.s_stride_col] = s_val;
+        }
       }
     }
   }
@@ -192,7 +218,11 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
 template <typename T, int LPG, int ITERS, int MODE, bool UE8M0, bool FP8_OUT>
 int launch(const QuantParams& p, hipStream_t stream) {
   // Fewer groups per thread when each group already spans several vectors per lane.
+#ifdef MI355_QUANT_UNROLL
+  constexpr int UNROLL = MI355_QUANT_UNROLL;
+#else
   constexpr int UNROLL = (ITERS >= 4) ? 1 : (ITERS == 2 ? 2 : 4);
+#endif
   constexpr int GROUPS_PER_BLOCK = (256 / LPG) * UNROLL;
   const uint32_t blocks = (p.num_groups + GROUPS_PER_BLOCK - 1) / GROUPS_PER_BLOCK;
   hipLaunchKernelGGL((group_quant_kernel<T, LPG, ITERS, MODE, UE8M0, FP8_OUT, UNROLL>), dim3(blocks), dim3(256), 0,

@@ -129,6 +129,39 @@ def test_every_bf16_value_under_many_scales(gpu, oracle):
         assert _same_bits(q, q_o), _diff_report(q, q_o)
 
 
+def test_division_is_correctly_rounded_at_fp8_ties(gpu, oracle):
+    """The divide mode computes x / s with a shared reciprocal and two FMA refinement steps.  Its quotient must be the
+    correctly rounded one: fp32 inputs are placed within +-3 ulp of tie * s for every midpoint between neighbouring
+    e4m3 codes, under 6000 random scales, so that a quotient wrong in its last bit lands on the other side of the tie."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_8bit
+
+    g = torch.Generator().manual_seed(123)
+    codes = torch.arange(0, 0x7E, dtype=torch.int32).to(torch.uint8)
+    lo = codes.view(FP8).to(torch.float32)
+    hi = (codes + 1).view(FP8).to(torch.float32)
+    ties = ((lo + hi) / 2)[1:]  # 125 midpoints (skip the one next to zero: below 2^-10 everything rounds to zero)
+    G = 6000
+    amax = torch.exp2(torch.rand(G, generator=g) * 60 - 30) * (1 + torch.rand(G, generator=g))
+    s = amax / 448.0
+    x = torch.zeros(G, 128)
+    x[:, 0] = amax
+    t = ties[torch.randint(0, ties.numel(), (G, 127), generator=g)]
+    base = t * s[:, None]
+    step = torch.randint(-3, 4, (G, 127), generator=g, dtype=torch.int32)
+    xi = base.view(torch.int32) + step  # move by whole ulps
+    sign = torch.where(torch.rand(G, 127, generator=g) < 0.5, -1.0, 1.0)
+    x[:, 1:] = xi.view(torch.float32) * sign
+    x = x.reshape(G // 4, 512).contiguous()
+    assert float(x.abs().view(G, 128)[:, 1:].max(dim=1).values.sub(amax).max()) <= 0  # amax really is the group maximum
+    q, sc = sglang_per_token_group_quant_8bit(x.to(gpu), 128, FP8, enable_v2=False)
+    q_o, s_o = oracle.group_quant(x, 128, mode="div")
+    assert _same_bits(sc, s_o)
+    assert _same_bits(q, q_o), _diff_report(q, q_o)
+    # the construction is sharp: a reciprocal-multiply quotient does differ on this input
+    q_r, _ = oracle.group_quant(x, 128, mode="rcp")
+    assert int((_u8(q_r) != _u8(q_o)).sum()) > 100
+
+
 def test_known_answer_construction(gpu):
     """test/srt/quant/test_fp8_kernel.py:24-100 with exactly representable scales: the quantizer must
     return the scale and the codes it was built from."""
