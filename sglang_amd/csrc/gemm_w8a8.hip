@@ -330,10 +330,20 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
   return pl;
 }
 
-size_t workspace_bytes(int64_t M, int64_t N, int64_t K) {
+constexpr int64_t DECODE_MAX_M = 16;  // beyond one token tile the LDS-tiled kernel amortizes the token fetch better
+
+// Upper bound over the kernels a shape may be routed to (the choice also depends on pointer alignment, which is not
+// known here).
+size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const Plan pl = make_plan(M, N, K);
-  return pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
+  size_t need = pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
+  if (is_fp8 && M <= DECODE_MAX_M) {
+    const int ds = decode_splits(M, N, K);
+    const size_t dneed = ds > 1 ? (size_t)ds * (size_t)M * (size_t)N * 4u : 0;
+    if (dneed > need) need = dneed;
+  }
+  return need;
 }
 
 template <bool IS_FP8, int BM, int BN, int WGM, int WGN>
@@ -376,8 +386,29 @@ int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* wha
 
 template <bool IS_FP8>
 int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipStream_t stream, const char* what) {
-  const Plan pl = make_plan(p.M, p.N, p.K);
   p.kb_total = (p.K + KSTEP - 1) / KSTEP;
+  const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
+                       ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
+  if constexpr (IS_FP8) {
+    if (p.M <= DECODE_MAX_M && aligned) {  // weight streaming without LDS
+      p.splits = decode_splits(p.M, p.N, p.K);
+      p.kb_per_split = (p.kb_total + p.splits - 1) / p.splits;
+      if (p.splits > 1) {
+        const size_t need = (size_t)p.splits * (size_t)p.M * (size_t)p.N * 4u;
+        MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
+                      "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
+        MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
+                      "%s: workspace must be 16-byte aligned", what);
+        p.ws = workspace;
+      }
+      int rc = launch_fp8_decode(p, stream, what);
+      if (rc != MI355_OK || p.splits == 1) return rc;
+      const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
+      hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
+      return check_launch(what);
+    }
+  }
+  const Plan pl = make_plan(p.M, p.N, p.K);
   p.splits = pl.splits;
   p.kb_per_split = pl.kb_per_split;
   if (pl.splits > 1) {
@@ -388,8 +419,6 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
                   "%s: workspace must be 16-byte aligned", what);
     p.ws = workspace;
   }
-  const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
-                       ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
   if constexpr (IS_FP8) {
     // the pipelined kernel addresses rows with 32-bit byte offsets from the matrix base
     const bool small_offsets = (int64_t)p.M * p.lda < (1ll << 32) && (int64_t)p.N * p.ldb < (1ll << 32);
@@ -418,7 +447,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
 using namespace mi355;
 
 extern "C" size_t mi355_fp8_blockwise_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  return workspace_bytes(M, N, K);
+  return workspace_bytes(M, N, K, true);
 }
 
 extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const float* sb, void* out,
@@ -449,7 +478,7 @@ extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float*
 }
 
 extern "C" size_t mi355_int8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  return workspace_bytes(M, N, K);
+  return workspace_bytes(M, N, K, false);
 }
 
 extern "C" int mi355_int8_scaled_mm(const void* a, const void* b, const float* sa, const float* sb, const void* bias,
