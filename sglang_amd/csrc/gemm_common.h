@@ -94,6 +94,10 @@ int launch_fp8_pipelined(GemmParams& p, hipStream_t stream, const char* what);
 int launch_fp8_dma(GemmParams& p, hipStream_t stream, const char* what);
 
 
+// Large-M INT8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, 32x32x32 MFMA); gemm_int8_dma.hip.
+// Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
+int launch_int8_dma(GemmParams& p, hipStream_t stream, const char* what);
+
 // Small-M blockwise FP8 GEMM streaming the weight through wave-private LDS, no barriers; gemm_fp8_decode.hip.
 // decode_splits() is the split count it wants for a shape; the caller sets p.splits, p.kb_per_split and p.ws.
 int decode_splits(int64_t M, int64_t N, int64_t K);

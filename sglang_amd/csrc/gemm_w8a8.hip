@@ -430,6 +430,12 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
       if (tiles_128 >= NUM_CUS) return launch_fp8_pipelined(p, stream, what);
     }
   }
+  if constexpr (!IS_FP8) {
+    const bool small_offsets = (int64_t)p.M * p.lda < (1ll << 32) && (int64_t)p.N * p.ldb < (1ll << 32);
+    const int64_t tiles_256 = ((int64_t)(p.M + 255) / 256) * ((p.N + 255) / 256);
+    if (pl.bm == 256 && pl.splits == 1 && aligned && small_offsets && p.K % KSTEP == 0 && tiles_256 >= NUM_CUS / 2)
+      return launch_int8_dma(p, stream, what);
+  }
   int bm = pl.bm;
   if (bm == 256 && ((int64_t)(p.M + 255) / 256) * ((p.N + 127) / 128) < NUM_CUS) bm = 128;  // too few 256-row tiles to fill the chip
   switch (bm) {

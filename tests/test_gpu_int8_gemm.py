@@ -77,6 +77,30 @@ def test_int8_scaled_mm(gpu, oracle, M, N, K, with_bias, out_dtype):
     torch.testing.assert_close(out.cpu(), o.to(out_dtype))
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 512), (4000, 4088, 1024), (2048, 8192, 256)])
+def test_large_m_kernel(gpu, oracle, M, N, K):
+    """The 256x256 direct-to-LDS kernel (32x32x32 MFMA): raw accumulators and epilogue on a sample of rows that includes
+    tile borders and the ragged last tile, all columns."""
+    from sglang_amd import ops
+    from sglang_amd.sgl_kernel import int8_scaled_mm
+
+    print(f"case M={M} N={N} K={K}", flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int8)
+    w = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int8)
+    sa, sb = torch.rand(M, generator=g) * 0.1, torch.rand(N, generator=g) * 0.01
+    bias = (torch.randn(N, generator=g) * 10).to(torch.bfloat16)
+    ag, wg = a.to(gpu), w.to(gpu)
+    acc = ops.int8_mm_raw_accumulators(ag, wg.t())
+    out = int8_scaled_mm(ag, wg.t(), sa.to(gpu), sb.to(gpu), torch.bfloat16, bias.to(gpu))
+    rows = torch.cat([torch.tensor([0, 31, 32, 127, 128, 255, 256, M - 257, M - 33, M - 2, M - 1]),
+                      torch.randperm(M, generator=g)[:24]])
+    want_acc = oracle.int8_mm_acc(a[rows].contiguous(), w)
+    assert torch.equal(acc[rows.to(gpu)].cpu(), want_acc)
+    want = oracle.int8_epilogue(want_acc, sa[rows], sb, torch.bfloat16, bias)
+    assert torch.equal(_bits16(out[rows.to(gpu)]), _bits16(want))
+
+
 def test_reference_test_distribution(gpu, oracle):
     """sgl-kernel/tests/test_int8_gemm.py:20-31: int8 from randn*5, scales randn (negative values included)."""
     from sglang_amd.sgl_kernel import int8_scaled_mm
