@@ -44,6 +44,15 @@ __device__ __attribute__((aligned(16))) const uint32_t d_zero16[4] = {0, 0, 0, 0
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
+typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
+
+// Per-lane LDS base of one stage (typed as an LDS pointer so that tile offsets fold into ds_read immediates).
+__device__ __forceinline__ lds_cptr lds_base(const uint8_t* stage, uint32_t off) {
+  return (lds_cptr)stage + off;
+}
+__device__ __forceinline__ u32x4 lds16(lds_cptr p, int imm) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(p + imm);
+}
 
 struct Frag {
   u32x4 lo, hi;
@@ -69,7 +78,10 @@ struct DmaState {
 template <bool KFULL>
 __device__ __forceinline__ void issue_one(const DmaState& s, int i, uint8_t* stage, float* scale, int kb) {
   if (i < D_LOADS) {
-    const uint8_t* base = (i < D_LOADS / 2 ? s.a_base : s.b_base) + (int64_t)kb * KSTEP;
+    // scalar base + 32-bit lane offset (saddr form).  The asm keeps the compiler from folding the lane offset into
+    // per-lane 64-bit pointers, which costs 16 registers and a 64-bit vector add per load.
+    const uint8_t* base = (i < D_LOADS / 2 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;
+    asm volatile("" : "+s"(base));
     const uint8_t* src = base + s.goff[i];
     if constexpr (!KFULL) {
       if (kb * KSTEP + s.chunk_byte >= s.K) src = reinterpret_cast<const uint8_t*>(d_zero16);
@@ -86,27 +98,24 @@ __device__ __forceinline__ void issue_block(const DmaState& s, uint8_t* stage, f
   for (int i = 0; i <= D_LOADS; ++i) issue_one<KFULL>(s, i, stage, scale, kb);
 }
 
-// One K block out of `cur` / `sc_cur`; meanwhile the direct-to-LDS loads of block kb_next go out, one every third step,
-// into `nxt` / `sc_nxt` (issuing them all at once would hold the wave at the front of the iteration until the address
-// unit has taken them, since a wave issues in order).
+// One K block out of `cur` / `sc_cur`; meanwhile the direct-to-LDS loads of block kb_next go out into `nxt` / `sc_nxt`,
+// one per step over the first nine steps: early, so that they have the rest of the iteration to land before the barrier,
+// but not in one burst, which would hold the wave until the address unit has taken them (a wave issues in order).
 template <bool KFULL>
 __device__ __forceinline__ void k_block(const DmaState& s, const uint8_t* cur, const float* sc_cur, float sbv,
                                         float (&acc)[D_NT][D_MT][4], uint8_t* nxt, float* sc_nxt, int kb_next) {
   Frag w[D_NT], tokb[2];
   float scb[2];
-#pragma unroll
-  for (int f = 0; f < D_NT; ++f) {
-    w[f].lo = *reinterpret_cast<const u32x4*>(cur + s.ch_off[0] + f * 2048);
-    w[f].hi = *reinterpret_cast<const u32x4*>(cur + s.ch_off[1] + f * 2048);
-  }
-  tokb[0].lo = *reinterpret_cast<const u32x4*>(cur + s.tok_off[0]);
-  tokb[0].hi = *reinterpret_cast<const u32x4*>(cur + s.tok_off[1]);
+  const lds_cptr ch0 = lds_base(cur, s.ch_off[0]), ch1 = lds_base(cur, s.ch_off[1]);
+  const lds_cptr tk0 = lds_base(cur, s.tok_off[0]), tk1 = lds_base(cur, s.tok_off[1]);
+  // only what the first MFMA needs is read up front (all eight waves hit the LDS at once after the barrier); the
+  // other weight fragments follow in steps 0..2
+  w[0].lo = lds16(ch0, 0);
+  w[0].hi = lds16(ch1, 0);
+  tokb[0].lo = lds16(tk0, 0);
+  tokb[0].hi = lds16(tk1, 0);
   const float* scp = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(sc_cur) + s.sc_off);
-#ifdef MI355_ABLATE_SCALE
-  scb[0] = sbv;
-#else
   scb[0] = scp[0] * sbv;
-#endif
   __builtin_amdgcn_sched_barrier(0);
 
   v4f part[2];
@@ -121,20 +130,20 @@ __device__ __forceinline__ void k_block(const DmaState& s, const uint8_t* cur, c
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[(t - 1) & 1][v], scb[pj & 1], acc[pi][pj][v]);
     }
-    if (i == 0 && j + 1 < D_MT) {  // next token tile
-      tokb[(j + 1) & 1].lo = *reinterpret_cast<const u32x4*>(cur + s.tok_off[0] + (j + 1) * 2048);
-      tokb[(j + 1) & 1].hi = *reinterpret_cast<const u32x4*>(cur + s.tok_off[1] + (j + 1) * 2048);
+    if (t + 1 < D_NT) {  // weight fragment of the next step (first pass over the channel tiles only)
+      w[t + 1].lo = lds16(ch0, (t + 1) * 2048);
+      w[t + 1].hi = lds16(ch1, (t + 1) * 2048);
     }
-#ifdef MI355_ABLATE_SCALE
-    if (i == 1 && j + 1 < D_MT) scb[(j + 1) & 1] = sbv;
-#else
+    if (i == 0 && j + 1 < D_MT) {  // next token tile
+      tokb[(j + 1) & 1].lo = lds16(tk0, (j + 1) * 2048);
+      tokb[(j + 1) & 1].hi = lds16(tk1, (j + 1) * 2048);
+    }
     if (i == 1 && j + 1 < D_MT) scb[(j + 1) & 1] = scp[(j + 1) * 16] * sbv;
+#ifndef MI355_DMA_SPACING
+#define MI355_DMA_SPACING 1
 #endif
-#ifdef MI355_ABLATE_SAMEBLOCK
-    if (t % 3 == 2 && t / 3 <= D_LOADS) issue_one<KFULL>(s, t / 3, nxt, sc_nxt, 0);
-#else
-    if (t % 3 == 2 && t / 3 <= D_LOADS) issue_one<KFULL>(s, t / 3, nxt, sc_nxt, kb_next);
-#endif
+    if (t % MI355_DMA_SPACING == MI355_DMA_SPACING - 1 && t / MI355_DMA_SPACING <= D_LOADS)
+      issue_one<KFULL>(s, t / MI355_DMA_SPACING, nxt, sc_nxt, kb_next);
     __builtin_amdgcn_sched_barrier(0);
   }
   {
@@ -148,7 +157,8 @@ __device__ __forceinline__ void k_block(const DmaState& s, const uint8_t* cur, c
 template <bool KFULL>
 __global__ __launch_bounds__(D_THREADS) void fp8_gemm_dma_kernel(const GemmParams p) {
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS destinations and scale pointers stay scalar
   const int wave_m = wave >> 2, wave_n = wave & 3;
   const int l16 = lane & 15, q = lane >> 4;
 
