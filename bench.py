@@ -11,6 +11,7 @@ bandwidth-bound steps stream from HBM rather than from the 256 MB Infinity Cache
   fp8_gemm   (headline, default) blockwise-FP8 GEMM, M=4096, DeepSeek-V3 gate_up K=7168 -> N=36864
   quant      per-token-group FP8 quantization, M=16384 K=7168 g=128, row-major fp32 scales
   quant_ue8m0  the same with column-major packed UE8M0 scales
+  copy       a plain 256 MiB device copy (calibration of the HBM traffic counters)
   all        (what the default run does) headline as `value`, every other configuration the
              baseline names under "also": both quantizer variants, the M=4096 MLP/MLA shapes,
              the decode shapes M in {1,8,32,128}, the single linear, and the INT8 GEMM shapes.
@@ -247,6 +248,37 @@ def bench_int8_gemm(name, M, K, N, steps, warmup):
     }
 
 
+def bench_copy(steps, warmup):
+    """Plain device-to-device copy of a known size (256 MiB read + 256 MiB written per launch): the calibration
+    workload for the FETCH_SIZE / WRITE_SIZE counters behind `roofline.traffic`."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    n = 256 << 20
+    srcs = [torch.randint(0, 255, (n,), dtype=torch.uint8, device=dev) for _ in range(3)]
+    dsts = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in range(3)]
+    wall, ms = _time_launches(lambda i: dsts[i].copy_(srcs[i]), 3, steps, warmup)
+    st = _stats(ms)
+    gbs = 2 * n / (st["avg"] * 1e-3) / 1e9
+    return {
+        "workload": f"copy {n} bytes device to device (torch copy kernel; {n} read + {n} written)",
+        "value": 2 * n / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "u8",
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes_per_launch": 2 * n},
+    }
+
+
+def _measured_traffic():
+    """HBM bytes per launch measured with rocprofv3 counters (profiles/traffic.json), keyed by workload name."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get("bytes_per_launch", {})
+    except (OSError, ValueError):
+        return {}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -275,6 +307,8 @@ def main():
     also = []
     if args.workload in ("quant", "quant_ue8m0"):
         rec = bench_quant(S, W, args.workload == "quant_ue8m0", cpu)
+    elif args.workload == "copy":
+        rec = bench_copy(S, W)
     else:
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 4096, K, N, S, W, cpu)
@@ -292,6 +326,12 @@ def main():
             for M in (1, 256, 4096):
                 for nm, (K, N) in LLAMA3_8B.items():
                     also.append(bench_int8_gemm(nm, M, K, N, S, W))
+
+    traffic = _measured_traffic()
+    for r in [rec] + also:
+        key = r["workload"].split(" M=")[0].replace(" ", "_")
+        if key in traffic:
+            r["roofline"]["traffic"] = traffic[key]
 
     line = {
         "metric": METRIC, "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": S, "warmup": W,

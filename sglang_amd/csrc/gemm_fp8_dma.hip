@@ -139,11 +139,7 @@ __device__ __forceinline__ void k_block(const DmaState& s, const uint8_t* cur, c
       tokb[(j + 1) & 1].hi = lds16(tk1, (j + 1) * 2048);
     }
     if (i == 1 && j + 1 < D_MT) scb[(j + 1) & 1] = scp[(j + 1) * 16] * sbv;
-#ifndef MI355_DMA_SPACING
-#define MI355_DMA_SPACING 1
-#endif
-    if (t % MI355_DMA_SPACING == MI355_DMA_SPACING - 1 && t / MI355_DMA_SPACING <= D_LOADS)
-      issue_one<KFULL>(s, t / MI355_DMA_SPACING, nxt, sc_nxt, kb_next);
+    if (t <= D_LOADS) issue_one<KFULL>(s, t, nxt, sc_nxt, kb_next);
     __builtin_amdgcn_sched_barrier(0);
   }
   {

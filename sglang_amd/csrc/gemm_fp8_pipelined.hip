@@ -104,23 +104,16 @@ __device__ __forceinline__ void k_block(PipeState& s, uint8_t* smem, float (&acc
     __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first; everything below runs in its shadow
     if (t > 0) {
       const int pj = (t - 1) >> 2, pi = (t - 1) & 3;
-#ifdef MI355_ABLATE_FMA
-      if (pj == 0)
-#endif
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[(t - 1) & 1][v], scb[pj & 1], acc[pi][pj][v]);
     }
     // ---- memory slots of this step
     if (t < P_LOADS) {  // register set SET, filled two iterations ago -> stage st_write
-#ifndef MI355_ABLATE_LDSWRITE
       *reinterpret_cast<u32x4*>(wr + s.wr_off + t * 4096) = s.stage_regs[SET][t];
       if (t == 0) sc_wr[threadIdx.x] = s.stage_sa[SET] * s.stage_sb[SET];
-#endif
     } else if (t < 2 * P_LOADS) {  // refill it with the block four ahead
-#ifndef MI355_ABLATE_GLOAD
       load_one<KFULL, SET>(s, t - P_LOADS, kb_load);
       if (t == P_LOADS) load_scale<SET>(s, kb_load);
-#endif
     }
     if (i == 0 && j + 1 < P_MT) {  // next token tile of this block
       tokb[(j + 1) & 1].lo = *reinterpret_cast<const u32x4*>(cur + s.tok_off[0] + (j + 1) * 2048);

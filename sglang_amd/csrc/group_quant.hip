@@ -218,11 +218,7 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
 template <typename T, int LPG, int ITERS, int MODE, bool UE8M0, bool FP8_OUT>
 int launch(const QuantParams& p, hipStream_t stream) {
   // Fewer groups per thread when each group already spans several vectors per lane.
-#ifdef MI355_QUANT_UNROLL
-  constexpr int UNROLL = MI355_QUANT_UNROLL;
-#else
   constexpr int UNROLL = (ITERS >= 4) ? 1 : (ITERS == 2 ? 2 : 4);
-#endif
   constexpr int GROUPS_PER_BLOCK = (256 / LPG) * UNROLL;
   const uint32_t blocks = (p.num_groups + GROUPS_PER_BLOCK - 1) / GROUPS_PER_BLOCK;
   hipLaunchKernelGGL((group_quant_kernel<T, LPG, ITERS, MODE, UE8M0, FP8_OUT, UNROLL>), dim3(blocks), dim3(256), 0,
