@@ -40,19 +40,38 @@ INT8_PEAK_TOPS = 5000.0   # dense int8 MFMA
 METRIC = "blockwise-FP8 GEMM TFLOPS & %MFMA peak; quant GB/s & %HBM peak (1 GPU)"
 
 
-def _time_launches(fn, nbuf, steps, warmup):
+def _time_launches(fn, nbuf, steps, warmup, graph=False):
     """fn(i % nbuf) is launched warmup + steps times on the current stream.  Returns the wall seconds of
-    the timed steps (synchronize on both sides) and the per-launch milliseconds from HIP events."""
+    the timed steps (synchronize on both sides) and the per-launch milliseconds from HIP events.
+
+    graph=True: each fn(i) is captured once into a HIP graph and the graphs are replayed, the way a serving loop runs
+    decode-sized steps; otherwise microsecond kernels would be timed together with the Python launch overhead."""
     import torch
 
+    if graph:
+        stream = torch.cuda.Stream()
+        graphs = []
+        with torch.cuda.stream(stream):
+            for i in range(nbuf):
+                fn(i)  # warm up allocator and lazy initialisation outside capture
+            stream.synchronize()
+            for i in range(nbuf):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    fn(i)
+                graphs.append(g)
+        torch.cuda.synchronize()
+        run = lambda i: graphs[i].replay()
+    else:
+        run = fn
     for i in range(warmup):
-        fn(i % nbuf)
+        run(i % nbuf)
     torch.cuda.synchronize()
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     t0 = time.perf_counter()
     for i in range(steps):
         evs[i][0].record()
-        fn(i % nbuf)
+        run(i % nbuf)
         evs[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -161,8 +180,28 @@ def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
         def step(i):
             return fp8_kernel.w8a8_block_fp8_matmul(x_q, ws[i], x_s, wss[i], [128, 128], torch.bfloat16)
 
+    direct = M <= 256
+    if direct:
+        # decode-sized steps take tens of microseconds: call the C ABI directly with preallocated output and workspace,
+        # so that the host keeps the queue full and the events time kernels rather than Python
+        from sglang_amd import _lib
+
+        L = _lib.lib()
+        wsb = L.mi355_fp8_blockwise_mm_workspace_bytes(M, N, K)
+        wsbuf = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+        outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+        stream = torch.cuda.current_stream().cuda_stream
+        args = [(x_q.data_ptr(), ws[i].data_ptr(), x_s.data_ptr(), wss[i].data_ptr(), outs[i].data_ptr(), _lib.BF16, M, N, K,
+                 x_q.stride(0), ws[i].stride(0), x_s.stride(0), x_s.stride(1), wss[i].stride(0), wss[i].stride(1),
+                 outs[i].stride(0), wsbuf.data_ptr(), wsb, stream) for i in range(nbuf)]
+
+        def step(i):  # noqa: F811
+            _lib.check(L.mi355_fp8_blockwise_mm(*args[i]))
+
     wall, ms = _time_launches(step, nbuf, steps, warmup)
     st = _stats(ms)
+    if direct:  # per-launch events still see a little host jitter; the region average is the kernel time here
+        st["avg"] = wall / steps * 1e3
     flops = gemm_flops(M, N, K)
     nbytes = fp8_gemm_algorithmic_bytes(M, N, K)
     tflops_avg = flops / (st["avg"] * 1e-3) / 1e12
@@ -170,7 +209,8 @@ def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
     # which roof binds: time at peak MFMA rate vs time at peak HBM rate
     mfma_bound = flops / (FP8_PEAK_TFLOPS * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9)
     rec = {
-        "workload": f"fp8_gemm {name} M={M} K={K} N={N} (e4m3fn x e4m3fn, 1x128 / 128x128 fp32 scales, bf16 out)",
+        "workload": f"fp8_gemm {name} M={M} K={K} N={N} (e4m3fn x e4m3fn, 1x128 / 128x128 fp32 scales, bf16 out"
+        + (", direct C-ABI calls)" if direct else ")"),
         "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
         "gbytes_per_s": gbs_avg, "dtype": "fp8(e4m3fn) MFMA, f32 accumulate",
         "roofline": ({"bound": "mfma", "achieved": tflops_avg, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -231,13 +271,31 @@ def bench_int8_gemm(name, M, K, N, steps, warmup):
     def step(i):
         return sgl_kernel.int8_scaled_mm(a, ws[i].t(), sa, sb, torch.bfloat16, bias)
 
+    direct = M <= 256
+    if direct:
+        from sglang_amd import _lib
+
+        L = _lib.lib()
+        wsb = L.mi355_int8_scaled_mm_workspace_bytes(M, N, K)
+        wsbuf = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+        outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+        stream = torch.cuda.current_stream().cuda_stream
+        args = [(a.data_ptr(), ws[i].data_ptr(), sa.data_ptr(), sb.data_ptr(), bias.data_ptr(), outs[i].data_ptr(), _lib.BF16,
+                 M, N, K, a.stride(0), ws[i].stride(0), outs[i].stride(0), wsbuf.data_ptr(), wsb, stream) for i in range(nbuf)]
+
+        def step(i):  # noqa: F811
+            _lib.check(L.mi355_int8_scaled_mm(*args[i]))
+
     wall, ms = _time_launches(step, nbuf, steps, warmup)
     st = _stats(ms)
+    if direct:
+        st["avg"] = wall / steps * 1e3
     ops_, nbytes = gemm_flops(M, N, K), int8_gemm_algorithmic_bytes(M, N, K)
     tops, gbs = ops_ / (st["avg"] * 1e-3) / 1e12, nbytes / (st["avg"] * 1e-3) / 1e9
     mfma_bound = ops_ / (INT8_PEAK_TOPS * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9)
     return {
-        "workload": f"int8_gemm {name} M={M} K={K} N={N} (int8 x int8 -> int32, per-token x per-channel scales, bias, bf16 out)",
+        "workload": f"int8_gemm {name} M={M} K={K} N={N} (int8 x int8 -> int32, per-token x per-channel scales, bias, bf16 out"
+        + (", direct C-ABI calls)" if direct else ")"),
         "value": ops_ / (wall / steps) / 1e12, "unit": "TOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
         "gbytes_per_s": gbs, "dtype": "int8 MFMA, int32 accumulate",
         "roofline": ({"bound": "mfma", "achieved": tops, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",

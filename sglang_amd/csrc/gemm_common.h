@@ -101,6 +101,7 @@ int launch_int8_dma(GemmParams& p, hipStream_t stream, const char* what);
 // Small-M blockwise FP8 GEMM streaming the weight through wave-private LDS, no barriers; gemm_fp8_decode.hip.
 // decode_splits() is the split count it wants for a shape; the caller sets p.splits, p.kb_per_split and p.ws.
 int decode_splits(int64_t M, int64_t N, int64_t K);
+bool decode_supported(int64_t M, int64_t N, int64_t K);
 int launch_fp8_decode(GemmParams& p, hipStream_t stream, const char* what);
 
 }  // namespace mi355

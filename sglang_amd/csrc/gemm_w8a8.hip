@@ -330,15 +330,13 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
   return pl;
 }
 
-constexpr int64_t DECODE_MAX_M = 16;  // beyond one token tile the LDS-tiled kernel amortizes the token fetch better
-
 // Upper bound over the kernels a shape may be routed to (the choice also depends on pointer alignment, which is not
 // known here).
 size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const Plan pl = make_plan(M, N, K);
   size_t need = pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
-  if (is_fp8 && M <= DECODE_MAX_M) {
+  if (is_fp8 && decode_supported(M, N, K)) {
     const int ds = decode_splits(M, N, K);
     const size_t dneed = ds > 1 ? (size_t)ds * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
@@ -390,7 +388,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
   const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
                        ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
   if constexpr (IS_FP8) {
-    if (p.M <= DECODE_MAX_M && aligned) {  // weight streaming without LDS
+    if (decode_supported(p.M, p.N, p.K) && aligned && (int64_t)p.N * p.ldb < (1ll << 32)) {  // barrier-free weight streaming
       p.splits = decode_splits(p.M, p.N, p.K);
       p.kb_per_split = (p.kb_total + p.splits - 1) / p.splits;
       if (p.splits > 1) {
