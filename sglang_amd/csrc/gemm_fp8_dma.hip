@@ -44,6 +44,8 @@ __device__ __attribute__((aligned(16))) const uint32_t d_zero16[4] = {0, 0, 0, 0
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
+// read-only scalars fetched through the constant address space become s_load (own counter, no vmcnt traffic)
+typedef const __attribute__((address_space(4))) float* cfloat_ptr;
 typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
 
 // Per-lane LDS base of one stage (typed as an LDS pointer so that tile offsets fold into ds_read immediates).
@@ -67,7 +69,7 @@ struct DmaState {
   uint32_t goff[D_LOADS];  // byte offset of this lane's chunk from the matrix base (rows clamped); loads 0..3 tokens, 4..7 channels
   int chunk_byte;          // 16 * logical chunk this lane fetches
   const float* sa_ptr;     // &sa[m, 0] for the token whose scale this thread fetches (waves 0..3)
-  const float* sb_ptr;     // &sb[nb, 0] of this wave's 128-channel block
+  cfloat_ptr sb_ptr;       // &sb[nb, 0] of this wave's 128-channel block
   int64_t sa_sk, sb_sk;
   int K;
   int wave;
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(D_THREADS) void fp8_gemm_dma_kernel(const GemmParam
   s.sa_ptr = p.sa + (int64_t)min(m0 + (tid & (D_BM - 1)), p.M - 1) * p.sa_sm;
   s.sa_sk = p.sa_sk;
   // wave-uniform by construction; readfirstlane tells the compiler so, which turns the per-block fetch into a scalar load
-  s.sb_ptr = p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * D_WN, p.N - 1) / 128) * p.sb_sn;
+  s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * D_WN, p.N - 1) / 128) * p.sb_sn);
   s.sb_sk = p.sb_sk;
   {
     const int trow = wave_m * D_WM + l16, crow = D_BM + wave_n * D_WN + l16;
