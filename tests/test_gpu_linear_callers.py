@@ -1,0 +1,51 @@
+"""The linear-method callers (quantize -> GEMM -> bias -> reshape) against the same pipeline run on the CPU oracle."""
+import pytest
+import torch
+
+from sglang_amd.workloads import make_activation, make_fp8_weight, make_int8_weight
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape,N,K", [((2, 5), 384, 512), ((16,), 2048, 7168), ((3, 7), 576, 1024), ((300,), 1088, 384)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
+    from sglang_amd.fp8_utils import dispatch_w8a8_block_fp8_linear, triton_w8a8_block_fp8_linear
+
+    M = 1
+    for d in shape:
+        M *= d
+    x = make_activation(M, K, seed=N + K).view(*shape, K)
+    w_q, w_s = make_fp8_weight(N, K)
+    g = torch.Generator().manual_seed(1)
+    bias = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
+    for fn, mode in ((dispatch_w8a8_block_fp8_linear(), "div" if N % 128 == 0 else "rcp"), (triton_w8a8_block_fp8_linear, "rcp")):
+        out = fn(x.to(gpu), w_q.to(gpu), [128, 128], w_s.to(gpu), None, bias.to(gpu) if with_bias else None)
+        assert out.dtype == torch.bfloat16 and tuple(out.shape) == (*shape, N)
+        xq, xs = oracle.group_quant(x.view(M, K), 128, mode=mode)
+        ref, mag = oracle.fp8_blockwise_mm(xq, w_q, xs, w_s, torch.float32, want_abs=True)
+        want = ref.to(torch.bfloat16)
+        if with_bias:
+            want = want + bias  # bf16 += bf16, as the reference does after the GEMM
+        err = (out.float().cpu().view(M, N) - want.float()).abs()
+        # the GEMM result is rounded to bf16 before the bias is added, so its rounding is relative to |ref|, not to the sum
+        tol = 1e-2 * want.float().abs() + 1e-4 * mag + (2.0 ** -7 * (ref.abs() + bias.float().abs()[None, :]) if with_bias else 0)
+        assert bool((err <= tol).all()), float((err - tol).max())
+
+
+@pytest.mark.parametrize("shape,N,K", [((4, 3), 6144, 4096), ((1,), 4096, 14336), ((300,), 264, 512)])
+def test_int8_linear(gpu, oracle, shape, N, K):
+    from sglang_amd.w8a8_int8 import apply_w8a8_int8_linear
+
+    M = 1
+    for d in shape:
+        M *= d
+    x = make_activation(M, K, seed=N, outlier_frac=0.0).view(*shape, K)
+    w_q, w_s = make_int8_weight(N, K)
+    g = torch.Generator().manual_seed(2)
+    bias = torch.randn(N, generator=g).to(torch.bfloat16)
+    out = apply_w8a8_int8_linear(x.to(gpu), w_q.to(gpu).t(), w_s.view(N, 1).to(gpu), bias.to(gpu))
+    assert tuple(out.shape) == (*shape, N) and out.dtype == torch.bfloat16
+    xq, xs = oracle.per_token_quant_int8(x.view(M, K))
+    want = oracle.int8_scaled_mm(xq, w_q, xs, w_s, torch.bfloat16, bias)
+    assert torch.equal(out.cpu().view(M, N).view(torch.int16), want.view(torch.int16))
