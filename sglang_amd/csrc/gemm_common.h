@@ -103,5 +103,6 @@ int launch_int8_dma(GemmParams& p, hipStream_t stream, const char* what);
 int decode_splits(int64_t M, int64_t N, int64_t K);
 bool decode_supported(int64_t M, int64_t N, int64_t K);
 int launch_fp8_decode(GemmParams& p, hipStream_t stream, const char* what);
+int launch_int8_decode(GemmParams& p, hipStream_t stream, const char* what);  // same kernel, int8 MFMA, int32 partials
 
 }  // namespace mi355

@@ -1,4 +1,4 @@
-// Decode (M <= 16) blockwise-scaled FP8 GEMM for gfx950: barrier-free weight streaming.
+// Decode (M <= 16) GEMMs for gfx950 - blockwise-scaled FP8 and per-token x per-channel INT8: barrier-free weight streaming.
 //
 // With at most 16 tokens every weight byte is used by exactly one MFMA and never again, so the kernel is bound by how
 // fast the weight leaves HBM.  Measured on MI355X, a wave instruction that fetches 8 rows x 128 contiguous bytes streams
@@ -20,7 +20,9 @@
 // kernels (chunks q and q + 4 per lane quarter: full-rate LDS reads).
 //
 // Split along K: every K range writes a partial tile to the caller's workspace and splitk_reduce_kernel adds them in a
-// fixed order.  Requires K % 128 == 0, N % 128 == 0 and 16-byte aligned rows; other shapes take the generic kernel.
+// fixed order (for INT8 the partials are int32 and the reduce kernel applies the epilogue).  INT8 uses two
+// v_mfma_i32_16x16x64_i8 per K block (chunk q of both operands, then chunk q + 4) and has no scales in the loop.
+// Requires K % 128 == 0, N % 128 == 0 and 16-byte aligned rows; other shapes take the generic kernel.
 #include "gemm_common.h"
 
 namespace mi355 {
@@ -39,6 +41,10 @@ __shared__ __attribute__((aligned(1024))) uint8_t r_stage1[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_stage2[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_stage3[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_tok[KB_PER * TOK_BLOCK];
+
+// 16 zero bytes in global memory: the source of token chunks that lie past the end of K (short last range), so that
+// whatever weight block is refetched there multiplies zeros.  Not const: it must share the operands' address space.
+__device__ __attribute__((aligned(16))) uint32_t r_zero16[4] = {0, 0, 0, 0};
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -97,7 +103,8 @@ __device__ __forceinline__ void wait_ring() {
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-__device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* stage, int d, float scale, float (&acc)[NT][4]) {
+template <bool IS_FP8, typename AccT>
+__device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* stage, int d, float scale, AccT (&acc)[NT][4]) {
   const uint8_t* sl = stage + s.wave * SLICE;
   Frag t;
   t.lo = *reinterpret_cast<const u32x4*>(r_tok + d * TOK_BLOCK + s.tk_off[0]);
@@ -107,16 +114,27 @@ __device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* sta
     Frag w;
     w.lo = *reinterpret_cast<const u32x4*>(sl + s.rd_off[i][0]);
     w.hi = *reinterpret_cast<const u32x4*>(sl + s.rd_off[i][1]);
-    const v4f part =
-        __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w), as_v8i(t), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+    if constexpr (IS_FP8) {
+      const v4f part =
+          __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w), as_v8i(t), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
 #pragma unroll
-    for (int v = 0; v < 4; ++v) acc[i][v] = fmaf(part[v], scale, acc[i][v]);
+      for (int v = 0; v < 4; ++v) acc[i][v] = fmaf(part[v], scale, acc[i][v]);
+    } else {
+      v4i c = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+      c = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)w.lo.x, (int)w.lo.y, (int)w.lo.z, (int)w.lo.w},
+                                                v4i{(int)t.lo.x, (int)t.lo.y, (int)t.lo.z, (int)t.lo.w}, c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)w.hi.x, (int)w.hi.y, (int)w.hi.z, (int)w.hi.w},
+                                                v4i{(int)t.hi.x, (int)t.hi.y, (int)t.hi.z, (int)t.hi.w}, c, 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][v] = c[v];
+    }
   }
 }
 
 // SPLIT: raw partial sums to the workspace (more than one K range).
-template <bool SPLIT>
-__global__ __launch_bounds__(64 * WAVES) void fp8_decode_kernel(const GemmParams p, int groups_per_wg, int wg_per_split) {
+template <bool IS_FP8, bool SPLIT>
+__global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, int groups_per_wg, int wg_per_split) {
+  using AccT = typename std::conditional<IS_FP8, float, int>::type;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l16 = lane & 15, q = lane >> 4;
@@ -159,30 +177,38 @@ __global__ __launch_bounds__(64 * WAVES) void fp8_decode_kernel(const GemmParams
     const int inst = wave * (2 * KB_PER / WAVES) + e;
     const int d = inst >> 1, half = inst & 1;
     const int m = min(half * 8 + lrow, p.M - 1);           // rows past M repeat the last token, never stored
-    const int kb = min(kb_begin + d, p.kb_total - 1);      // blocks past K repeat the last block, scaled by zero
-    const uint8_t* src = p.a + (int64_t)m * p.lda + (int64_t)kb * KSTEP + logical * 16;
+    const uint8_t* src = p.a + (int64_t)m * p.lda + (int64_t)(kb_begin + d) * KSTEP + logical * 16;
+    if (kb_begin + d >= p.kb_total) src = reinterpret_cast<const uint8_t*>(r_zero16);  // blocks past K: zeros
     __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(r_tok + d * TOK_BLOCK + half * 1024), 16, 0, 0);
   }
-  // token scales of the range, zero for blocks past the end of K (their products then add nothing)
+  // FP8: token scales of the range (blocks past the end of K multiply zero tokens; their scale is set to zero too)
   float sa_r[KB_PER];
-  {
+  if constexpr (IS_FP8) {
     const float* sa_row = p.sa + (int64_t)min(l16, p.M - 1) * p.sa_sm;
 #pragma unroll
     for (int d = 0; d < KB_PER; ++d) {
       const float v = sa_row[(int64_t)min(kb_begin + d, p.kb_total - 1) * p.sa_sk];
       sa_r[d] = d < kb_valid ? v : 0.f;
     }
+  } else {
+#pragma unroll
+    for (int d = 0; d < KB_PER; ++d) sa_r[d] = 0.f;
   }
   __syncthreads();  // the only barrier: tokens are in LDS
 
   const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-  // weight-block scales: one per K block and 128-channel group; fetched one group ahead so that using them never
+  // FP8 weight-block scales: one per K block and 128-channel group; fetched one group ahead so that using them never
   // has to wait for loads younger than the ring's
   float sb_cur[KB_PER], sb_nxt[KB_PER];
   auto load_sb = [&](int g, float (&dst)[KB_PER]) {
-    const float* sb_row = p.sb + (int64_t)(g_first + min(g, groups - 1)) * p.sb_sn + (int64_t)kb_begin * p.sb_sk;
+    if constexpr (IS_FP8) {
+      const float* sb_row = p.sb + (int64_t)(g_first + min(g, groups - 1)) * p.sb_sn + (int64_t)kb_begin * p.sb_sk;
 #pragma unroll
-    for (int d = 0; d < KB_PER; ++d) dst[d] = sb_row[(int64_t)min(d, kb_valid - 1) * p.sb_sk];
+      for (int d = 0; d < KB_PER; ++d) dst[d] = sb_row[(int64_t)min(d, kb_valid - 1) * p.sb_sk];
+    } else {
+#pragma unroll
+      for (int d = 0; d < KB_PER; ++d) dst[d] = 0.f;
+    }
   };
   load_sb(0, sb_cur);
   for (int g = 0; g < groups; ++g) {
@@ -193,11 +219,11 @@ __global__ __launch_bounds__(64 * WAVES) void fp8_decode_kernel(const GemmParams
     for (int d = 0; d < KB_PER; ++d) sc[d] = sa_r[d] * sb_cur[d];
 #pragma unroll
     for (int d = 0; d < KB_PER; ++d) sb_cur[d] = sb_nxt[d];
-    float acc[NT][4];
+    AccT acc[NT][4];
 #pragma unroll
     for (int i = 0; i < NT; ++i)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[i][v] = 0.f;
+      for (int v = 0; v < 4; ++v) acc[i][v] = 0;
 
     const int f0 = g * KB_PER;
 #pragma unroll
@@ -206,19 +232,19 @@ __global__ __launch_bounds__(64 * WAVES) void fp8_decode_kernel(const GemmParams
       // that is due (the two requested after it may still be in flight), multiply it
       issue_weights<true>(s, r_stage3, f0 + d + 3);
       wait_ring<2>();
-      consume(s, r_stage0, d + 0, sc[d + 0], acc);
+      consume<IS_FP8>(s, r_stage0, d + 0, sc[d + 0], acc);
       __builtin_amdgcn_sched_barrier(0);
       issue_weights<true>(s, r_stage0, f0 + d + 4);
       wait_ring<2>();
-      consume(s, r_stage1, d + 1, sc[d + 1], acc);
+      consume<IS_FP8>(s, r_stage1, d + 1, sc[d + 1], acc);
       __builtin_amdgcn_sched_barrier(0);
       issue_weights<true>(s, r_stage1, f0 + d + 5);
       wait_ring<2>();
-      consume(s, r_stage2, d + 2, sc[d + 2], acc);
+      consume<IS_FP8>(s, r_stage2, d + 2, sc[d + 2], acc);
       __builtin_amdgcn_sched_barrier(0);
       issue_weights<true>(s, r_stage2, f0 + d + 6);
       wait_ring<2>();
-      consume(s, r_stage3, d + 3, sc[d + 3], acc);
+      consume<IS_FP8>(s, r_stage3, d + 3, sc[d + 3], acc);
       __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -228,11 +254,28 @@ __global__ __launch_bounds__(64 * WAVES) void fp8_decode_kernel(const GemmParams
       for (int i = 0; i < NT; ++i) {
         const int n = nb * GROUP_N + wave * WAVE_N + i * 16 + 4 * q;
         if constexpr (SPLIT) {
-          float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)split * p.M + l16) * p.N + n;
+          AccT* wsp = reinterpret_cast<AccT*>(p.ws) + ((int64_t)split * p.M + l16) * p.N + n;
 #pragma unroll
           for (int v = 0; v < 4; ++v) wsp[v] = acc[i][v];
-        } else {
+        } else if constexpr (IS_FP8) {
           store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, acc[i], 4, vec_ok);
+        } else if (p.out_dtype == MI355_I32) {
+          int* o = reinterpret_cast<int*>(p.out) + (int64_t)l16 * p.ldo + n;
+#pragma unroll
+          for (int v = 0; v < 4; ++v) o[v] = acc[i][v];
+        } else {
+          const float sa_m = p.sa[l16];
+          float r[4];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            float t = __fmul_rn((float)acc[i][v], __fmul_rn(p.sb[n + v], sa_m));
+            if (p.bias) {
+              const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
+              t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+            }
+            r[v] = t;
+          }
+          store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r, 4, vec_ok);
         }
       }
     }
@@ -251,7 +294,8 @@ int decode_splits(int64_t M, int64_t N, int64_t K) {
 bool decode_supported(int64_t M, int64_t N, int64_t K) { return M >= 1 && M <= 16 && K % KSTEP == 0 && N % GROUP_N == 0; }
 
 // Also needs 16-byte aligned rows and row offsets below 4 GiB.  The caller sets p.splits (= decode_splits) and p.ws.
-int launch_fp8_decode(GemmParams& p, hipStream_t stream, const char* what) {
+template <bool IS_FP8>
+static int launch_decode(GemmParams& p, hipStream_t stream, const char* what) {
   const int groups_n = p.N / GROUP_N;
   // about two workgroups per CU; each walks `gpw` consecutive channel groups with the same tokens
   int gpw = (int)(((int64_t)groups_n * p.splits + 511) / 512);
@@ -261,10 +305,13 @@ int launch_fp8_decode(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_n = groups_n;
   const dim3 grid((unsigned)(wg_per_split * p.splits));
   if (p.splits > 1)
-    hipLaunchKernelGGL(fp8_decode_kernel<true>, grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+    hipLaunchKernelGGL((decode_kernel<IS_FP8, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
   else
-    hipLaunchKernelGGL(fp8_decode_kernel<false>, grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+    hipLaunchKernelGGL((decode_kernel<IS_FP8, false>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
   return check_launch(what);
 }
+
+int launch_fp8_decode(GemmParams& p, hipStream_t stream, const char* what) { return launch_decode<true>(p, stream, what); }
+int launch_int8_decode(GemmParams& p, hipStream_t stream, const char* what) { return launch_decode<false>(p, stream, what); }
 
 }  // namespace mi355

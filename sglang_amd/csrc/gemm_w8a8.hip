@@ -336,7 +336,7 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const Plan pl = make_plan(M, N, K);
   size_t need = pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
-  if (is_fp8 && decode_supported(M, N, K)) {
+  if (decode_supported(M, N, K)) {
     const int ds = decode_splits(M, N, K);
     const size_t dneed = ds > 1 ? (size_t)ds * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
@@ -387,24 +387,22 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
   p.kb_total = (p.K + KSTEP - 1) / KSTEP;
   const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
                        ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
-  if constexpr (IS_FP8) {
-    if (decode_supported(p.M, p.N, p.K) && aligned && (int64_t)p.N * p.ldb < (1ll << 32)) {  // barrier-free weight streaming
-      p.splits = decode_splits(p.M, p.N, p.K);
-      p.kb_per_split = (p.kb_total + p.splits - 1) / p.splits;
-      if (p.splits > 1) {
-        const size_t need = (size_t)p.splits * (size_t)p.M * (size_t)p.N * 4u;
-        MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
-                      "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
-        MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
-                      "%s: workspace must be 16-byte aligned", what);
-        p.ws = workspace;
-      }
-      int rc = launch_fp8_decode(p, stream, what);
-      if (rc != MI355_OK || p.splits == 1) return rc;
-      const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
-      hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
-      return check_launch(what);
+  if (decode_supported(p.M, p.N, p.K) && aligned && (int64_t)p.N * p.ldb < (1ll << 32)) {  // barrier-free weight streaming
+    p.splits = decode_splits(p.M, p.N, p.K);
+    p.kb_per_split = (p.kb_total + p.splits - 1) / p.splits;
+    if (p.splits > 1) {
+      const size_t need = (size_t)p.splits * (size_t)p.M * (size_t)p.N * 4u;
+      MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
+                    "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
+      MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
+                    "%s: workspace must be 16-byte aligned", what);
+      p.ws = workspace;
     }
+    int rc = IS_FP8 ? launch_fp8_decode(p, stream, what) : launch_int8_decode(p, stream, what);
+    if (rc != MI355_OK || p.splits == 1) return rc;
+    const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
+    hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
+    return check_launch(what);
   }
   const Plan pl = make_plan(p.M, p.N, p.K);
   p.splits = pl.splits;
