@@ -94,6 +94,16 @@ int launch_fp8_pipelined(GemmParams& p, hipStream_t stream, const char* what);
 int launch_fp8_dma(GemmParams& p, hipStream_t stream, const char* what);
 
 
+// Mid-M blockwise FP8 GEMM (64/128 x 256 tile, 8 waves, three LDS stages, hand-issued direct-to-LDS loads);
+// gemm_fp8_dma3.hip.  Needs 16-byte aligned rows, K % 128 == 0, row offsets below 4 GiB.  dma3_plan() gives the split it
+// wants; the caller sets p.splits, p.kb_per_split and p.ws accordingly.
+struct Dma3Plan {
+  int bm, splits, kb_per_split;
+  double efficiency;  // modelled fraction of the streaming time that is useful (balance, partial sums, pipeline fill)
+};
+Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K);
+int launch_fp8_dma3(GemmParams& p, hipStream_t stream, const char* what);
+
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, 32x32x32 MFMA); gemm_int8_dma.hip.
 // Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
 int launch_int8_dma(GemmParams& p, hipStream_t stream, const char* what);

@@ -248,6 +248,7 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
       __builtin_amdgcn_sched_barrier(0);
     }
 
+    if (g == groups - 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no ring refetch may outlive the workgroup's LDS
     // ---- lane holds channels 16 i + 4q .. +3 of this wave's 32, for token l16
     if (l16 < p.M) {
 #pragma unroll

@@ -224,6 +224,9 @@ __global__ __launch_bounds__(D_THREADS) void fp8_gemm_dma_kernel(const GemmParam
   }
   if (kb < nkb) k_block<KFULL>(s, d_stage0, d_scale0, sb_cur, acc, d_stage1, d_scale1, kb);
 
+  // the last iterations refetch a block into a stage nobody reads: those writes must not outlive this workgroup's LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
   // ---- epilogue: lane holds channels n .. n+3 of token m
   const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
 #pragma unroll

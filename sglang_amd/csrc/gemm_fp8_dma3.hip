@@ -1,0 +1,292 @@
+// Mid-M blockwise-scaled FP8 GEMM for gfx950: (64 or 128) x 256 macro tile, 8 waves (two per SIMD), THREE LDS stages.
+//
+// For 16 < M <= 1024 a linear layer is between weight streaming and MFMA-bound.  The tile is short in the token dimension
+// (64 or 128 tokens) and wide in channels (256), so a stage of LDS is (BM + 256) x 128 B <= 48 KB and three stages fit in
+// the CU's 160 KB.  With three stages the direct-to-LDS loads of K block k+2 are issued while block k is multiplied and
+// only have to land before block k+2 is multiplied, two barriers later: the wait that precedes the barrier at the end of
+// iteration k covers block k+1 only.  The compiler cannot express that (its wait before a barrier covers every load it
+// knows about), so inside the loop the loads, the wait and the barrier are written as instructions:
+//   * every iteration issues exactly LOADS + 1 loads per wave (tile rows plus the token scales), always, even past the
+//     end of K (they refetch the last block into a stage nobody reads), so "block k+1 has landed" is the constant
+//     s_waitcnt vmcnt(LOADS + 1): everything but the youngest LOADS + 1 loads;
+//   * nothing else in the loop counts in vmcnt (weight-block scales come by scalar loads);
+//   * the barrier is a bare s_barrier: LDS written by the loads is complete when vmcnt says so, and a stage is
+//     overwritten only after the barrier that follows its last read.
+// Operand roles, swizzle, chunk mapping, promotion FMA and the {MFMA of tile t, FMAs of tile t-1} step are those of
+// gemm_fp8_dma.hip.  Optional split along K (partials to the workspace, ordered reduce afterwards).
+// Requires K % 128 == 0, 16-byte aligned rows, row offsets below 4 GiB.
+#include "gemm_common.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int T_THREADS = 512;
+constexpr int T_BN = 256, T_WN = 64, T_NT = T_WN / 16;
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
+typedef const __attribute__((address_space(4))) float* cfloat_ptr;
+
+// three stages: tiles (rows 0..BM-1 tokens, BM.. channels) and token scales (8 waves x 64 floats, see below)
+__shared__ __attribute__((aligned(1024))) uint8_t t_stage0[(128 + T_BN) * KSTEP];
+__shared__ __attribute__((aligned(1024))) uint8_t t_stage1[(128 + T_BN) * KSTEP];
+__shared__ __attribute__((aligned(1024))) uint8_t t_stage2[(128 + T_BN) * KSTEP];
+__shared__ __attribute__((aligned(256))) float t_scale0[512];
+__shared__ __attribute__((aligned(256))) float t_scale1[512];
+__shared__ __attribute__((aligned(256))) float t_scale2[512];
+
+struct Frag {
+  u32x4 lo, hi;
+};
+__device__ __forceinline__ v8i as_v8i(const Frag& f) {
+  return v8i{(int)f.lo.x, (int)f.lo.y, (int)f.lo.z, (int)f.lo.w, (int)f.hi.x, (int)f.hi.y, (int)f.hi.z, (int)f.hi.w};
+}
+__device__ __forceinline__ u32x4 lds16(lds_cptr p, int imm) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(p + imm);
+}
+
+template <int BM>
+struct Dma3State {
+  static constexpr int LOADS = (BM + T_BN) / 64;  // tile loads per wave and stage (a wave fills 8 rows per load)
+  const uint8_t* a_base;
+  const uint8_t* b_base;
+  uint32_t goff[LOADS];   // lane's byte offset from the matrix base (rows clamped); first BM/64 loads are token rows
+  const float* sa_ptr;    // &sa[m, 0] of the token whose scale this lane fetches (lanes beyond BM refetch a valid one)
+  cfloat_ptr sb_ptr;      // &sb[nb, 0] of this wave's 128-channel block
+  int64_t sa_sk, sb_sk;
+  int wave, kb_last;
+  uint32_t tok_off[2], ch_off[2], sc_off;
+};
+
+// Load number i (< LOADS: tile rows; == LOADS: token scales) of K block kb, written as instructions.
+template <int BM>
+__device__ __forceinline__ void issue_one(const Dma3State<BM>& s, int i, uint8_t* stage, float* scale, int kb) {
+  constexpr int LOADS = Dma3State<BM>::LOADS;
+  kb = min(kb, s.kb_last);
+  if (i < LOADS) {
+    const uint8_t* base = (i < BM / 64 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
+    asm volatile("" : "+s"(base));
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
+  } else {
+    const float* src = s.sa_ptr + (int64_t)kb * s.sa_sk;
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(scale + s.wave * 64);
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+  }
+}
+
+// One K block out of `cur`; the loads of block kb_next go out over the first LOADS + 1 steps into `nxt`.
+template <int BM>
+__device__ __forceinline__ void k_block(const Dma3State<BM>& s, const uint8_t* cur, const float* sc_cur, float sbv,
+                                        float (&acc)[T_NT][BM / 32][4], uint8_t* nxt, float* sc_nxt, int kb_next) {
+  constexpr int MT = BM / 32, LOADS = Dma3State<BM>::LOADS;
+  static_assert(LOADS + 1 <= MT * T_NT, "one load per step");
+  Frag w[T_NT], tokb[2];
+  float scb[2];
+  const lds_cptr ch0 = (lds_cptr)cur + s.ch_off[0], ch1 = (lds_cptr)cur + s.ch_off[1];
+  const lds_cptr tk0 = (lds_cptr)cur + s.tok_off[0], tk1 = (lds_cptr)cur + s.tok_off[1];
+  w[0].lo = lds16(ch0, 0);
+  w[0].hi = lds16(ch1, 0);
+  tokb[0].lo = lds16(tk0, 0);
+  tokb[0].hi = lds16(tk1, 0);
+  const float* scp = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(sc_cur) + s.sc_off);
+  scb[0] = scp[0] * sbv;
+  __builtin_amdgcn_sched_barrier(0);
+
+  v4f part[2];
+#pragma unroll
+  for (int t = 0; t < MT * T_NT; ++t) {
+    const int j = t >> 2, i = t & 3;
+    part[t & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w[i]), as_v8i(tokb[j & 1]),
+                                                                   v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first; the rest of the step runs in its shadow
+    if (t > 0) {
+      const int pj = (t - 1) >> 2, pi = (t - 1) & 3;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[(t - 1) & 1][v], scb[pj & 1], acc[pi][pj][v]);
+    }
+    if (t + 1 < T_NT) {  // remaining weight fragments, one per step
+      w[t + 1].lo = lds16(ch0, (t + 1) * 2048);
+      w[t + 1].hi = lds16(ch1, (t + 1) * 2048);
+    }
+    if (i == 0 && j + 1 < MT) {  // next token tile
+      tokb[(j + 1) & 1].lo = lds16(tk0, (j + 1) * 2048);
+      tokb[(j + 1) & 1].hi = lds16(tk1, (j + 1) * 2048);
+    }
+    if (i == 1 && j + 1 < MT) scb[(j + 1) & 1] = scp[(j + 1) * 16] * sbv;
+    if (t <= LOADS) issue_one<BM>(s, t, nxt, sc_nxt, kb_next);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  {
+    constexpr int t = MT * T_NT - 1;
+    constexpr int pj = t >> 2, pi = t & 3;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[t & 1][v], scb[pj & 1], acc[pi][pj][v]);
+  }
+}
+
+// Everything but the youngest block's loads has landed; then the workgroup barrier.  Instructions, see the file comment.
+template <int YOUNGER>
+__device__ __forceinline__ void wait_and_barrier() {
+  static_assert(YOUNGER == 6 || YOUNGER == 7, "LOADS + 1 for BM = 64 / 128");
+  if constexpr (YOUNGER == 7) asm volatile("s_waitcnt vmcnt(7)\n\ts_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
+}
+
+template <int BM, bool SPLIT>
+__global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmParams p) {
+  constexpr int WM = BM / 2, MT = WM / 16, LOADS = Dma3State<BM>::LOADS;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave >> 2, wave_n = wave & 3;
+  const int l16 = lane & 15, q = lane >> 4;
+
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
+  const int m0 = tc.tile_m * BM, n0 = tc.tile_n * T_BN;
+  const int kb_begin = tc.split * p.kb_per_split;
+  const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
+  const int nkb = kb_end - kb_begin;
+
+  Dma3State<BM> s;
+  s.wave = wave;
+  s.kb_last = kb_end - 1;
+  s.a_base = p.a;
+  s.b_base = p.b;
+  {
+    const int lrow = lane >> 3;
+    const int chunk_byte = ((lane & 7) ^ lrow) * 16;  // lane fetches the chunk that lands swizzled by (row & 7)
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int row = i * 64 + wave * 8 + lrow;
+      if (row < BM)
+        s.goff[i] = (uint32_t)((int64_t)min(m0 + row, p.M - 1) * p.lda + chunk_byte);
+      else
+        s.goff[i] = (uint32_t)((int64_t)min(n0 + row - BM, p.N - 1) * p.ldb + chunk_byte);
+    }
+    const int trow = wave_m * WM + l16, crow = BM + wave_n * T_WN + l16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      s.tok_off[h] = trow * KSTEP + (((q + 4 * h) ^ (trow & 7)) << 4);
+      s.ch_off[h] = crow * KSTEP + (((q + 4 * h) ^ (crow & 7)) << 4);
+    }
+    s.sc_off = (wave_m * WM + l16) * 4;
+  }
+  // all eight waves fetch 64 token scales each (branch-free); the tile only has BM of them, the rest are refetched copies
+  s.sa_ptr = p.sa + (int64_t)min(m0 + (tid & (BM - 1)), p.M - 1) * p.sa_sm;
+  s.sa_sk = p.sa_sk;
+  s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * T_WN, p.N - 1) / 128) * p.sb_sn);
+  s.sb_sk = p.sb_sk;
+
+  float acc[T_NT][MT][4];
+#pragma unroll
+  for (int i = 0; i < T_NT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+  // ---- prologue: blocks 0 and 1 (clamped) into stages 0 and 1
+#pragma unroll
+  for (int i = 0; i <= LOADS; ++i) issue_one<BM>(s, i, t_stage0, t_scale0, kb_begin);
+#pragma unroll
+  for (int i = 0; i <= LOADS; ++i) issue_one<BM>(s, i, t_stage1, t_scale1, kb_begin + 1);
+  wait_and_barrier<LOADS + 1>();  // block 0 has landed everywhere
+
+  // ---- three blocks per trip over the three stages; iteration k multiplies block k, requests block k + 2
+  int k = 0;
+  for (; k + 2 < nkb; k += 3) {
+    const float sb0 = s.sb_ptr[(int64_t)(kb_begin + k) * s.sb_sk];
+    const float sb1 = s.sb_ptr[(int64_t)(kb_begin + k + 1) * s.sb_sk];
+    const float sb2 = s.sb_ptr[(int64_t)(kb_begin + k + 2) * s.sb_sk];
+    k_block<BM>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2);
+    wait_and_barrier<LOADS + 1>();
+    k_block<BM>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3);
+    wait_and_barrier<LOADS + 1>();
+    k_block<BM>(s, t_stage2, t_scale2, sb2, acc, t_stage1, t_scale1, kb_begin + k + 4);
+    wait_and_barrier<LOADS + 1>();
+  }
+  if (k < nkb) {  // one or two blocks left, in stages 0 and 1
+    k_block<BM>(s, t_stage0, t_scale0, s.sb_ptr[(int64_t)(kb_begin + k) * s.sb_sk], acc, t_stage2, t_scale2, kb_begin + k + 2);
+    wait_and_barrier<LOADS + 1>();
+    if (k + 1 < nkb)
+      k_block<BM>(s, t_stage1, t_scale1, s.sb_ptr[(int64_t)(kb_begin + k + 1) * s.sb_sk], acc, t_stage0, t_scale0, kb_begin + k + 3);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
+
+  // ---- epilogue: lane holds channels n .. n+3 of token m
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = m0 + wave_m * WM + j * 16 + l16;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int i = 0; i < T_NT; ++i) {
+      const int n = n0 + wave_n * T_WN + i * 16 + 4 * q;
+      if (n >= p.N) continue;
+      const int nvalid = min(4, p.N - n);
+      if constexpr (SPLIT) {
+        float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)tc.split * p.M + m) * p.N + n;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (v < nvalid) wsp[v] = acc[i][j][v];
+      } else {
+        store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
+      }
+    }
+  }
+}
+
+template <int BM>
+int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
+  p.tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + T_BN - 1) / T_BN;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits));
+  if (p.splits > 1)
+    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true>), grid, dim3(T_THREADS), 0, stream, p);
+  else
+    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false>), grid, dim3(T_THREADS), 0, stream, p);
+  return check_launch(what);
+}
+
+}  // namespace
+
+// Token-tile height and split count for the mid-M kernel.  One workgroup per CU fits (three stages fill the LDS).
+// The estimate is a byte model, since this regime is bound by weight streaming: a split multiplies the number of
+// workgroups (better balance over 256 CUs when there are few tiles) but every extra split writes and re-reads an
+// M x N fp32 partial tile, and short K ranges pay the pipeline fill (two blocks) each.
+//   efficiency = balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2)
+// `efficiency` is returned so that the dispatcher can prefer another kernel when no split does well.
+Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
+  Dma3Plan pl;
+  pl.bm = M <= 64 ? 64 : 128;
+  const int64_t kb_total = (K + KSTEP - 1) / KSTEP;
+  const int64_t tiles = ((M + pl.bm - 1) / pl.bm) * ((N + T_BN - 1) / T_BN);
+  const double useful = (double)N * K + (double)M * K + 2.0 * M * N;
+  int best = 1;
+  double best_score = -1.0;
+  const int max_split = (N % 4 == 0) ? 16 : 1;  // the reduce kernel works on aligned quads of one row
+  for (int sp = 1; sp <= max_split; ++sp) {
+    const int64_t per = (kb_total + sp - 1) / sp;
+    if (sp > 1 && per < 4) break;
+    if ((kb_total + per - 1) / per != sp) continue;  // some split would get no work
+    const int64_t wgs = tiles * sp;
+    const int64_t rounds = (wgs + 255) / 256;
+    const double balance = (double)wgs / (double)(rounds * 256);
+    const double partial = sp > 1 ? 8.0 * sp * M * N : 0.0;
+    const double score = balance * useful / (useful + partial) * (double)per / (double)(per + 2);
+    if (score > best_score) best_score = score, best = sp;
+  }
+  pl.splits = best;
+  pl.kb_per_split = (int)((kb_total + best - 1) / best);
+  pl.efficiency = best_score;
+  return pl;
+}
+
+int launch_fp8_dma3(GemmParams& p, hipStream_t stream, const char* what) {
+  const Dma3Plan pl = dma3_plan(p.M, p.N, p.K);
+  return pl.bm == 64 ? launch_bm<64>(p, stream, what) : launch_bm<128>(p, stream, what);
+}
+
+}  // namespace mi355

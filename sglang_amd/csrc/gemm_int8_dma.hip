@@ -139,6 +139,9 @@ __global__ __launch_bounds__(I_THREADS) void int8_gemm_dma_kernel(const GemmPara
   }
   if (kb < nkb) k_step(s, i_stage0, acc, i_stage1, kb);
 
+  // the last iterations refetch a block into a stage nobody reads: those writes must not outlive this workgroup's LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
   // ---- epilogue: lane holds, for token m, channels n0 + 32 i + 8 g + 4 kh + (0..3), g = 0..3
   const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
   const bool raw = p.out_dtype == MI355_I32;

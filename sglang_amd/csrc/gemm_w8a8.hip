@@ -301,6 +301,10 @@ struct Plan {
   int bm, bn, splits, kb_per_split;
 };
 
+// below this modelled efficiency of the three-stage mid-M kernel's best tiling the generic kernel (128-wide channel
+// tiles, two workgroups per CU) does better
+constexpr double DMA3_MIN_EFFICIENCY = 0.30;
+
 constexpr int NUM_CUS = 256;
 
 // Tile and split selection.  Large token counts are MFMA-bound and want the biggest tile; small ones
@@ -336,6 +340,11 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const Plan pl = make_plan(M, N, K);
   size_t need = pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
+  if (is_fp8 && M > 16 && M <= 1024 && K % KSTEP == 0) {
+    const Dma3Plan dp = dma3_plan(M, N, K);  // (an upper bound: the dispatcher may still pick the generic kernel)
+    const size_t dneed = dp.splits > 1 ? (size_t)dp.splits * (size_t)M * (size_t)N * 4u : 0;
+    if (dneed > need) need = dneed;
+  }
   if (decode_supported(M, N, K)) {
     const int ds = decode_splits(M, N, K);
     const size_t dneed = ds > 1 ? (size_t)ds * (size_t)M * (size_t)N * 4u : 0;
@@ -403,6 +412,28 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
     const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
     hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
     return check_launch(what);
+  }
+  if constexpr (IS_FP8) {
+    if (p.M > 16 && p.M <= 1024 && p.K % KSTEP == 0 && aligned && (int64_t)p.M * p.lda < (1ll << 32) &&
+        (int64_t)p.N * p.ldb < (1ll << 32) && dma3_plan(p.M, p.N, p.K).efficiency >= DMA3_MIN_EFFICIENCY) {
+      // mid-M: three-stage direct-to-LDS kernel, when its tiling fills the chip well enough
+      const Dma3Plan dp = dma3_plan(p.M, p.N, p.K);
+      p.splits = dp.splits;
+      p.kb_per_split = dp.kb_per_split;
+      if (p.splits > 1) {
+        const size_t need = (size_t)p.splits * (size_t)p.M * (size_t)p.N * 4u;
+        MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
+                      "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
+        MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
+                      "%s: workspace must be 16-byte aligned", what);
+        p.ws = workspace;
+      }
+      int rc = launch_fp8_dma3(p, stream, what);
+      if (rc != MI355_OK || p.splits == 1) return rc;
+      const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
+      hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
+      return check_launch(what);
+    }
   }
   const Plan pl = make_plan(p.M, p.N, p.K);
   p.splits = pl.splits;
