@@ -103,6 +103,7 @@ struct Dma3Plan {
 };
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K);
 int launch_fp8_dma3(GemmParams& p, hipStream_t stream, const char* what);
+int launch_int8_dma3(GemmParams& p, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
 
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, 32x32x32 MFMA); gemm_int8_dma.hip.
 // Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.

@@ -1,0 +1,225 @@
+// Mid-M per-token x per-channel INT8 GEMM for gfx950: (64 or 128) x 256 macro tile, 8 waves, THREE LDS stages.
+//
+// The loop structure is the one of gemm_fp8_dma3.hip: the direct-to-LDS loads of K step k+2 are issued while step k is
+// multiplied, the wait before the bare s_barrier that ends iteration k covers step k+1 only (s_waitcnt vmcnt(LOADS), the
+// loads per wave and iteration being a constant), loads, wait and barrier are written as instructions.  The arithmetic
+// is the one of gemm_int8_dma.hip: v_mfma_i32_32x32x32_i8, four per 32 x 32 tile and 128-byte K step, exact int32
+// accumulation, fragments of 32 rows x 2 K halves read with the (row >> 1) & 7 swizzle.  A wave owns (BM / 2) x 64 outputs.
+// Optional split along K: int32 partials to the workspace, the ordered reduce applies the epilogue.
+// Requires K % 128 == 0, 16-byte aligned rows, row offsets below 4 GiB.
+#include "gemm_common.h"
+
+namespace mi355 {
+namespace {
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int U_THREADS = 512;
+constexpr int U_BN = 256, U_WN = 64, U_NT = U_WN / 32;
+
+typedef __attribute__((address_space(3))) void* lptr_t;
+typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
+
+__shared__ __attribute__((aligned(1024))) uint8_t u_stage0[(128 + U_BN) * KSTEP];
+__shared__ __attribute__((aligned(1024))) uint8_t u_stage1[(128 + U_BN) * KSTEP];
+__shared__ __attribute__((aligned(1024))) uint8_t u_stage2[(128 + U_BN) * KSTEP];
+
+__device__ __forceinline__ v4i lds16(lds_cptr p, int imm) {
+  const u32x4 v = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(p + imm);
+  return v4i{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+}
+
+template <int BM>
+struct U8State {
+  static constexpr int LOADS = (BM + U_BN) / 64;
+  const uint8_t* a_base;
+  const uint8_t* b_base;
+  uint32_t goff[LOADS];
+  int wave, kb_last;
+  uint32_t tok_off[4], ch_off[4];  // per K sub-step: this lane's 16 bytes in the first token / channel tile
+};
+
+template <int BM>
+__device__ __forceinline__ void issue_one(const U8State<BM>& s, int i, uint8_t* stage, int kb) {
+  kb = min(kb, s.kb_last);
+  const uint8_t* base = (i < BM / 64 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
+  asm volatile("" : "+s"(base));
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
+}
+
+// One 128-byte K step out of `cur`; the loads of step kb_next go out in between, into `nxt`.
+template <int BM>
+__device__ __forceinline__ void k_step(const U8State<BM>& s, const uint8_t* cur, v16i (&acc)[U_NT][BM / 64], uint8_t* nxt,
+                                       int kb_next) {
+  constexpr int MT = BM / 64, LOADS = U8State<BM>::LOADS;
+  v4i w[U_NT][4], t[MT][4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+#pragma unroll
+    for (int i = 0; i < U_NT; ++i) w[i][k] = lds16((lds_cptr)cur + s.ch_off[k], i * 4096);
+#pragma unroll
+    for (int j = 0; j < MT; ++j) t[j][k] = lds16((lds_cptr)cur + s.tok_off[k], j * 4096);
+  }
+  int issued = 0;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+#pragma unroll
+      for (int i = 0; i < U_NT; ++i)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[i][k], t[j][k], acc[i][j], 0, 0, 0);
+      if (issued < LOADS) issue_one<BM>(s, issued++, nxt, kb_next);
+      if (issued < LOADS && MT == 1) issue_one<BM>(s, issued++, nxt, kb_next);  // 4 groups only: two loads per group
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+template <int LOADS>
+__device__ __forceinline__ void wait_and_barrier() {
+  static_assert(LOADS == 5 || LOADS == 6, "(BM + 256) / 64");
+  if constexpr (LOADS == 6) asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(5)\n\ts_barrier" ::: "memory");
+}
+
+template <int BM, bool SPLIT>
+__global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmParams p) {
+  constexpr int WM = BM / 2, MT = WM / 32, LOADS = U8State<BM>::LOADS;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave >> 2, wave_n = wave & 3;
+  const int l32 = lane & 31, kh = lane >> 5;
+
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
+  const int m0 = tc.tile_m * BM, n0 = tc.tile_n * U_BN;
+  const int kb_begin = tc.split * p.kb_per_split;
+  const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
+  const int nkb = kb_end - kb_begin;
+
+  U8State<BM> s;
+  s.wave = wave;
+  s.kb_last = kb_end - 1;
+  s.a_base = p.a;
+  s.b_base = p.b;
+  {
+    // lane l lands in row l / 8, physical chunk l % 8 of the 8 rows one load fills; rows start at multiples of 8, so
+    // (row >> 1) & 7 == (4 * wave + (l >> 4)) & 7 for every load of this wave
+    const int lrow = lane >> 3;
+    const int key = (4 * wave + (lane >> 4)) & 7;
+    const int chunk_byte = ((lane & 7) ^ key) * 16;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int row = i * 64 + wave * 8 + lrow;
+      if (row < BM)
+        s.goff[i] = (uint32_t)((int64_t)min(m0 + row, p.M - 1) * p.lda + chunk_byte);
+      else
+        s.goff[i] = (uint32_t)((int64_t)min(n0 + row - BM, p.N - 1) * p.ldb + chunk_byte);
+    }
+    const int trow = wave_m * WM + l32, crow = BM + wave_n * U_WN + l32;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {  // K sub-step k takes the 16-byte chunk 2k + kh of the row
+      s.tok_off[k] = trow * KSTEP + (((2 * k + kh) ^ ((trow >> 1) & 7)) << 4);
+      s.ch_off[k] = crow * KSTEP + (((2 * k + kh) ^ ((crow >> 1) & 7)) << 4);
+    }
+  }
+
+  v16i acc[U_NT][MT];
+#pragma unroll
+  for (int i = 0; i < U_NT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) issue_one<BM>(s, i, u_stage0, kb_begin);
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) issue_one<BM>(s, i, u_stage1, kb_begin + 1);
+  wait_and_barrier<LOADS>();
+
+  int k = 0;
+  for (; k + 2 < nkb; k += 3) {
+    k_step<BM>(s, u_stage0, acc, u_stage2, kb_begin + k + 2);
+    wait_and_barrier<LOADS>();
+    k_step<BM>(s, u_stage1, acc, u_stage0, kb_begin + k + 3);
+    wait_and_barrier<LOADS>();
+    k_step<BM>(s, u_stage2, acc, u_stage1, kb_begin + k + 4);
+    wait_and_barrier<LOADS>();
+  }
+  if (k < nkb) {
+    k_step<BM>(s, u_stage0, acc, u_stage2, kb_begin + k + 2);
+    wait_and_barrier<LOADS>();
+    if (k + 1 < nkb) k_step<BM>(s, u_stage1, acc, u_stage0, kb_begin + k + 3);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
+
+  // ---- epilogue: lane holds, for token m, channels n0 + 32 i + 8 g + 4 kh + (0..3), g = 0..3
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+  const bool raw = p.out_dtype == MI355_I32;
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = m0 + wave_m * WM + j * 32 + l32;
+    if (m >= p.M) continue;
+    float sa_m = 1.f;
+    if constexpr (!SPLIT) {
+      if (!raw) sa_m = p.sa[m];
+    }
+#pragma unroll
+    for (int i = 0; i < U_NT; ++i) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wave_n * U_WN + i * 32 + 8 * g + 4 * kh;
+        if (n >= p.N) continue;
+        const int nvalid = min(4, p.N - n);
+        if constexpr (SPLIT) {
+          int* wsp = reinterpret_cast<int*>(p.ws) + ((int64_t)tc.split * p.M + m) * p.N + n;
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (v < nvalid) wsp[v] = acc[i][j][4 * g + v];
+        } else if (raw) {
+          int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            if (v < nvalid) o[v] = acc[i][j][4 * g + v];
+        } else {
+          float r[4];
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int nn = min(n + v, p.N - 1);
+            float t = __fmul_rn((float)acc[i][j][4 * g + v], __fmul_rn(p.sb[nn], sa_m));
+            if (p.bias) {
+              const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[nn];
+              t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+            }
+            r[v] = t;
+          }
+          store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, nvalid, vec_ok);
+        }
+      }
+    }
+  }
+}
+
+template <int BM>
+int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
+  p.tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + U_BN - 1) / U_BN;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits));
+  if (p.splits > 1)
+    hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, true>), grid, dim3(U_THREADS), 0, stream, p);
+  else
+    hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, false>), grid, dim3(U_THREADS), 0, stream, p);
+  return check_launch(what);
+}
+
+}  // namespace
+
+// Tiling and split are those of the FP8 mid-M kernel (dma3_plan): same tile shapes, same byte model.
+int launch_int8_dma3(GemmParams& p, hipStream_t stream, const char* what) {
+  const Dma3Plan pl = dma3_plan(p.M, p.N, p.K);
+  return pl.bm == 64 ? launch_bm<64>(p, stream, what) : launch_bm<128>(p, stream, what);
+}
+
+}  // namespace mi355

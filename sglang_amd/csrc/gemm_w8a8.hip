@@ -340,7 +340,7 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const Plan pl = make_plan(M, N, K);
   size_t need = pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
-  if (is_fp8 && M > 16 && M <= 1024 && K % KSTEP == 0) {
+  if (M > 16 && M <= 1024 && K % KSTEP == 0) {
     const Dma3Plan dp = dma3_plan(M, N, K);  // (an upper bound: the dispatcher may still pick the generic kernel)
     const size_t dneed = dp.splits > 1 ? (size_t)dp.splits * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
@@ -413,7 +413,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
     hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
     return check_launch(what);
   }
-  if constexpr (IS_FP8) {
+  {
     if (p.M > 16 && p.M <= 1024 && p.K % KSTEP == 0 && aligned && (int64_t)p.M * p.lda < (1ll << 32) &&
         (int64_t)p.N * p.ldb < (1ll << 32) && dma3_plan(p.M, p.N, p.K).efficiency >= DMA3_MIN_EFFICIENCY) {
       // mid-M: three-stage direct-to-LDS kernel, when its tiling fills the chip well enough
@@ -428,10 +428,10 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
                       "%s: workspace must be 16-byte aligned", what);
         p.ws = workspace;
       }
-      int rc = launch_fp8_dma3(p, stream, what);
+      int rc = IS_FP8 ? launch_fp8_dma3(p, stream, what) : launch_int8_dma3(p, stream, what);
       if (rc != MI355_OK || p.splits == 1) return rc;
       const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
-      hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
+      hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
       return check_launch(what);
     }
   }
