@@ -125,6 +125,19 @@ int mi355_int8_scaled_mm(const void* a, const void* b, const float* sa, const fl
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Host-only query: which kernel and tiling mi355_fp8_blockwise_mm / mi355_int8_scaled_mm would run for a shape.
+ * Stands in for the reference's shape dispatchers, which are compile-time ladders nobody can ask
+ * (sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:181-195, sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:603-661);
+ * here the choice is observable so that tests can prove every kernel variant is reached.
+ *   aligned  nonzero if both operand base pointers and row strides are multiples of 16 bytes (rows are assumed dense)
+ *   buf      receives a NUL-terminated "key=value ..." line:
+ *            kernel=decode|dma3|dma256|pipelined|int8_dma256|generic bm= bn= splits= kb_per_split= groups_per_wg= aligned=
+ * Launches nothing and touches no device state.
+ */
+int mi355_fp8_blockwise_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len);
+int mi355_int8_scaled_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len);
+
+/*
  * Per-token INT8 activation quantization: absmax = max(1e-10, max |x[m,:]|), s[m] = absmax / 127,
  * q = round-half-away-from-zero(x * (127 / absmax)).
  * Replaces per_token_quant_int8 (python/sglang/srt/layers/quantization/int8_kernel.py:28-89, without cal_sum).

@@ -26,6 +26,8 @@ EXPORTS = (
     "mi355_fp8_blockwise_mm",
     "mi355_int8_scaled_mm_workspace_bytes",
     "mi355_int8_scaled_mm",
+    "mi355_fp8_blockwise_mm_plan",
+    "mi355_int8_scaled_mm_plan",
     "mi355_per_token_quant_int8",
 )
 
@@ -67,6 +69,9 @@ def lib() -> ctypes.CDLL:
     L.mi355_int8_scaled_mm_workspace_bytes.restype = sz
     L.mi355_int8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32] + [i64] * 6 + [vp, sz, vp]
     L.mi355_int8_scaled_mm.restype = i32
+    for fn in (L.mi355_fp8_blockwise_mm_plan, L.mi355_int8_scaled_mm_plan):
+        fn.argtypes = [i64, i64, i64, i32, ctypes.c_char_p, sz]
+        fn.restype = i32
     L.mi355_per_token_quant_int8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
     L.mi355_per_token_quant_int8.restype = i32
     got = L.mi355_qlinear_abi_version()
@@ -74,6 +79,19 @@ def lib() -> ctypes.CDLL:
         raise ImportError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}: rebuild it")
     _lib = L
     return L
+
+
+def gemm_plan(kind: str, M: int, N: int, K: int, aligned: bool = True) -> dict:
+    """Kernel and tiling the library would use for an FP8 (`kind` "fp8") or INT8 ("int8") GEMM of this shape:
+    {"kernel": str, "bm": int, "bn": int, "splits": int, "kb_per_split": int, "groups_per_wg": int, "aligned": int}."""
+    fn = {"fp8": lib().mi355_fp8_blockwise_mm_plan, "int8": lib().mi355_int8_scaled_mm_plan}[kind]
+    buf = ctypes.create_string_buffer(256)
+    check(fn(M, N, K, int(aligned), buf, len(buf)))
+    out = {}
+    for item in buf.value.decode().split():
+        k, v = item.split("=")
+        out[k] = v if k == "kernel" else int(v)
+    return out
 
 
 def check(status: int) -> None:

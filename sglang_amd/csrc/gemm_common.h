@@ -102,8 +102,8 @@ struct Dma3Plan {
   double efficiency;  // modelled fraction of the streaming time that is useful (balance, partial sums, pipeline fill)
 };
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K);
-int launch_fp8_dma3(GemmParams& p, hipStream_t stream, const char* what);
-int launch_int8_dma3(GemmParams& p, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
+int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);   // bm: 64 or 128, from dma3_plan()
+int launch_int8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
 
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, 32x32x32 MFMA); gemm_int8_dma.hip.
 // Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
@@ -112,8 +112,10 @@ int launch_int8_dma(GemmParams& p, hipStream_t stream, const char* what);
 // Small-M blockwise FP8 GEMM streaming the weight through wave-private LDS, no barriers; gemm_fp8_decode.hip.
 // decode_splits() is the split count it wants for a shape; the caller sets p.splits, p.kb_per_split and p.ws.
 int decode_splits(int64_t M, int64_t N, int64_t K);
+int decode_kb_per_range();  // K blocks per split (the last range may be shorter)
 bool decode_supported(int64_t M, int64_t N, int64_t K);
-int launch_fp8_decode(GemmParams& p, hipStream_t stream, const char* what);
-int launch_int8_decode(GemmParams& p, hipStream_t stream, const char* what);  // same kernel, int8 MFMA, int32 partials
+int decode_groups_per_wg(int64_t N, int splits);  // consecutive 128-channel groups one workgroup walks
+int launch_fp8_decode(GemmParams& p, int groups_per_wg, hipStream_t stream, const char* what);
+int launch_int8_decode(GemmParams& p, int groups_per_wg, hipStream_t stream, const char* what);  // same kernel, int8 MFMA, int32 partials
 
 }  // namespace mi355

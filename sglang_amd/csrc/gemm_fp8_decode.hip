@@ -88,7 +88,7 @@ __device__ __forceinline__ void issue_weights(const DecodeState& s, uint8_t* sta
     if constexpr (MANUAL) {
       const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)dst;
       asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.woff[j]), "s"(base), "s"(lds_addr)
-                   : "memory");  // m0 is written here; no compiler-managed instruction in the loop depends on it
+                   : "memory", "m0");
     } else {
       __builtin_amdgcn_global_load_lds((gptr_t)(base + s.woff[j]), (lptr_t)dst, 16, 0, 0);
     }
@@ -291,16 +291,21 @@ int decode_splits(int64_t M, int64_t N, int64_t K) {
   return (int)((kb_total + KB_PER - 1) / KB_PER);
 }
 
+int decode_kb_per_range() { return KB_PER; }
+
 // Shapes the decode kernel takes: one token tile, whole K blocks, channels in whole groups of 128.
 bool decode_supported(int64_t M, int64_t N, int64_t K) { return M >= 1 && M <= 16 && K % KSTEP == 0 && N % GROUP_N == 0; }
 
 // Also needs 16-byte aligned rows and row offsets below 4 GiB.  The caller sets p.splits (= decode_splits) and p.ws.
+// About two workgroups per CU; each walks this many consecutive channel groups with the same tokens.
+int decode_groups_per_wg(int64_t N, int splits) {
+  const int gpw = (int)(((N / GROUP_N) * splits + 511) / 512);
+  return gpw < 1 ? 1 : gpw;
+}
+
 template <bool IS_FP8>
-static int launch_decode(GemmParams& p, hipStream_t stream, const char* what) {
+static int launch_decode(GemmParams& p, int gpw, hipStream_t stream, const char* what) {
   const int groups_n = p.N / GROUP_N;
-  // about two workgroups per CU; each walks `gpw` consecutive channel groups with the same tokens
-  int gpw = (int)(((int64_t)groups_n * p.splits + 511) / 512);
-  if (gpw < 1) gpw = 1;
   const int wg_per_split = (groups_n + gpw - 1) / gpw;
   p.tiles_m = 1;
   p.tiles_n = groups_n;
@@ -312,7 +317,7 @@ static int launch_decode(GemmParams& p, hipStream_t stream, const char* what) {
   return check_launch(what);
 }
 
-int launch_fp8_decode(GemmParams& p, hipStream_t stream, const char* what) { return launch_decode<true>(p, stream, what); }
-int launch_int8_decode(GemmParams& p, hipStream_t stream, const char* what) { return launch_decode<false>(p, stream, what); }
+int launch_fp8_decode(GemmParams& p, int gpw, hipStream_t stream, const char* what) { return launch_decode<true>(p, gpw, stream, what); }
+int launch_int8_decode(GemmParams& p, int gpw, hipStream_t stream, const char* what) { return launch_decode<false>(p, gpw, stream, what); }
 
 }  // namespace mi355

@@ -68,11 +68,11 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM>& s, int i, uint8_t
     const uint8_t* base = (i < BM / 64 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
     asm volatile("" : "+s"(base));
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory", "m0");
   } else {
     const float* src = s.sa_ptr + (int64_t)kb * s.sa_sk;
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(scale + s.wave * 64);
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds_addr) : "memory", "m0");
   }
 }
 
@@ -284,9 +284,8 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
   return pl;
 }
 
-int launch_fp8_dma3(GemmParams& p, hipStream_t stream, const char* what) {
-  const Dma3Plan pl = dma3_plan(p.M, p.N, p.K);
-  return pl.bm == 64 ? launch_bm<64>(p, stream, what) : launch_bm<128>(p, stream, what);
+int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what) {
+  return bm == 64 ? launch_bm<64>(p, stream, what) : launch_bm<128>(p, stream, what);
 }
 
 }  // namespace mi355

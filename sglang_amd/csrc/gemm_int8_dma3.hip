@@ -45,7 +45,7 @@ __device__ __forceinline__ void issue_one(const U8State<BM>& s, int i, uint8_t* 
   const uint8_t* base = (i < BM / 64 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
   asm volatile("" : "+s"(base));
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
 // One 128-byte K step out of `cur`; the loads of step kb_next go out in between, into `nxt`.
@@ -217,9 +217,8 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 }  // namespace
 
 // Tiling and split are those of the FP8 mid-M kernel (dma3_plan): same tile shapes, same byte model.
-int launch_int8_dma3(GemmParams& p, hipStream_t stream, const char* what) {
-  const Dma3Plan pl = dma3_plan(p.M, p.N, p.K);
-  return pl.bm == 64 ? launch_bm<64>(p, stream, what) : launch_bm<128>(p, stream, what);
+int launch_int8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what) {
+  return bm == 64 ? launch_bm<64>(p, stream, what) : launch_bm<128>(p, stream, what);
 }
 
 }  // namespace mi355

@@ -20,6 +20,8 @@
 //     workspace and a second kernel adds them in a fixed order (deterministic, no atomics);
 //   * workgroups are renumbered so that each of the 8 XCDs (own L2) works on a contiguous, M-grouped
 //     patch of output tiles.
+#include <mutex>
+
 #include "gemm_common.h"
 
 namespace mi355 {
@@ -353,6 +355,25 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   return need;
 }
 
+template <bool IS_FP8, int BM, int BN, int WGM, int WGN, bool ALIGNED, bool SPLIT>
+int launch_tile_inst(const GemmParams& p, unsigned grid, size_t lds, hipStream_t stream, const char* what) {
+  auto kfn = gemm_kernel<IS_FP8, BM, BN, WGM, WGN, ALIGNED, SPLIT>;
+  if (lds > 64 * 1024) {
+    // more than 64 KB of dynamic LDS has to be granted once per kernel; concurrent first calls may both ask, which is harmless
+    static std::once_flag once;
+    static hipError_t granted = hipSuccess;
+    std::call_once(once, [&] {
+      granted = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
+    if (granted != hipSuccess) {
+      set_error("%s: cannot reserve %zu bytes of LDS: %s", what, lds, hipGetErrorString(granted));
+      return MI355_ERR_LAUNCH;
+    }
+  }
+  hipLaunchKernelGGL(kfn, dim3(grid), dim3(THREADS), lds, stream, p);
+  return check_launch(what);
+}
+
 template <bool IS_FP8, int BM, int BN, int WGM, int WGN>
 int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + BM - 1) / BM;
@@ -360,35 +381,70 @@ int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* wha
   const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n * p.splits);
   const size_t lds = 2 * (size_t)(BM + BN) * KSTEP + (IS_FP8 ? 2 * BM * sizeof(float) : 0);
   const bool split = p.splits > 1;
-#define MI355_LAUNCH(AL, SP)                                                                                   \
-  do {                                                                                                         \
-    auto kfn = gemm_kernel<IS_FP8, BM, BN, WGM, WGN, AL, SP>;                                                  \
-    static bool lds_reserved = false;                                                                          \
-    if (lds > 64 * 1024 && !lds_reserved) {                                                                    \
-      lds_reserved = true;                                                                                     \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                                   \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                \
-      if (e != hipSuccess) {                                                                                   \
-        set_error("%s: cannot reserve %zu bytes of LDS: %s", what, lds, hipGetErrorString(e));                 \
-        return MI355_ERR_LAUNCH;                                                                               \
-      }                                                                                                        \
-    }                                                                                                          \
-    hipLaunchKernelGGL(kfn, dim3(grid), dim3(THREADS), lds, stream, p);                                        \
-  } while (0)
-  if (aligned) {
-    if (split) MI355_LAUNCH(true, true); else MI355_LAUNCH(true, false);
-  } else {
-    if (split) MI355_LAUNCH(false, true); else MI355_LAUNCH(false, false);
+  if (aligned)
+    return split ? launch_tile_inst<IS_FP8, BM, BN, WGM, WGN, true, true>(p, grid, lds, stream, what)
+                 : launch_tile_inst<IS_FP8, BM, BN, WGM, WGN, true, false>(p, grid, lds, stream, what);
+  return split ? launch_tile_inst<IS_FP8, BM, BN, WGM, WGN, false, true>(p, grid, lds, stream, what)
+               : launch_tile_inst<IS_FP8, BM, BN, WGM, WGN, false, false>(p, grid, lds, stream, what);
+}
+
+// Which kernel serves a problem, with which tiling.  One function decides for the launcher and for the plan query, so
+// what the query reports is what runs.
+enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_DMA256, RK_PIPELINED, RK_INT8_DMA256, RK_GENERIC };
+const char* const ROUTE_NAMES[] = {"decode", "dma3", "dma256", "pipelined", "int8_dma256", "generic"};
+
+struct Route {
+  int kernel;
+  int bm, bn;
+  int splits, kb_per_split;
+  int groups_per_wg;  // decode only
+  bool aligned;
+};
+
+// `aligned`: both operand base pointers and row strides are multiples of 16 bytes and K % 16 == 0.
+Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, bool aligned) {
+  Route r{};
+  r.aligned = aligned;
+  const int kb_total = (int)((K + KSTEP - 1) / KSTEP);
+  const bool small_b = N * ldb < (1ll << 32);                 // kernels that address rows by 32-bit byte offsets
+  const bool small_offsets = M * lda < (1ll << 32) && small_b;
+  if (decode_supported(M, N, K) && aligned && small_b) {  // barrier-free weight streaming
+    r.kernel = RK_DECODE, r.bm = 16, r.bn = 128;
+    r.splits = decode_splits(M, N, K);
+    r.kb_per_split = decode_kb_per_range();
+    r.groups_per_wg = decode_groups_per_wg(N, r.splits);
+    return r;
   }
-#undef MI355_LAUNCH
-  int rc = check_launch(what);
-  if (rc != MI355_OK) return rc;
-  if (split) {
-    const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
-    hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
-    rc = check_launch(what);
+  if (M > 16 && M <= 1024 && K % KSTEP == 0 && aligned && small_offsets) {
+    // mid-M: three-stage direct-to-LDS kernel, when its tiling fills the chip well enough
+    const Dma3Plan dp = dma3_plan(M, N, K);
+    if (dp.efficiency >= DMA3_MIN_EFFICIENCY) {
+      r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = 256, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
+      return r;
+    }
   }
-  return rc;
+  const Plan pl = make_plan(M, N, K);
+  r.kernel = RK_GENERIC, r.bm = pl.bm, r.bn = pl.bn, r.splits = pl.splits, r.kb_per_split = pl.kb_per_split;
+  const int64_t tiles_256 = ((M + 255) / 256) * ((N + 255) / 256);
+  const int64_t tiles_128 = ((M + 255) / 256) * ((N + 127) / 128);
+  if (pl.bm == 256 && pl.splits == 1 && aligned && small_offsets) {
+    if (is_fp8) {
+      // 256 x 256 tiles (8 waves, direct-to-LDS) when they still give every CU a workgroup, else 256 x 128
+      if (tiles_256 >= NUM_CUS) {
+        r.kernel = RK_DMA256, r.bn = 256;
+        return r;
+      }
+      if (tiles_128 >= NUM_CUS) {
+        r.kernel = RK_PIPELINED;
+        return r;
+      }
+    } else if (K % KSTEP == 0 && tiles_256 >= NUM_CUS / 2) {
+      r.kernel = RK_INT8_DMA256, r.bn = 256;
+      return r;
+    }
+  }
+  if (r.bm == 256 && tiles_128 < NUM_CUS) r.bm = 128;  // too few 256-row tiles to fill the chip
+  return r;
 }
 
 template <bool IS_FP8>
@@ -396,82 +452,55 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
   p.kb_total = (p.K + KSTEP - 1) / KSTEP;
   const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
                        ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
-  if (decode_supported(p.M, p.N, p.K) && aligned && (int64_t)p.N * p.ldb < (1ll << 32)) {  // barrier-free weight streaming
-    p.splits = decode_splits(p.M, p.N, p.K);
-    p.kb_per_split = (p.kb_total + p.splits - 1) / p.splits;
-    if (p.splits > 1) {
-      const size_t need = (size_t)p.splits * (size_t)p.M * (size_t)p.N * 4u;
-      MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
-                    "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
-      MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
-                    "%s: workspace must be 16-byte aligned", what);
-      p.ws = workspace;
-    }
-    int rc = IS_FP8 ? launch_fp8_decode(p, stream, what) : launch_int8_decode(p, stream, what);
-    if (rc != MI355_OK || p.splits == 1) return rc;
-    const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
-    hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
-    return check_launch(what);
-  }
-  {
-    if (p.M > 16 && p.M <= 1024 && p.K % KSTEP == 0 && aligned && (int64_t)p.M * p.lda < (1ll << 32) &&
-        (int64_t)p.N * p.ldb < (1ll << 32) && dma3_plan(p.M, p.N, p.K).efficiency >= DMA3_MIN_EFFICIENCY) {
-      // mid-M: three-stage direct-to-LDS kernel, when its tiling fills the chip well enough
-      const Dma3Plan dp = dma3_plan(p.M, p.N, p.K);
-      p.splits = dp.splits;
-      p.kb_per_split = dp.kb_per_split;
-      if (p.splits > 1) {
-        const size_t need = (size_t)p.splits * (size_t)p.M * (size_t)p.N * 4u;
-        MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
-                      "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
-        MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
-                      "%s: workspace must be 16-byte aligned", what);
-        p.ws = workspace;
-      }
-      int rc = IS_FP8 ? launch_fp8_dma3(p, stream, what) : launch_int8_dma3(p, stream, what);
-      if (rc != MI355_OK || p.splits == 1) return rc;
-      const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
-      hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
-      return check_launch(what);
-    }
-  }
-  const Plan pl = make_plan(p.M, p.N, p.K);
-  p.splits = pl.splits;
-  p.kb_per_split = pl.kb_per_split;
-  if (pl.splits > 1) {
-    const size_t need = (size_t)pl.splits * (size_t)p.M * (size_t)p.N * 4u;
+  const Route r = choose_route(IS_FP8, p.M, p.N, p.K, p.lda, p.ldb, aligned);
+  p.splits = r.splits;
+  p.kb_per_split = r.kb_per_split;
+  if (r.splits > 1) {
+    const size_t need = (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u;
     MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
                   "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
     MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
                   "%s: workspace must be 16-byte aligned", what);
     p.ws = workspace;
   }
-  if constexpr (IS_FP8) {
-    // the pipelined kernel addresses rows with 32-bit byte offsets from the matrix base
-    const bool small_offsets = (int64_t)p.M * p.lda < (1ll << 32) && (int64_t)p.N * p.ldb < (1ll << 32);
-    if (pl.bm == 256 && pl.splits == 1 && aligned && small_offsets) {
-      // 256 x 256 tiles (8 waves, direct-to-LDS) when they still give every CU a workgroup, else 256 x 128
-      const int64_t tiles_256 = ((int64_t)(p.M + 255) / 256) * ((p.N + 255) / 256);
-      const int64_t tiles_128 = ((int64_t)(p.M + 255) / 256) * ((p.N + 127) / 128);
-      if (tiles_256 >= NUM_CUS) return launch_fp8_dma(p, stream, what);
-      if (tiles_128 >= NUM_CUS) return launch_fp8_pipelined(p, stream, what);
-    }
+  int rc;
+  switch (r.kernel) {
+    case RK_DECODE:
+      rc = IS_FP8 ? launch_fp8_decode(p, r.groups_per_wg, stream, what) : launch_int8_decode(p, r.groups_per_wg, stream, what);
+      break;
+    case RK_DMA3:
+      rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, stream, what) : launch_int8_dma3(p, r.bm, stream, what);
+      break;
+    case RK_DMA256: return launch_fp8_dma(p, stream, what);
+    case RK_PIPELINED: return launch_fp8_pipelined(p, stream, what);
+    case RK_INT8_DMA256: return launch_int8_dma(p, stream, what);
+    default:
+      // the generic kernel runs its own ordered reduce
+      switch (r.bm) {
+        case 16: rc = launch_tile<IS_FP8, 16, 128, 1, 4>(p, aligned, stream, what); break;
+        case 32: rc = launch_tile<IS_FP8, 32, 128, 1, 4>(p, aligned, stream, what); break;
+        case 64: rc = launch_tile<IS_FP8, 64, 128, 1, 4>(p, aligned, stream, what); break;
+        case 128: rc = launch_tile<IS_FP8, 128, 128, 2, 2>(p, aligned, stream, what); break;
+        default: rc = launch_tile<IS_FP8, 256, 128, 2, 2>(p, aligned, stream, what); break;
+      }
   }
-  if constexpr (!IS_FP8) {
-    const bool small_offsets = (int64_t)p.M * p.lda < (1ll << 32) && (int64_t)p.N * p.ldb < (1ll << 32);
-    const int64_t tiles_256 = ((int64_t)(p.M + 255) / 256) * ((p.N + 255) / 256);
-    if (pl.bm == 256 && pl.splits == 1 && aligned && small_offsets && p.K % KSTEP == 0 && tiles_256 >= NUM_CUS / 2)
-      return launch_int8_dma(p, stream, what);
-  }
-  int bm = pl.bm;
-  if (bm == 256 && ((int64_t)(p.M + 255) / 256) * ((p.N + 127) / 128) < NUM_CUS) bm = 128;  // too few 256-row tiles to fill the chip
-  switch (bm) {
-    case 16: return launch_tile<IS_FP8, 16, 128, 1, 4>(p, aligned, stream, what);
-    case 32: return launch_tile<IS_FP8, 32, 128, 1, 4>(p, aligned, stream, what);
-    case 64: return launch_tile<IS_FP8, 64, 128, 1, 4>(p, aligned, stream, what);
-    case 128: return launch_tile<IS_FP8, 128, 128, 2, 2>(p, aligned, stream, what);
-    default: return launch_tile<IS_FP8, 256, 128, 2, 2>(p, aligned, stream, what);
-  }
+  if (rc != MI355_OK || p.splits == 1) return rc;
+  const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
+  hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
+  return check_launch(what);
+}
+
+int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len, const char* what) {
+  clear_error();
+  MI355_REQUIRE(buf != nullptr && buf_len > 0, MI355_ERR_INVALID_ARGUMENT, "%s: no buffer", what);
+  MI355_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31),
+                MI355_ERR_INVALID_ARGUMENT, "%s: shape out of range", what);
+  const Route r = choose_route(is_fp8, M, N, K, K, K, aligned != 0 && K % 16 == 0);
+  const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d",
+                         ROUTE_NAMES[r.kernel], r.bm, r.bn, r.splits, r.kb_per_split, r.groups_per_wg, (int)r.aligned);
+  MI355_REQUIRE(n > 0 && (size_t)n < buf_len, MI355_ERR_INVALID_ARGUMENT, "%s: buffer of %zu bytes is too small", what,
+                buf_len);
+  return MI355_OK;
 }
 
 }  // namespace
@@ -540,4 +569,12 @@ extern "C" int mi355_int8_scaled_mm(const void* a, const void* b, const float* s
   p.lda = lda, p.ldb = ldb, p.ldo = ldo;
   p.out_dtype = out_dtype;
   return run_gemm<false>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
+}
+
+extern "C" int mi355_fp8_blockwise_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len) {
+  return describe_route(true, M, N, K, aligned, buf, buf_len, "mi355_fp8_blockwise_mm_plan");
+}
+
+extern "C" int mi355_int8_scaled_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len) {
+  return describe_route(false, M, N, K, aligned, buf, buf_len, "mi355_int8_scaled_mm_plan");
 }

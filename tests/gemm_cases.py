@@ -1,0 +1,83 @@
+"""Shapes that steer the GEMM dispatcher into every kernel variant, shared by the CPU coverage test and the GPU
+parity tests, plus the full-size shapes of the benchmark configurations.
+
+A *variant* is one compiled code path: the kernel, its token-tile height, whether it writes split-K partial sums,
+for the decode kernel how many 128-channel groups a workgroup walks, for the large-M kernels whether K ends on a
+128-byte block.  `variant_of` maps a plan (sglang_amd._lib.gemm_plan) to such a key.
+"""
+
+# ---- FP8 (M, N, K); K % 16 != 0 means unaligned rows (byte-granular loader)
+FP8_ROUTE_SHAPES = [
+    # decode kernel (M <= 16, K % 128 == 0, N % 128 == 0): whole-K and split, 1 / 2 / 3+ channel groups per workgroup,
+    # an uneven last workgroup (16640 = 130 groups), short last K ranges (4480 = 35 blocks, 2176 = 17 blocks)
+    (1, 128, 128), (3, 256, 512), (1, 512, 7168), (16, 2048, 7168), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432),
+    (7, 33280, 4096), (5, 66048, 512), (2, 133120, 384),
+    # three-stage mid-M kernel: 64 / 128 token tiles, whole-K and split, ragged M, K blocks per range = 1, 2, 0 mod 3
+    (48, 16384, 2048), (33, 16384, 2176), (40, 65536, 512), (200, 16384, 2048), (100, 32768, 640), (130, 8192, 7168),
+    (250, 8192, 7296),
+    # 256 x 256 direct-to-LDS and 256 x 128 pipelined kernels, K a multiple of 128 and not
+    (4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 512), (4000, 2100, 272),
+    # generic kernel: every token-tile height, aligned and byte-granular loads, whole-K and split
+    (7, 1088, 512), (16, 576, 7168), (1, 1088, 3884), (17, 384, 2304), (20, 256, 264), (33, 512, 512), (64, 128, 3884),
+    (50, 300, 520), (127, 128, 4096), (130, 640, 896), (1500, 640, 1000), (130, 200, 300), (2048, 4224, 264),
+]
+
+FP8_REQUIRED_VARIANTS = {
+    ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
+    ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
+    ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
+    ("dma256", "kfull"), ("dma256", "ktail"), ("pipelined", "kfull"), ("pipelined", "ktail"),
+    ("generic", 16, "aligned", "whole"), ("generic", 16, "aligned", "split"), ("generic", 16, "bytes", "split"),
+    ("generic", 32, "aligned", "split"), ("generic", 32, "bytes", "whole"),
+    ("generic", 64, "aligned", "whole"), ("generic", 64, "bytes", "whole"), ("generic", 64, "bytes", "split"),
+    ("generic", 128, "aligned", "whole"), ("generic", 128, "aligned", "split"), ("generic", 128, "bytes", "whole"),
+    ("generic", 128, "bytes", "split"), ("generic", 256, "bytes", "whole"),
+}
+
+# ---- INT8 (M, N, K): the operator requires K % 16 == 0 and N % 8 == 0
+INT8_ROUTE_SHAPES = [
+    (16, 128, 512), (1, 6144, 4096), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432), (7, 33280, 4096),
+    (5, 66048, 512), (2, 133120, 384),
+    (20, 8192, 4096), (40, 65536, 512), (200, 16384, 2048), (300, 4096, 14336), (130, 8192, 7168),
+    (4096, 4096, 512), (4000, 4088, 1024),
+    (1, 16, 512), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
+]
+
+INT8_REQUIRED_VARIANTS = {
+    ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
+    ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
+    ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
+    ("int8_dma256",),
+    ("generic", 16, "aligned", "whole"), ("generic", 32, "aligned", "split"), ("generic", 64, "aligned", "whole"),
+    ("generic", 128, "aligned", "whole"), ("generic", 128, "aligned", "split"), ("generic", 256, "aligned", "whole"),
+}
+
+# ---- the benchmark configurations at full size: name -> (K, N)
+DSV3_MLP = {"gate_up": (7168, 36864), "down": (18432, 7168)}
+DSV3_MLA = {"q_a": (7168, 1536), "kv_a": (7168, 576), "q_b": (1536, 24576), "kv_b": (512, 32768)}
+LLAMA3_8B = {"qkv": (4096, 6144), "gate_up": (4096, 28672), "down": (14336, 4096)}
+
+FP8_DECODE_CONFIG = [(M, N, K) for M in (1, 8, 32, 128) for (K, N) in DSV3_MLP.values()]
+FP8_PREFILL_CONFIG = [(4096, N, K) for (K, N) in list(DSV3_MLP.values()) + list(DSV3_MLA.values())]
+INT8_CONFIG = [(M, N, K) for M in (1, 256, 4096) for (K, N) in LLAMA3_8B.values()]
+
+
+def variant_of(plan: dict, K: int):
+    k = plan["kernel"]
+    sp = "split" if plan["splits"] > 1 else "whole"
+    if k == "decode":
+        g = plan["groups_per_wg"]
+        return (k, sp, f"gpw{g}" if g < 3 else "gpw3+")
+    if k == "dma3":
+        return (k, plan["bm"], sp)
+    if k in ("dma256", "pipelined"):
+        return (k, "kfull" if K % 128 == 0 else "ktail")
+    if k == "int8_dma256":
+        return (k,)
+    return (k, plan["bm"], "aligned" if plan["aligned"] else "bytes", sp)
+
+
+def plan_for(kind: str, M: int, N: int, K: int) -> dict:
+    from sglang_amd import _lib
+
+    return _lib.gemm_plan(kind, M, N, K, aligned=(K % 16 == 0))
