@@ -109,6 +109,24 @@ int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const 
                            void* stream);
 
 /*
+ * mi355_fp8_blockwise_mm for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose operators allocate
+ * their workspaces through the framework.  Same arguments and results as mi355_fp8_blockwise_mm without the workspace:
+ * split-K partial sums go to a MI355_NOALLOC_SCRATCH_BYTES array that lives in the library's device image (each GPU
+ * that loads the library holds one until the process ends).  The call allocates and frees nothing.
+ *   - A problem whose partial sums do not fit (splits * M * N * 4 bytes, see mi355_fp8_blockwise_mm_plan) is rejected
+ *     with MI355_ERR_WORKSPACE; problems that need no split always pass.
+ *   - All calls on one GPU share that GPU's array: calls that may overlap in time on one GPU (different streams,
+ *     different threads) race on it and must be serialized by the caller.  Calls on one stream are ordered and safe.
+ *   - The device must be the current device of the calling thread.  The first call on a device looks up the array's
+ *     address (hipGetSymbolAddress); make that call outside graph capture.
+ */
+#define MI355_NOALLOC_SCRATCH_BYTES (32u << 20)
+int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                   int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                   int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo, void* stream);
+
+/*
  * Per-token x per-channel INT8 GEMM:  acc = sum_k a[m,k] * b[n,k] exactly in int32;
  *   out[m,n] = cast( f32(acc) * (sb[n] * sa[m]) + f32(bias[n]) ).
  * Replaces int8_scaled_mm (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; epilogue order of

@@ -17,6 +17,7 @@ ABI_VERSION = 1
 F32, F16, BF16, FP8_E4M3FN, I8, I32 = range(6)
 QUANT_DIV, QUANT_RCP, QUANT_MUL = range(3)
 SCALE_F32, SCALE_UE8M0_PACKED = range(2)
+NOALLOC_SCRATCH_BYTES = 32 << 20
 
 EXPORTS = (
     "mi355_qlinear_abi_version",
@@ -24,6 +25,7 @@ EXPORTS = (
     "mi355_group_quant_8bit",
     "mi355_fp8_blockwise_mm_workspace_bytes",
     "mi355_fp8_blockwise_mm",
+    "mi355_fp8_blockwise_mm_noalloc",
     "mi355_int8_scaled_mm_workspace_bytes",
     "mi355_int8_scaled_mm",
     "mi355_fp8_blockwise_mm_plan",
@@ -65,6 +67,8 @@ def lib() -> ctypes.CDLL:
     L.mi355_fp8_blockwise_mm_workspace_bytes.restype = sz
     L.mi355_fp8_blockwise_mm.argtypes = [vp, vp, vp, vp, vp, i32] + [i64] * 10 + [vp, sz, vp]
     L.mi355_fp8_blockwise_mm.restype = i32
+    L.mi355_fp8_blockwise_mm_noalloc.argtypes = [vp, vp, vp, vp, vp, i32] + [i64] * 10 + [vp]
+    L.mi355_fp8_blockwise_mm_noalloc.restype = i32
     L.mi355_int8_scaled_mm_workspace_bytes.argtypes = [i64, i64, i64]
     L.mi355_int8_scaled_mm_workspace_bytes.restype = sz
     L.mi355_int8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32] + [i64] * 6 + [vp, sz, vp]

@@ -88,7 +88,7 @@ __device__ __forceinline__ void issue_weights(const DecodeState& s, uint8_t* sta
     if constexpr (MANUAL) {
       const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)dst;
       asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.woff[j]), "s"(base), "s"(lds_addr)
-                   : "memory", "m0");
+                   : "memory");  // m0 cannot be named as a clobber (the compiler reserves it and rejects the entry); no compiler-managed use of m0 lies between these statements
     } else {
       __builtin_amdgcn_global_load_lds((gptr_t)(base + s.woff[j]), (lptr_t)dst, 16, 0, 0);
     }

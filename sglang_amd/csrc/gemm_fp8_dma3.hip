@@ -60,6 +60,8 @@ struct Dma3State {
 };
 
 // Load number i (< LOADS: tile rows; == LOADS: token scales) of K block kb, written as instructions.
+// The statements write m0; it cannot be listed as a clobber (the compiler reserves the register and rejects the entry), and
+// no compiler-managed use of m0 lies between them and the next statement that sets it.
 template <int BM>
 __device__ __forceinline__ void issue_one(const Dma3State<BM>& s, int i, uint8_t* stage, float* scale, int kb) {
   constexpr int LOADS = Dma3State<BM>::LOADS;
@@ -68,11 +70,11 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM>& s, int i, uint8_t
     const uint8_t* base = (i < BM / 64 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
     asm volatile("" : "+s"(base));
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
   } else {
     const float* src = s.sa_ptr + (int64_t)kb * s.sa_sk;
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(scale + s.wave * 64);
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds_addr) : "memory");
   }
 }
 

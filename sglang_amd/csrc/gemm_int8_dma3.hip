@@ -39,13 +39,14 @@ struct U8State {
   uint32_t tok_off[4], ch_off[4];  // per K sub-step: this lane's 16 bytes in the first token / channel tile
 };
 
+// Writes m0, which cannot be listed as a clobber (reserved register); no compiler-managed use of m0 lies in the K loop.
 template <int BM>
 __device__ __forceinline__ void issue_one(const U8State<BM>& s, int i, uint8_t* stage, int kb) {
   kb = min(kb, s.kb_last);
   const uint8_t* base = (i < BM / 64 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
   asm volatile("" : "+s"(base));
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
 }
 
 // One 128-byte K step out of `cur`; the loads of step kb_next go out in between, into `nxt`.

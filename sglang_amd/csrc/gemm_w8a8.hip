@@ -405,7 +405,6 @@ struct Route {
 Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, bool aligned) {
   Route r{};
   r.aligned = aligned;
-  const int kb_total = (int)((K + KSTEP - 1) / KSTEP);
   const bool small_b = N * ldb < (1ll << 32);                 // kernels that address rows by 32-bit byte offsets
   const bool small_offsets = M * lda < (1ll << 32) && small_b;
   if (decode_supported(M, N, K) && aligned && small_b) {  // barrier-free weight streaming
@@ -447,11 +446,15 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   return r;
 }
 
+bool operands_aligned(const GemmParams& p) {
+  return (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) &&
+         ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
+}
+
 template <bool IS_FP8>
 int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipStream_t stream, const char* what) {
   p.kb_total = (p.K + KSTEP - 1) / KSTEP;
-  const bool aligned = (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) &&
-                       ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) && ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
+  const bool aligned = operands_aligned(p);
   const Route r = choose_route(IS_FP8, p.M, p.N, p.K, p.lda, p.ldb, aligned);
   p.splits = r.splits;
   p.kb_per_split = r.kb_per_split;
@@ -512,23 +515,29 @@ extern "C" size_t mi355_fp8_blockwise_mm_workspace_bytes(int64_t M, int64_t N, i
   return workspace_bytes(M, N, K, true);
 }
 
-extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const float* sb, void* out,
-                                      int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-                                      int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo,
-                                      void* workspace, size_t workspace_bytes_given, void* stream) {
-  const char* what = "mi355_fp8_blockwise_mm";
+namespace {
+
+// Argument checks and parameter block shared by the two FP8 entry points.  Returns MI355_OK with `empty` set when there
+// is nothing to do.
+int fp8_mm_params(const char* what, const void* a, const void* b, const float* sa, const float* sb, void* out,
+                  int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t sa_sm, int64_t sa_sk,
+                  int64_t sb_sn, int64_t sb_sk, int64_t ldo, GemmParams& p, bool& empty) {
   clear_error();
+  empty = false;
   MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
   MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16 || out_dtype == MI355_F32,
                 MI355_ERR_INVALID_ARGUMENT, "%s: out_dtype must be bfloat16, float16 or float32", what);
-  if (M == 0 || N == 0) return MI355_OK;
+  if (M == 0 || N == 0) {
+    empty = true;
+    return MI355_OK;
+  }
   MI355_REQUIRE(K > 0, MI355_ERR_INVALID_ARGUMENT, "%s: K must be positive", what);
   MI355_REQUIRE(a && b && sa && sb && out, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
   MI355_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MI355_ERR_INVALID_ARGUMENT,
                 "%s: dimensions must fit in 31 bits", what);
   MI355_REQUIRE(lda >= K && ldb >= K && ldo >= N, MI355_ERR_INVALID_ARGUMENT,
                 "%s: row strides smaller than the row length", what);
-  GemmParams p{};
+  p = GemmParams{};
   p.a = static_cast<const uint8_t*>(a);
   p.b = static_cast<const uint8_t*>(b);
   p.sa = sa, p.sb = sb, p.bias = nullptr, p.out = out, p.ws = nullptr;
@@ -536,7 +545,77 @@ extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float*
   p.lda = lda, p.ldb = ldb, p.ldo = ldo;
   p.sa_sm = sa_sm, p.sa_sk = sa_sk, p.sb_sn = sb_sn, p.sb_sk = sb_sk;
   p.out_dtype = out_dtype;
+  return MI355_OK;
+}
+
+// ---- scratch of the entry point that allocates nothing.  One array per GPU (every device that loads this code object
+// holds its own copy at its own address); the name below is only a host-side handle, the device address comes from
+// hipGetSymbolAddress, once per device, and is what kernels and host calls are given.
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)MI355_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) uint8_t scratch[NOALLOC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES];  // guarded by scratch_mutex
+
+int scratch_of_current_device(void** ptr, const char* what) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    set_error("%s: cannot identify the current device (%s, device %d)", what, hipGetErrorString(e), dev);
+    return MI355_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("%s: cannot resolve the scratch array on device %d: %s", what, dev, hipGetErrorString(e));
+      return MI355_ERR_LAUNCH;
+    }
+    scratch_ptr[dev] = p;
+  }
+  *ptr = scratch_ptr[dev];
+  return MI355_OK;
+}
+
+}  // namespace
+
+extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                      int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                      int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo,
+                                      void* workspace, size_t workspace_bytes_given, void* stream) {
+  const char* what = "mi355_fp8_blockwise_mm";
+  GemmParams p;
+  bool empty;
+  const int rc = fp8_mm_params(what, a, b, sa, sb, out, out_dtype, M, N, K, lda, ldb, sa_sm, sa_sk, sb_sn, sb_sk, ldo, p, empty);
+  if (rc != MI355_OK || empty) return rc;
   return run_gemm<true>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
+}
+
+extern "C" int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                              int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                              int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo,
+                                              void* stream) {
+  const char* what = "mi355_fp8_blockwise_mm_noalloc";
+  GemmParams p;
+  bool empty;
+  int rc = fp8_mm_params(what, a, b, sa, sb, out, out_dtype, M, N, K, lda, ldb, sa_sm, sa_sk, sb_sn, sb_sk, ldo, p, empty);
+  if (rc != MI355_OK || empty) return rc;
+  // the same plan the launcher will make: how many partial-sum bytes it needs
+  const Route r = choose_route(true, p.M, p.N, p.K, p.lda, p.ldb, operands_aligned(p));
+  const size_t need = r.splits > 1 ? (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u : 0;
+  MI355_REQUIRE(need <= NOALLOC_SCRATCH_BYTES, MI355_ERR_WORKSPACE,
+                "%s: M=%lld N=%lld K=%lld needs %zu bytes of split-K partial sums, the built-in scratch holds %zu; use "
+                "mi355_fp8_blockwise_mm with a caller workspace",
+                what, (long long)M, (long long)N, (long long)K, need, NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0) {
+    rc = scratch_of_current_device(&ws, what);
+    if (rc != MI355_OK) return rc;
+  }
+  // every partial sum that the reduce kernel reads is written by this call first, so nothing has to be cleared
+  return run_gemm<true>(p, ws, need > 0 ? NOALLOC_SCRATCH_BYTES : 0, static_cast<hipStream_t>(stream), what);
 }
 
 extern "C" size_t mi355_int8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
