@@ -89,9 +89,13 @@ __device__ __forceinline__ TileCoord tile_of_block(int bid, int total, int tiles
 // Needs 16-byte aligned rows and K % 16 == 0.  Returns an MI355_* status.
 int launch_fp8_pipelined(GemmParams& p, hipStream_t stream, const char* what);
 
-// Large-M blockwise FP8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, two LDS stages); gemm_fp8_dma.hip.
-// Same requirements.
-int launch_fp8_dma(GemmParams& p, hipStream_t stream, const char* what);
+// Large-M blockwise FP8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases);
+// gemm_fp8_pp.hip.  Same requirements.
+int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what);
+// Its token scales must be M-major with a 16-byte friendly pitch; otherwise it copies them into p.ws first, which must
+// then hold fp8_pp_workspace_bytes(M, K) bytes.
+size_t fp8_pp_workspace_bytes(int64_t M, int64_t K);
+bool fp8_pp_scales_conform(const GemmParams& p);
 
 
 // Mid-M blockwise FP8 GEMM (64/128 x 256 tile, 8 waves, three LDS stages, hand-issued direct-to-LDS loads);

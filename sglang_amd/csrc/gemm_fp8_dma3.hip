@@ -12,8 +12,8 @@
 //   * nothing else in the loop counts in vmcnt (weight-block scales come by scalar loads);
 //   * the barrier is a bare s_barrier: LDS written by the loads is complete when vmcnt says so, and a stage is
 //     overwritten only after the barrier that follows its last read.
-// Operand roles, swizzle, chunk mapping, promotion FMA and the {MFMA of tile t, FMAs of tile t-1} step are those of
-// gemm_fp8_dma.hip.  Optional split along K (partials to the workspace, ordered reduce afterwards).
+// Operand roles, swizzle, chunk mapping and promotion FMA are those of gemm_w8a8.hip; a step is {MFMA of tile t, FMAs of
+// tile t-1}.  Optional split along K (partials to the workspace, ordered reduce afterwards).
 // Requires K % 128 == 0, 16-byte aligned rows, row offsets below 4 GiB.
 #include "gemm_common.h"
 

@@ -1,0 +1,385 @@
+// Large-M blockwise-scaled FP8 GEMM for gfx950: 256 x 256 macro tile, 8 waves, two-phase ("ping-pong") schedule.
+//
+// What the counters of a kernel that interleaves everything say: with the MFMAs, the promotion FMAs, the LDS operand
+// reads and the direct-to-LDS loads of the next K block mixed into one instruction stream per wave, the matrix pipe is
+// busy 53 % of the time.  Taking the loads out (nothing else changed) brings it to 94 %; making them hit in L2 or never
+// waiting for them changes little.  A wave issues in order, so whenever one of its vector-memory instructions has to wait
+// for a slot in the address path the MFMAs behind it wait too, and with two such waves per SIMD both are often stuck.
+//
+// So the two waves of a SIMD take turns.  Waves 0..3 (token rows 0..127 of the tile) and waves 4..7 (rows 128..255) sit
+// one per SIMD each; while one group runs a COMPUTE phase - sixteen MFMAs with their promotion FMAs, operands already in
+// registers, nothing else - the other runs a MEMORY phase: LDS operand reads for its next compute phase, the direct-to-LDS
+// loads of the next K block, scale fetches.  A workgroup barrier ends every phase; group 1 starts one phase late, so the
+// groups alternate and the matrix pipe of every SIMD always has exactly one wave feeding it.
+//
+// One K block (128 bytes of K) per wave = 32 MFMAs (v_mfma_f32_16x16x128_f8f6f4) = two compute phases of four token tiles
+// x four channel tiles, each preceded by a memory phase that copies its operands from LDS into registers:
+//   M0(k): weight fragments + token tiles 0..3 of block k -> registers        C0(k): 16 MFMAs / 64 FMAs
+//   M1(k): token tiles 4..7 -> registers                                       C1(k): 16 MFMAs / 64 FMAs
+// Because operands leave LDS a phase before they are used, a 64-row band of a stage is free again long before the block
+// is finished, and its successor (block k + 2, same stage) can be requested early.  Measured on this part: LDS reads a
+// wave issues behind its own direct-to-LDS loads return ~65 cycles later per load in front of them, so inside a memory
+// phase the LDS reads go first and the loads last.  Every wave fetches one 8-row slice of every band:
+//   set A(b) = token scales, the four channel bands, token rows 0..63 and 128..191 of block b: requested in M1(b - 2),
+//              when both groups have copied those rows of block b - 2 out (M0 phases); needed from M0(b) of group 0 on;
+//   set B(b) = token rows 64..127 and 192..255: requested in M0(b - 1), after the M1 phases that read them; needed
+//              from M1(b) of group 0 on.
+// Loads complete in order, so "set X has landed" is a constant count: at the end of every memory phase exactly nine
+// younger loads may still be in flight (s_waitcnt vmcnt(9)), and each set has four phases - a whole K block - to land.
+// Token scales: measured, ONE 4-byte-per-lane load per wave and K block (direct-to-LDS or to a register, whatever its
+// address or position in the stream) makes this kernel 1.5x slower, while 16-byte-per-lane loads stream freely.  So the
+// scales must be M-major (256 consecutive floats per tile and K block, the layout fp8_blockwise_scaled_mm prescribes),
+// and each wave fetches 32 of them with the first eight lanes of a 16-byte direct-to-LDS load; the launcher re-lays
+// other layouts out into the workspace first.  They use four small LDS stages so that they can travel with set A.
+// Loads, waits and barriers are written as instructions (the compiler would wait for all loads at every barrier).
+// Arithmetic, operand roles, LDS layout and swizzle are those of gemm_w8a8.hip.
+#include "gemm_common.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int G_THREADS = 512;
+constexpr int G_BM = 256, G_BN = 256, G_WM = 128, G_WN = 64;
+constexpr int G_MT = G_WM / 16, G_NT = G_WN / 16;  // 8 token tiles x 4 channel tiles per wave
+constexpr int G_HT = G_MT / 2;                     // token tiles per compute phase
+constexpr int G_ROWS = G_BM + G_BN;
+constexpr int G_LOADS = G_ROWS / 64;               // 8 direct-to-LDS tile loads per wave and K block
+constexpr int G_STAGE = G_ROWS * KSTEP;
+
+__shared__ __attribute__((aligned(1024))) uint8_t g_stage0[G_STAGE];
+__shared__ __attribute__((aligned(1024))) uint8_t g_stage1[G_STAGE];
+// token scales: four stages (block b in stage b % 4) of 256 floats
+__shared__ __attribute__((aligned(256))) float g_scale[4 * G_BM];
+
+__device__ __attribute__((aligned(16))) uint32_t g_zero16[4] = {0, 0, 0, 0};  // source of chunks past the end of K
+
+typedef __attribute__((address_space(3))) void* lptr_t;
+typedef const __attribute__((address_space(4))) float* cfloat_ptr;
+typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
+
+__device__ __forceinline__ u32x4 lds16(lds_cptr p, int imm) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(p + imm);
+}
+
+struct Frag {
+  u32x4 lo, hi;
+};
+__device__ __forceinline__ v8i as_v8i(const Frag& f) {
+  return v8i{(int)f.lo.x, (int)f.lo.y, (int)f.lo.z, (int)f.lo.w, (int)f.hi.x, (int)f.hi.y, (int)f.hi.z, (int)f.hi.w};
+}
+
+struct PpState {
+  const uint8_t* a_base;
+  const uint8_t* b_base;
+  uint32_t goff[G_LOADS];  // lane's byte offset from the matrix base (rows clamped); loads 0..3 token rows, 4..7 channel rows
+  int chunk_byte;          // 16 * logical chunk this lane fetches
+  const float* sa_base;    // token scales, M-major: element (m, kb) at sa_base[kb * sa_sk + m]
+  uint32_t sa_off;         // byte offset of the four scales this lane fetches (lanes 0..7), clamped to the last valid quad
+  cfloat_ptr sb_ptr;       // &sb[nb, 0] of this wave's 128-channel block
+  int64_t sa_sk, sb_sk;
+  int K, wave, kb_last;
+  uint32_t tok_off[2], ch_off[2], sc_off;
+};
+
+// Direct-to-LDS load number i (< 8) of K block kb (clamped to the last block): tile rows i * 64 + 8 * wave .. + 7 into
+// `stage`.  Written as instructions so that the compiler does not count them.  They write m0 (it cannot be named as a
+// clobber: reserved register); no compiler-managed use of m0 lies between these statements.
+template <bool KFULL>
+__device__ __forceinline__ void issue_one(const PpState& s, int i, uint8_t* stage, int kb) {
+  kb = min(kb, s.kb_last);
+  const uint8_t* base = (i < G_LOADS / 2 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
+  if constexpr (KFULL) {
+    asm volatile("" : "+s"(base));
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
+  } else {
+    // K ends inside the last block: chunks past the end come from a block of zeros (per-lane 64-bit addresses)
+    const uint8_t* src = base + s.goff[i];
+    if (kb * KSTEP + s.chunk_byte >= s.K) src = reinterpret_cast<const uint8_t*>(g_zero16);
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+  }
+}
+
+// The wave's 32 token scales of block b (tokens 32 * wave .. + 31 of the tile) into scale stage b % 4: lanes 0..7 fetch
+// 16 bytes each.  exec is narrowed and restored inside the statement.
+__device__ __forceinline__ void issue_scales(const PpState& s, int b) {
+  const float* base = s.sa_base + (int64_t)min(b, s.kb_last) * s.sa_sk;  // wave-uniform
+  asm volatile("" : "+s"(base));
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(g_scale + (b & 3) * G_BM + s.wave * 32);
+  uint64_t saved;
+  asm volatile(
+      "s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xff\n\ts_mov_b32 m0, %3\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+      : "=&s"(saved)
+      : "v"(s.sa_off), "s"(base), "s"(lds_addr)
+      : "memory");
+}
+
+// Set A of block b: scales, channel bands, token rows 0..63 and 128..191 (7 loads).  Set B: token rows 64..127, 192..255.
+constexpr int SET_A = 7, SET_B = 2;
+template <bool KFULL>
+__device__ __forceinline__ void issue_set_a(const PpState& s, uint8_t* stage, int b) {
+  issue_scales(s, b);
+#pragma unroll
+  for (int i = 4; i < 8; ++i) issue_one<KFULL>(s, i, stage, b);
+  issue_one<KFULL>(s, 0, stage, b);
+  issue_one<KFULL>(s, 2, stage, b);
+}
+template <bool KFULL>
+__device__ __forceinline__ void issue_set_b(const PpState& s, uint8_t* stage, int b) {
+  issue_one<KFULL>(s, 1, stage, b);
+  issue_one<KFULL>(s, 3, stage, b);
+}
+
+// End of a compute phase.
+__device__ __forceinline__ void compute_end() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// End of a memory phase: its LDS reads have returned (the compute phase that follows must not start with a wait) and
+// all but the nine youngest of this wave's loads have landed.
+__device__ __forceinline__ void memory_end() {
+  static_assert(SET_A + SET_B == 9, "the wait is written for nine loads per K block");
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// Memory phase, operand part: token tiles 4 * HALF .. + 3 of `cur` (and, for HALF == 0, the four weight fragments)
+// into registers; their scales times the weight-block scale.
+template <int HALF>
+__device__ __forceinline__ void read_operands(const PpState& s, const uint8_t* cur, const float* sc_cur, float sbv,
+                                              Frag (&w)[G_NT], Frag (&tok)[G_HT], float (&scb)[G_HT]) {
+  const lds_cptr ch0 = (lds_cptr)cur + s.ch_off[0], ch1 = (lds_cptr)cur + s.ch_off[1];
+  const lds_cptr tk0 = (lds_cptr)cur + s.tok_off[0], tk1 = (lds_cptr)cur + s.tok_off[1];
+  const float* scp = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(sc_cur) + s.sc_off);
+  if constexpr (HALF == 0) {
+#pragma unroll
+    for (int i = 0; i < G_NT; ++i) {
+      w[i].lo = lds16(ch0, i * 2048);
+      w[i].hi = lds16(ch1, i * 2048);
+    }
+  }
+#pragma unroll
+  for (int jj = 0; jj < G_HT; ++jj) {
+    tok[jj].lo = lds16(tk0, (HALF * G_HT + jj) * 2048);
+    tok[jj].hi = lds16(tk1, (HALF * G_HT + jj) * 2048);
+  }
+#pragma unroll
+  for (int jj = 0; jj < G_HT; ++jj) scb[jj] = scp[(HALF * G_HT + jj) * 16] * sbv;
+}
+
+// The promotion of the last MFMA of a compute phase is left to the start of the wave's next memory phase (the other
+// group's MFMAs already own the pipe by then), so a compute phase does not end on a wait for its own last result.
+struct Pending {
+  v4f part;
+  float scale;
+};
+
+template <int HALF>
+__device__ __forceinline__ void retire(const Pending& pd, float (&acc)[G_NT][G_MT][4]) {
+#pragma unroll
+  for (int v = 0; v < 4; ++v)
+    acc[G_NT - 1][HALF * G_HT + G_HT - 1][v] = fmaf(pd.part[v], pd.scale, acc[G_NT - 1][HALF * G_HT + G_HT - 1][v]);
+}
+
+// Compute phase: 16 steps of {MFMA of tile t, promotion FMAs of tile t - 2}.  The FMAs lag by two MFMAs (three result
+// buffers), so they never wait for a result that is still in the pipe (measured 3.5 % faster than a lag of one).
+template <int HALF>
+__device__ __forceinline__ void compute(const Frag (&w)[G_NT], const Frag (&tok)[G_HT], const float (&scb)[G_HT],
+                                        float (&acc)[G_NT][G_MT][4], Pending& pd) {
+  constexpr int STEPS = G_HT * G_NT;
+  v4f part[3];
+#pragma unroll
+  for (int t = 0; t < STEPS + 1; ++t) {
+    if (t < STEPS) {
+      const int jj = t >> 2, i = t & 3;
+      part[t % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w[i]), as_v8i(tok[jj]), v4f{0.f, 0.f, 0.f, 0.f},
+                                                                     0, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first; the FMAs run in its shadow
+    }
+    if (t > 1) {
+      const int pj = (t - 2) >> 2, pi = (t - 2) & 3;
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        acc[pi][HALF * G_HT + pj][v] = fmaf(part[(t - 2) % 3][v], scb[pj], acc[pi][HALF * G_HT + pj][v]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  pd.part = part[(STEPS - 1) % 3];
+  pd.scale = scb[G_HT - 1];
+}
+
+template <bool KFULL>
+__global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams p) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2;  // 0: starts computing first; 1: one phase behind.  Also the wave's token half of the tile.
+  const int wave_n = wave & 3;
+  const int l16 = lane & 15, q = lane >> 4;
+
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
+  const int m0 = tc.tile_m * G_BM, n0 = tc.tile_n * G_BN;
+  const int nkb = p.kb_total;
+
+  PpState s;
+  s.K = p.K;
+  s.wave = wave;
+  s.kb_last = nkb - 1;
+  s.a_base = p.a;
+  s.b_base = p.b;
+  {
+    // lane l of a wave lands in row l / 8, physical chunk l % 8 of the 8 rows one load fills; it fetches the logical
+    // chunk that belongs there under the (row & 7) swizzle
+    const int lrow = lane >> 3;
+    s.chunk_byte = ((lane & 7) ^ lrow) * 16;
+#pragma unroll
+    for (int i = 0; i < G_LOADS; ++i) {
+      const int row = i * 64 + wave * 8 + lrow;
+      if (row < G_BM)
+        s.goff[i] = (uint32_t)((int64_t)min(m0 + row, p.M - 1) * p.lda + s.chunk_byte);
+      else
+        s.goff[i] = (uint32_t)((int64_t)min(n0 + row - G_BM, p.N - 1) * p.ldb + s.chunk_byte);
+    }
+    const int trow = grp * G_WM + l16, crow = G_BM + wave_n * G_WN + l16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      s.tok_off[h] = trow * KSTEP + (((q + 4 * h) ^ (trow & 7)) << 4);
+      s.ch_off[h] = crow * KSTEP + (((q + 4 * h) ^ (crow & 7)) << 4);
+    }
+    s.sc_off = (grp * G_WM + l16) * 4;
+  }
+  s.sa_base = p.sa;
+  s.sa_off = (uint32_t)min(m0 + wave * 32 + (lane & 7) * 4, (p.M - 1) & ~3) * 4u;  // quads past M refetch the last one
+  s.sa_sk = p.sa_sk;
+  s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * G_WN, p.N - 1) / 128) * p.sb_sn);
+  s.sb_sk = p.sb_sk;
+
+  float acc[G_NT][G_MT][4];
+#pragma unroll
+  for (int i = 0; i < G_NT; ++i)
+#pragma unroll
+    for (int j = 0; j < G_MT; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+  Frag w[G_NT], tok[G_HT];
+  float scb[G_HT];
+  Pending pd;
+  pd.part = v4f{0.f, 0.f, 0.f, 0.f};
+  pd.scale = 0.f;
+
+  // ---- prologue: all of block 0 and set A of block 1
+  issue_set_a<KFULL>(s, g_stage0, 0);
+  issue_set_b<KFULL>(s, g_stage0, 0);
+  issue_set_a<KFULL>(s, g_stage1, 1);
+  float sb_cur = s.sb_ptr[0];
+  asm volatile("s_waitcnt vmcnt(7)\n\ts_barrier" ::: "memory");  // block 0 is in LDS (set A of block 1 may be in flight)
+  if (grp == 1) compute_end();  // group 1 runs one phase behind group 0
+
+  // One K block: M0, C0, M1, C1.  `cur` holds block kb; `nxt` takes set B of block kb + 1, `cur` set A of block kb + 2.
+  auto k_block = [&](uint8_t* cur, uint8_t* nxt, int kb, float sbv) {
+    const float* sc_cur = g_scale + (kb & 3) * G_BM;
+    retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
+    read_operands<0>(s, cur, sc_cur, sbv, w, tok, scb);
+    issue_set_b<KFULL>(s, nxt, kb + 1);
+    memory_end();
+    compute<0>(w, tok, scb, acc, pd);
+    compute_end();
+    retire<0>(pd, acc);
+    read_operands<1>(s, cur, sc_cur, sbv, w, tok, scb);
+    issue_set_a<KFULL>(s, cur, kb + 2);
+    memory_end();
+    compute<1>(w, tok, scb, acc, pd);
+    compute_end();
+  };
+
+  int kb = 0;
+  for (; kb + 1 < nkb; kb += 2) {
+    const float sb_1 = s.sb_ptr[(int64_t)(kb + 1) * s.sb_sk];
+    const float sb_2 = s.sb_ptr[(int64_t)min(kb + 2, nkb - 1) * s.sb_sk];
+    k_block(g_stage0, g_stage1, kb, sb_cur);
+    k_block(g_stage1, g_stage0, kb + 1, sb_1);
+    sb_cur = sb_2;
+  }
+  if (kb < nkb) k_block(g_stage0, g_stage1, kb, sb_cur);
+  retire<1>(pd, acc);
+  if (grp == 0) compute_end();  // as many barriers as group 1
+  // the last requests refetch the last block into rows nobody reads any more: they must not outlive the workgroup's LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  // ---- epilogue: lane holds channels n .. n+3 of token m
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+#pragma unroll
+  for (int j = 0; j < G_MT; ++j) {
+    const int m = m0 + grp * G_WM + j * 16 + l16;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int i = 0; i < G_NT; ++i) {
+      const int n = n0 + wave_n * G_WN + i * 16 + 4 * q;
+      if (n >= p.N) continue;
+      store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], min(4, p.N - n), vec_ok);
+    }
+  }
+}
+
+
+
+// out[kb * ld_out + m] = sa[m * sa_sm + kb * sa_sk]: token scales re-laid out M-major with a row pitch that is a multiple
+// of four floats.  One 32 x 32 tile per workgroup through LDS, so that reads and writes are both contiguous for either
+// input layout.
+__global__ __launch_bounds__(256) void relayout_scales_kernel(const float* sa, int64_t sa_sm, int64_t sa_sk, float* out,
+                                                              int64_t ld_out, int M, int KB) {
+  __shared__ float tile[32][33];
+  const int m0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const bool k_fast = sa_sk < sa_sm;                       // which index is contiguous in the input
+#pragma unroll
+  for (int r = ty; r < 32; r += 8) {
+    const int m = k_fast ? m0 + r : m0 + tx, kb = k_fast ? k0 + tx : k0 + r;
+    if (m < M && kb < KB) tile[kb - k0][m - m0] = sa[(int64_t)m * sa_sm + (int64_t)kb * sa_sk];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = ty; r < 32; r += 8) {
+    const int m = m0 + tx, kb = k0 + r;
+    if (m < M && kb < KB) out[(int64_t)kb * ld_out + m] = tile[r][tx];
+  }
+}
+
+}  // namespace
+
+// The kernel reads token scales M-major with 16-byte loads.  Scales that are not laid out that way (K-major, as
+// per_token_group_quant_fp8 returns them by default; a pitch or base that is not a multiple of 16 bytes) are first copied
+// into the workspace.
+size_t fp8_pp_workspace_bytes(int64_t M, int64_t K) { return (size_t)((M + 3) & ~3ll) * (size_t)((K + KSTEP - 1) / KSTEP) * 4u; }
+
+bool fp8_pp_scales_conform(const GemmParams& p) {
+  return p.sa_sm == 1 && (p.sa_sk & 3) == 0 && p.sa_sk >= ((p.M + 3) & ~3) && (reinterpret_cast<uintptr_t>(p.sa) & 15) == 0;
+}
+
+// Needs 16-byte aligned rows and row offsets below 4 GiB; p.ws must hold fp8_pp_workspace_bytes() when the scales do not
+// conform.
+int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what) {
+  p.tiles_m = (p.M + G_BM - 1) / G_BM;
+  p.tiles_n = (p.N + G_BN - 1) / G_BN;
+  if (!fp8_pp_scales_conform(p)) {
+    float* dst = static_cast<float*>(p.ws);
+    const int64_t ld = (p.M + 3) & ~3;
+    hipLaunchKernelGGL(relayout_scales_kernel, dim3((unsigned)((p.M + 31) / 32), (unsigned)((p.kb_total + 31) / 32)), dim3(256), 0,
+                       stream, p.sa, p.sa_sm, p.sa_sk, dst, ld, p.M, p.kb_total);
+    const int rc = check_launch(what);
+    if (rc != MI355_OK) return rc;
+    p.sa = dst, p.sa_sm = 1, p.sa_sk = ld;
+  }
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  if (p.K % KSTEP == 0)
+    hipLaunchKernelGGL(fp8_gemm_pp_kernel<true>, grid, dim3(G_THREADS), 0, stream, p);
+  else
+    hipLaunchKernelGGL(fp8_gemm_pp_kernel<false>, grid, dim3(G_THREADS), 0, stream, p);
+  return check_launch(what);
+}
+
+}  // namespace mi355

@@ -1,8 +1,8 @@
 // Large-M per-token x per-channel INT8 GEMM for gfx950: 256 x 256 macro tile, 8 waves (two per SIMD) of 128 x 64,
 // direct-to-LDS loads, v_mfma_i32_32x32x32_i8.
 //
-// The skeleton is the one of gemm_fp8_dma.hip (two static 64 KB LDS stages filled by global_load_lds_dwordx4, one barrier
-// per 128-byte K step, loads of the next step interleaved with the MFMAs).  Differences:
+// Two static 64 KB LDS stages filled by global_load_lds_dwordx4, one barrier per 128-byte K step, loads of the next step
+// interleaved with the MFMAs.  Compared with the FP8 kernels:
 //   * the int8 instruction with the full rate on this part is the 32x32x32 one (measured 3.4 POP/s against 2.1 POP/s
 //     for 16x16x64), so a wave's 128 x 64 tile is 4 x 2 tiles of 32 x 32 and a K step is four MFMAs per tile;
 //   * accumulation is exact int32 inside the MFMA; there are no per-block scales and no promotion FMAs;

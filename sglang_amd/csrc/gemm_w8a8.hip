@@ -352,6 +352,10 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
     const size_t dneed = ds > 1 ? (size_t)ds * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
   }
+  if (is_fp8 && M > 1024) {  // the large-M kernel may have to re-lay the token scales out
+    const size_t sneed = fp8_pp_workspace_bytes(M, K);
+    if (sneed > need) need = sneed;
+  }
   return need;
 }
 
@@ -390,8 +394,8 @@ int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* wha
 
 // Which kernel serves a problem, with which tiling.  One function decides for the launcher and for the plan query, so
 // what the query reports is what runs.
-enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_DMA256, RK_PIPELINED, RK_INT8_DMA256, RK_GENERIC };
-const char* const ROUTE_NAMES[] = {"decode", "dma3", "dma256", "pipelined", "int8_dma256", "generic"};
+enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_PINGPONG, RK_PIPELINED, RK_INT8_DMA256, RK_GENERIC };
+const char* const ROUTE_NAMES[] = {"decode", "dma3", "pingpong", "pipelined", "int8_dma256", "generic"};
 
 struct Route {
   int kernel;
@@ -428,9 +432,9 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   const int64_t tiles_128 = ((M + 255) / 256) * ((N + 127) / 128);
   if (pl.bm == 256 && pl.splits == 1 && aligned && small_offsets) {
     if (is_fp8) {
-      // 256 x 256 tiles (8 waves, direct-to-LDS) when they still give every CU a workgroup, else 256 x 128
+      // 256 x 256 tiles (8 waves in two alternating groups) when they still give every CU a workgroup, else 256 x 128
       if (tiles_256 >= NUM_CUS) {
-        r.kernel = RK_DMA256, r.bn = 256;
+        r.kernel = RK_PINGPONG, r.bn = 256;
         return r;
       }
       if (tiles_128 >= NUM_CUS) {
@@ -446,6 +450,13 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   return r;
 }
 
+// Workspace bytes the chosen route needs for this call: split-K partial sums, or a re-laid-out copy of the token scales.
+size_t route_workspace_need(bool is_fp8, const Route& r, const GemmParams& p) {
+  if (r.splits > 1) return (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u;
+  if (is_fp8 && r.kernel == RK_PINGPONG && !fp8_pp_scales_conform(p)) return fp8_pp_workspace_bytes(p.M, p.K);
+  return 0;
+}
+
 bool operands_aligned(const GemmParams& p) {
   return (p.K % 16 == 0) && (p.lda % 16 == 0) && (p.ldb % 16 == 0) && ((reinterpret_cast<uintptr_t>(p.a) & 15) == 0) &&
          ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
@@ -458,8 +469,8 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
   const Route r = choose_route(IS_FP8, p.M, p.N, p.K, p.lda, p.ldb, aligned);
   p.splits = r.splits;
   p.kb_per_split = r.kb_per_split;
-  if (r.splits > 1) {
-    const size_t need = (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u;
+  const size_t need = route_workspace_need(IS_FP8, r, p);
+  if (need > 0) {
     MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
                   "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
     MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
@@ -474,7 +485,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
     case RK_DMA3:
       rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, stream, what) : launch_int8_dma3(p, r.bm, stream, what);
       break;
-    case RK_DMA256: return launch_fp8_dma(p, stream, what);
+    case RK_PINGPONG: return launch_fp8_pp(p, stream, what);
     case RK_PIPELINED: return launch_fp8_pipelined(p, stream, what);
     case RK_INT8_DMA256: return launch_int8_dma(p, stream, what);
     default:
@@ -604,9 +615,9 @@ extern "C" int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, cons
   if (rc != MI355_OK || empty) return rc;
   // the same plan the launcher will make: how many partial-sum bytes it needs
   const Route r = choose_route(true, p.M, p.N, p.K, p.lda, p.ldb, operands_aligned(p));
-  const size_t need = r.splits > 1 ? (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u : 0;
+  const size_t need = route_workspace_need(true, r, p);
   MI355_REQUIRE(need <= NOALLOC_SCRATCH_BYTES, MI355_ERR_WORKSPACE,
-                "%s: M=%lld N=%lld K=%lld needs %zu bytes of split-K partial sums, the built-in scratch holds %zu; use "
+                "%s: M=%lld N=%lld K=%lld needs %zu bytes of scratch (split-K partial sums), the built-in scratch holds %zu; use "
                 "mi355_fp8_blockwise_mm with a caller workspace",
                 what, (long long)M, (long long)N, (long long)K, need, NOALLOC_SCRATCH_BYTES);
   void* ws = nullptr;

@@ -15,7 +15,7 @@ FP8_ROUTE_SHAPES = [
     # three-stage mid-M kernel: 64 / 128 token tiles, whole-K and split, ragged M, K blocks per range = 1, 2, 0 mod 3
     (48, 16384, 2048), (33, 16384, 2176), (40, 65536, 512), (200, 16384, 2048), (100, 32768, 640), (130, 8192, 7168),
     (250, 8192, 7296),
-    # 256 x 256 direct-to-LDS and 256 x 128 pipelined kernels, K a multiple of 128 and not
+    # 256 x 256 two-phase and 256 x 128 pipelined kernels, K a multiple of 128 and not
     (4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 512), (4000, 2100, 272),
     # generic kernel: every token-tile height, aligned and byte-granular loads, whole-K and split
     (7, 1088, 512), (16, 576, 7168), (1, 1088, 3884), (17, 384, 2304), (20, 256, 264), (33, 512, 512), (64, 128, 3884),
@@ -26,7 +26,7 @@ FP8_REQUIRED_VARIANTS = {
     ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
     ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
-    ("dma256", "kfull"), ("dma256", "ktail"), ("pipelined", "kfull"), ("pipelined", "ktail"),
+    ("pingpong", "kfull"), ("pingpong", "ktail"), ("pipelined", "kfull"), ("pipelined", "ktail"),
     ("generic", 16, "aligned", "whole"), ("generic", 16, "aligned", "split"), ("generic", 16, "bytes", "split"),
     ("generic", 32, "aligned", "split"), ("generic", 32, "bytes", "whole"),
     ("generic", 64, "aligned", "whole"), ("generic", 64, "bytes", "whole"), ("generic", 64, "bytes", "split"),
@@ -70,7 +70,7 @@ def variant_of(plan: dict, K: int):
         return (k, sp, f"gpw{g}" if g < 3 else "gpw3+")
     if k == "dma3":
         return (k, plan["bm"], sp)
-    if k in ("dma256", "pipelined"):
+    if k in ("pingpong", "pipelined"):
         return (k, "kfull" if K % 128 == 0 else "ktail")
     if k == "int8_dma256":
         return (k,)
