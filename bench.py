@@ -3,24 +3,26 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--quick]
 
-Prints ONE JSON line.  A "step" is one pass of the hot path over one batch of seeded synthetic
-input that is already resident in HBM; operands rotate over several buffers so that
-bandwidth-bound steps stream from HBM rather than from the 256 MB Infinity Cache.
+Prints ONE JSON line (kept short: every number has four significant digits).  A "step" is one pass of
+the hot path over one batch of seeded synthetic input that is already resident in HBM; weights rotate
+over several buffers so that bandwidth-bound steps stream from HBM rather than from the 256 MB
+Infinity Cache.
 
 --workload:
-  fp8_gemm   (headline, default) blockwise-FP8 GEMM, M=4096, DeepSeek-V3 gate_up K=7168 -> N=36864
-  quant      per-token-group FP8 quantization, M=16384 K=7168 g=128, row-major fp32 scales
-  quant_ue8m0  the same with column-major packed UE8M0 scales
-  copy       a plain 256 MiB device copy (calibration of the HBM traffic counters)
-  fp8_decode blockwise-FP8 GEMM at M=1 on gate_up (weight streaming)
-  int8_gemm  INT8 GEMM at M=4096 on Llama-3-8B gate_up (K=4096 -> N=28672)
-  all        (what the default run does) headline as `value`, every other configuration the
-             baseline names under "also": both quantizer variants, the M=4096 MLP/MLA shapes,
-             the decode shapes M in {1,8,32,128}, the single linear, and the INT8 GEMM shapes.
+  all          (default) headline = blockwise-FP8 GEMM, M=4096, DeepSeek-V3 gate_up K=7168 -> N=36864, as
+               `value`; every other configuration the baseline names as short rows under "also"; the
+               two quantizer rows (M=16384, K=7168) under "quant", last in the line
+  fp8_gemm     the headline alone          quant / quant_ue8m0   one quantizer variant alone
+  fp8_decode   FP8 gate_up at M=1          int8_gemm             INT8 gate_up (K=4096 -> N=28672) at M=4096
+  fp8:M:K:N    any blockwise-FP8 linear    int8:M:K:N            any INT8 linear
+  copy         a plain 256 MiB device copy (calibration of the HBM traffic counters)
 
-`roofline.achieved` = algorithmic FLOPs (2*M*N*K) or bytes per launch / average launch duration
-measured with HIP events on the launch stream.  `cpu_baseline` times the CPU oracle on a bounded
-sample of the same workload on this host's cores.
+Per-launch durations are HIP events on the launch stream (torch's current stream, which is the stream
+handed to the C ABI).  `roofline.achieved` = algorithmic FLOPs (2*M*N*K) or bytes per launch / MEDIAN
+launch duration; `b2b_ms` is the average over the same launches queued back to back between one event
+pair (no per-launch event overhead; for kernels of tens of microseconds it also hides the tail of one
+launch behind the head of the next).  `cpu_baseline` times the CPU oracle on a bounded sample of the
+same workload on this host's cores.
 """
 from __future__ import annotations
 
@@ -40,40 +42,35 @@ FP8_PEAK_TFLOPS = 5000.0  # dense fp8 MFMA, no sparsity
 INT8_PEAK_TOPS = 5000.0   # dense int8 MFMA
 
 METRIC = "blockwise-FP8 GEMM TFLOPS & %MFMA peak; quant GB/s & %HBM peak (1 GPU)"
+DATA = ("synthetic, seeded, resident in HBM before the timed region; activations bf16 N(0,1) + 0.1% x50 outliers quantized "
+        "1x128 by the GPU quantizer; FP8 weights N(0,0.02) quantized per 128x128 block (drawn on the device); INT8 operands "
+        "uniform in [-127,127]")
 
 
-def _time_launches(fn, nbuf, steps, warmup, graph=False):
-    """fn(i % nbuf) is launched warmup + steps times on the current stream.  Returns the wall seconds of
-    the timed steps (synchronize on both sides) and the per-launch milliseconds from HIP events.
+def r4(x):
+    """Four significant digits (keeps the JSON line short)."""
+    if isinstance(x, float):
+        return float(f"{x:.4g}")
+    if isinstance(x, dict):
+        return {k: r4(v) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [r4(v) for v in x]
+    return x
 
-    graph=True: each fn(i) is captured once into a HIP graph and the graphs are replayed, the way a serving loop runs
-    decode-sized steps; otherwise microsecond kernels would be timed together with the Python launch overhead."""
+
+def _time_launches(fn, nbuf, steps, warmup):
+    """fn(i % nbuf) is launched warmup + steps times on the current stream.  Returns (wall seconds of the timed
+    steps, per-launch milliseconds from HIP events, back-to-back average milliseconds)."""
     import torch
 
-    if graph:
-        stream = torch.cuda.Stream()
-        graphs = []
-        with torch.cuda.stream(stream):
-            for i in range(nbuf):
-                fn(i)  # warm up allocator and lazy initialisation outside capture
-            stream.synchronize()
-            for i in range(nbuf):
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g, stream=stream):
-                    fn(i)
-                graphs.append(g)
-        torch.cuda.synchronize()
-        run = lambda i: graphs[i].replay()
-    else:
-        run = fn
     for i in range(warmup):
-        run(i % nbuf)
+        fn(i % nbuf)
     torch.cuda.synchronize()
     # short kernels: keep warming up until ~30 ms of launches have run, so that clocks are up before the timed steps
     t_w = time.perf_counter()
     extra = 0
     while time.perf_counter() - t_w < 0.03 and extra < 2000:
-        run(extra % nbuf)
+        fn(extra % nbuf)
         extra += 1
         if extra % 32 == 0:
             torch.cuda.synchronize()
@@ -82,29 +79,22 @@ def _time_launches(fn, nbuf, steps, warmup, graph=False):
     t0 = time.perf_counter()
     for i in range(steps):
         evs[i][0].record()
-        run(i % nbuf)
+        fn(i % nbuf)
         evs[i][1].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    # a second pass of the same launches with ONE event pair around all of them: the per-launch event records of the
-    # pass above cost a few microseconds each, which matters for 50 us kernels; this is the average launch duration
-    global _last_region_ms
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for i in range(steps):
-        run(i % nbuf)
+        fn(i % nbuf)
     e1.record()
     torch.cuda.synchronize()
-    _last_region_ms = e0.elapsed_time(e1)
-    return wall, [a.elapsed_time(b) for a, b in evs]
+    return wall, [a.elapsed_time(b) for a, b in evs], e0.elapsed_time(e1) / steps
 
 
-_last_region_ms = 0.0
-
-
-def _stats(ms):
+def _stats(ms, b2b):
     s = sorted(ms)
-    return {"avg": sum(ms) / len(ms), "median": statistics.median(ms), "p20_p80": [s[len(s) // 5], s[len(s) * 4 // 5]]}
+    return {"median": statistics.median(ms), "p20_p80": [s[len(s) // 5], s[len(s) * 4 // 5]], "b2b": b2b}
 
 
 def _cpu_time_boxed(fn, seconds=10.0):
@@ -117,12 +107,23 @@ def _cpu_time_boxed(fn, seconds=10.0):
     return (time.perf_counter() - t0) / reps, reps
 
 
+def _roofline(flops, nbytes, ms, peak_ops, unit_ops):
+    """Which roof binds (time at peak MFMA rate vs time at peak HBM rate) and the achieved fraction of it."""
+    if flops / (peak_ops * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9):
+        a = flops / (ms * 1e-3) / 1e12
+        return {"bound": "mfma", "achieved": a, "peak": peak_ops, "unit": unit_ops, "frac": a / peak_ops, "traffic": None,
+                "per_launch": flops}
+    a = nbytes / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS, "traffic": None,
+            "per_launch": nbytes}
+
+
 # ------------------------------------------------------------------------------------------ quantizer
 
 def bench_quant(steps, warmup, ue8m0, with_cpu):
     import torch
 
-    from sglang_amd import fp8_kernel
+    from sglang_amd import _lib, fp8_kernel
     from sglang_amd.sgl_kernel import sgl_per_token_group_quant_fp8
     from sglang_amd.workloads import make_activation, quant_algorithmic_bytes
 
@@ -140,8 +141,6 @@ def bench_quant(steps, warmup, ue8m0, with_cpu):
     # one check through the reference-named entry point, then the timed loop calls the C ABI directly with the same
     # arguments: a 60 us kernel must not be timed together with the Python operator dispatch
     sgl_per_token_group_quant_fp8(xs[0], qs[0], ss[0], G, 1e-10, -448.0, 448.0, ue8m0, enable_v2=ue8m0)
-    from sglang_amd import _lib
-
     L = _lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
     if ue8m0:  # v2 arithmetic (q = x * 448/amax), packed exponents, words column-major
@@ -154,18 +153,15 @@ def bench_quant(steps, warmup, ue8m0, with_cpu):
     def step(i):
         _lib.check(L.mi355_group_quant_8bit(*args[i]))
 
-    wall, ms = _time_launches(step, nbuf, steps, warmup)
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
     alg = quant_algorithmic_bytes(M, K, G, 2, ue8m0)
-    st = _stats(ms)
-    st["avg"] = _last_region_ms / steps  # back-to-back launches: HIP-event time of the whole region / launches
+    st = _stats(ms, b2b)
     rec = {
-        "workload": ("quant_ue8m0" if ue8m0 else "quant") + f" M={M} K={K} g={G} bf16->e4m3fn, "
-        + ("column-major packed UE8M0 scales (q = x * 448/amax)" if ue8m0 else "row-major fp32 scales (q = x / s)"),
+        "workload": f"group quant M={M} K={K} g={G} bf16->e4m3fn, "
+        + ("column-major packed UE8M0 scales (q = x*448/amax)" if ue8m0 else "row-major fp32 scales (q = x/s)"),
         "value": alg / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
-        "dtype": "f32 arithmetic on bf16 input, e4m3fn output",
-        "roofline": {"bound": "hbm", "achieved": alg / (st["avg"] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": alg / (st["avg"] * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_launch": alg},
+        "dtype": "f32 on bf16 in, e4m3fn out",
+        "roofline": _roofline(0, alg, st["median"], FP8_PEAK_TFLOPS, "TFLOP/s"),
     }
     if with_cpu:
         from oracle import oracle
@@ -177,37 +173,49 @@ def bench_quant(steps, warmup, ue8m0, with_cpu):
         rec["cpu_baseline"] = {
             "value": quant_algorithmic_bytes(rows, K, G, 2, ue8m0) / dt / 1e9, "unit": "GB/s",
             "cores": oracle.num_threads(), "kind": "port",
-            "sample": f"first {rows} of {M} rows, {reps} repetitions in ~10 s, C oracle with OpenMP",
+            "sample": f"first {rows} of {M} rows, {reps} reps in ~10 s, C oracle with OpenMP",
         }
     return rec
 
 
 # ------------------------------------------------------------------------------------------ FP8 GEMM
 
-def _device_fp8_codes(shape, gen, dev):
+def device_block_fp8_weight(N, K, gen, dev):
+    """N(0, 0.02) weights quantized per 128x128 block on the device (same arithmetic as workloads.block_cast_to_fp8):
+    (e4m3fn [N, K], fp32 scales [ceil(N/128), ceil(K/128)]).  Rows are drawn in slabs to bound the fp32 scratch."""
     import torch
 
-    c = torch.randint(0, 256, shape, dtype=torch.uint8, device=dev, generator=gen)
-    return torch.where((c & 0x7F) == 0x7F, c & 0xF7, c).view(torch.float8_e4m3fn)  # no NaN codes
+    from sglang_amd.workloads import cdiv
+
+    Kp = cdiv(K, 128) * 128
+    q = torch.empty(N, K, dtype=torch.float8_e4m3fn, device=dev)
+    s = torch.empty(cdiv(N, 128), cdiv(K, 128), dtype=torch.float32, device=dev)
+    slab = 128 * 32
+    for n0 in range(0, N, slab):
+        n1 = min(N, n0 + slab)
+        rows = cdiv(n1 - n0, 128) * 128
+        w = torch.zeros(rows, Kp, dtype=torch.float32, device=dev)
+        w[: n1 - n0, :K] = torch.randn(n1 - n0, K, generator=gen, device=dev) * 0.02
+        v = w.view(rows // 128, 128, Kp // 128, 128)
+        amax = v.abs().amax(dim=(1, 3), keepdim=True).clamp(min=1e-4)
+        q[n0:n1] = (v * (448.0 / amax)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(rows, Kp)[: n1 - n0, :K]
+        s[n0 // 128: n0 // 128 + rows // 128] = (amax / 448.0).view(rows // 128, Kp // 128)
+    return q, s
 
 
-def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
-    """One blockwise-FP8 linear through sgl_kernel.fp8_blockwise_scaled_mm (or, for N not a multiple of
-    128, through w8a8_block_fp8_matmul).  Activations are N(0,1)+outliers quantized by the GPU quantizer;
-    weights are random finite e4m3fn codes with block scales around 2e-4 (drawn on the device: the value
-    distribution does not change the timing, and drawing 2.6e8 Gaussians on the host would dominate the run)."""
+def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu, w8a16_cpu=False):
+    """One blockwise-FP8 linear through sgl_kernel.fp8_blockwise_scaled_mm (or, for N or K not a multiple of 128,
+    through w8a8_block_fp8_matmul)."""
     import torch
 
-    from sglang_amd import fp8_kernel, sgl_kernel
+    from sglang_amd import _lib, fp8_kernel, sgl_kernel
     from sglang_amd.workloads import cdiv, fp8_gemm_algorithmic_bytes, gemm_flops, make_activation
 
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev)
     gen.manual_seed(N * 10007 + K)
-    wbytes = N * K
-    nbuf = max(2, min(6, int(600e6 // wbytes) + 1))  # rotate through > 512 MB of weights when they are small
-    ws = [_device_fp8_codes((N, K), gen, dev) for _ in range(nbuf)]
-    wss = [(torch.rand(cdiv(N, 128), cdiv(K, 128), device=dev, generator=gen) + 0.5) * 2e-4 for _ in range(nbuf)]
+    nbuf = max(2, min(6, int(600e6 // (N * K)) + 1))  # rotate through > 512 MB of weights when they are small
+    ws, wss = zip(*[device_block_fp8_weight(N, K, gen, dev) for _ in range(nbuf)])
     x = make_activation(M, K).to(dev)
     aligned = N % 128 == 0 and K % 128 == 0
     x_q, x_s = fp8_kernel.per_token_group_quant_fp8(x, 128, column_major_scales=aligned)
@@ -223,8 +231,6 @@ def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
     if direct:
         # decode-sized steps take tens of microseconds: call the C ABI directly with preallocated output and workspace,
         # so that the host keeps the queue full and the events time kernels rather than Python
-        from sglang_amd import _lib
-
         L = _lib.lib()
         wsb = L.mi355_fp8_blockwise_mm_workspace_bytes(M, N, K)
         wsbuf = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
@@ -237,26 +243,16 @@ def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
         def step(i):  # noqa: F811
             _lib.check(L.mi355_fp8_blockwise_mm(*args[i]))
 
-    wall, ms = _time_launches(step, nbuf, steps, warmup)
-    st = _stats(ms)
-    if direct:  # back-to-back launches: HIP-event time of the whole region / launches
-        st["avg"] = _last_region_ms / steps
-    flops = gemm_flops(M, N, K)
-    nbytes = fp8_gemm_algorithmic_bytes(M, N, K)
-    tflops_avg = flops / (st["avg"] * 1e-3) / 1e12
-    gbs_avg = nbytes / (st["avg"] * 1e-3) / 1e9
-    # which roof binds: time at peak MFMA rate vs time at peak HBM rate
-    mfma_bound = flops / (FP8_PEAK_TFLOPS * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9)
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms, b2b)
+    flops, nbytes = gemm_flops(M, N, K), fp8_gemm_algorithmic_bytes(M, N, K)
+    plan = _lib.gemm_plan("fp8", M, N, K, aligned=(K % 16 == 0))
     rec = {
         "workload": f"fp8_gemm {name} M={M} K={K} N={N} (e4m3fn x e4m3fn, 1x128 / 128x128 fp32 scales, bf16 out"
         + (", direct C-ABI calls)" if direct else ")"),
         "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
-        "gbytes_per_s": gbs_avg, "dtype": "fp8(e4m3fn) MFMA, f32 accumulate",
-        "roofline": ({"bound": "mfma", "achieved": tflops_avg, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                      "frac": tflops_avg / FP8_PEAK_TFLOPS, "traffic": None, "algorithmic_flops_per_launch": flops}
-                     if mfma_bound else
-                     {"bound": "hbm", "achieved": gbs_avg, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                      "frac": gbs_avg / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes_per_launch": nbytes}),
+        "dtype": "fp8(e4m3fn) MFMA, f32 accumulate", "kernel": plan["kernel"] + (f" x{plan['splits']}" if plan["splits"] > 1 else ""),
+        "roofline": _roofline(flops, nbytes, st["median"], FP8_PEAK_TFLOPS, "TFLOP/s"),
     }
     if with_cpu:
         from oracle import oracle
@@ -266,10 +262,8 @@ def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
         w_c, sw_c = ws[0][:ns_].cpu().contiguous(), wss[0][: cdiv(ns_, 128)].cpu().contiguous()
         dt, reps = _cpu_time_boxed(lambda: oracle.fp8_blockwise_mm(a_c, w_c, sa_c, sw_c, torch.bfloat16))
         rec["cpu_baseline"] = {
-            "value": gemm_flops(ms_, ns_, K) / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(),
-            "kind": "port",
-            "sample": f"first {ms_} tokens x first {ns_} channels x full K={K}, {reps} repetitions in ~10 s, "
-                      "C oracle with OpenMP (fp64 block sums)",
+            "value": gemm_flops(ms_, ns_, K) / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{ms_} tokens x {ns_} channels x K={K}, {reps} reps in ~10 s, C oracle with OpenMP (fp64 block sums)",
         }
         # the reference's torch-native formulation (test_block_fp8.py:273-325) on the same sample, fp32 matmul per K block
         A32, B32 = a_c.float(), w_c.float()
@@ -282,19 +276,26 @@ def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu):
             return C.to(torch.bfloat16)
 
         dt2, reps2 = _cpu_time_boxed(native, 5.0)
-        rec["cpu_baseline_torch_native"] = {
-            "value": gemm_flops(ms_, ns_, K) / dt2 / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-            "kind": "port", "sample": f"same sample, {reps2} repetitions in ~5 s, torch fp32 matmul per K block",
-        }
+        rec["cpu_torch_native"] = {"value": gemm_flops(ms_, ns_, K) / dt2 / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                                   "kind": "port", "sample": f"same sample, {reps2} reps in ~5 s, torch fp32 matmul per K block"}
+        if w8a16_cpu:
+            # the arithmetic of the reference's own CPU kernel (sgl-kernel/csrc/cpu/gemm_fp8.cpp:471-551): bf16 activations are
+            # NOT quantized, the fp8 weight is dequantized per block and multiplied in bf16 (w8a16) - a different operator
+            xb = x[:ms_].cpu()
+            wdq = (B32 * sw_c.repeat_interleave(128, 0)[:ns_].repeat_interleave(128, 1)[:, :K]).to(torch.bfloat16)
+            dt3, reps3 = _cpu_time_boxed(lambda: xb @ wdq.T, 5.0)
+            rec["cpu_w8a16_shape"] = {"value": gemm_flops(ms_, ns_, K) / dt3 / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                                      "kind": "port", "sample": f"same sample, {reps3} reps in ~5 s, bf16 x dequantized-weight matmul "
+                                      "(w8a16: what the reference's CPU build computes; different arithmetic, weight dequantized once)"}
     return rec
 
 
 # ------------------------------------------------------------------------------------------ INT8 GEMM
 
-def bench_int8_gemm(name, M, K, N, steps, warmup):
+def bench_int8_gemm(name, M, K, N, steps, warmup, with_cpu=False):
     import torch
 
-    from sglang_amd import sgl_kernel
+    from sglang_amd import _lib, sgl_kernel
     from sglang_amd.workloads import gemm_flops, int8_gemm_algorithmic_bytes
 
     dev = torch.device("cuda:0")
@@ -312,8 +313,6 @@ def bench_int8_gemm(name, M, K, N, steps, warmup):
 
     direct = M <= 256
     if direct:
-        from sglang_amd import _lib
-
         L = _lib.lib()
         wsb = L.mi355_int8_scaled_mm_workspace_bytes(M, N, K)
         wsbuf = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
@@ -325,24 +324,29 @@ def bench_int8_gemm(name, M, K, N, steps, warmup):
         def step(i):  # noqa: F811
             _lib.check(L.mi355_int8_scaled_mm(*args[i]))
 
-    wall, ms = _time_launches(step, nbuf, steps, warmup)
-    st = _stats(ms)
-    if direct:
-        st["avg"] = _last_region_ms / steps
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms, b2b)
     ops_, nbytes = gemm_flops(M, N, K), int8_gemm_algorithmic_bytes(M, N, K)
-    tops, gbs = ops_ / (st["avg"] * 1e-3) / 1e12, nbytes / (st["avg"] * 1e-3) / 1e9
-    mfma_bound = ops_ / (INT8_PEAK_TOPS * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9)
-    return {
+    plan = _lib.gemm_plan("int8", M, N, K)
+    rec = {
         "workload": f"int8_gemm {name} M={M} K={K} N={N} (int8 x int8 -> int32, per-token x per-channel scales, bias, bf16 out"
         + (", direct C-ABI calls)" if direct else ")"),
         "value": ops_ / (wall / steps) / 1e12, "unit": "TOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
-        "gbytes_per_s": gbs, "dtype": "int8 MFMA, int32 accumulate",
-        "roofline": ({"bound": "mfma", "achieved": tops, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                      "frac": tops / INT8_PEAK_TOPS, "traffic": None}
-                     if mfma_bound else
-                     {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                      "frac": gbs / HBM_PEAK_GBS, "traffic": None}),
+        "dtype": "int8 MFMA, int32 accumulate", "kernel": plan["kernel"] + (f" x{plan['splits']}" if plan["splits"] > 1 else ""),
+        "roofline": _roofline(ops_, nbytes, st["median"], INT8_PEAK_TOPS, "TOP/s"),
     }
+    if with_cpu:
+        from oracle import oracle
+
+        ms_, ns_ = min(M, 64), min(N, 1024)
+        a_c, w_c = a[:ms_].cpu().contiguous(), ws[0][:ns_].cpu().contiguous()
+        sa_c, sb_c, b_c = sa[:ms_].cpu().view(-1).contiguous(), sb[:ns_].cpu().contiguous(), bias[:ns_].cpu().contiguous()
+        dt, reps = _cpu_time_boxed(lambda: oracle.int8_scaled_mm(a_c, w_c, sa_c, sb_c, torch.bfloat16, b_c))
+        rec["cpu_baseline"] = {
+            "value": gemm_flops(ms_, ns_, K) / dt / 1e12, "unit": "TOP/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": f"{ms_} tokens x {ns_} channels x K={K}, {reps} reps in ~10 s, C oracle with OpenMP (exact int32 matmul + epilogue)",
+        }
+    return rec
 
 
 def bench_copy(steps, warmup):
@@ -354,15 +358,12 @@ def bench_copy(steps, warmup):
     n = 256 << 20
     srcs = [torch.randint(0, 255, (n,), dtype=torch.uint8, device=dev) for _ in range(3)]
     dsts = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in range(3)]
-    wall, ms = _time_launches(lambda i: dsts[i].copy_(srcs[i]), 3, steps, warmup)
-    st = _stats(ms)
-    gbs = 2 * n / (st["avg"] * 1e-3) / 1e9
+    wall, ms, b2b = _time_launches(lambda i: dsts[i].copy_(srcs[i]), 3, steps, warmup)
+    st = _stats(ms, b2b)
     return {
         "workload": f"copy {n} bytes device to device (torch copy kernel; {n} read + {n} written)",
         "value": 2 * n / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
-        "dtype": "u8",
-        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes_per_launch": 2 * n},
+        "dtype": "u8", "roofline": _roofline(0, 2 * n, st["median"], FP8_PEAK_TFLOPS, "TFLOP/s"),
     }
 
 
@@ -376,13 +377,36 @@ def _measured_traffic():
         return {}
 
 
+def _traffic_key(rec):
+    head = rec["workload"].split(" (")[0].split(",")[0]  # e.g. "fp8_gemm gate_up M=4096 K=7168 N=36864"
+    parts = head.split()
+    if parts[0] == "group":
+        return "quant_ue8m0" if "UE8M0" in rec["workload"] else "quant"
+    return "_".join(x for x in parts if "=" not in x) + "".join("_" + x.replace("=", "") for x in parts if x.startswith("M="))
+
+
+def _short(rec):
+    """One compact row of the "also" list."""
+    head = rec["workload"].split(" (")[0].replace("fp8_gemm ", "fp8 ").replace("int8_gemm ", "int8 ")
+    ro = rec["roofline"]
+    row = {"w": head, "ms": rec["kernel_ms"]["median"], "b2b": rec["kernel_ms"]["b2b"], "v": ro["achieved"], "u": ro["unit"],
+           "bound": ro["bound"], "frac": ro["frac"]}
+    if "kernel" in rec:
+        row["kern"] = rec["kernel"]
+    for k in ("cpu_baseline", "cpu_torch_native", "cpu_w8a16_shape"):
+        if k in rec:
+            row[k] = {"v": rec[k]["value"], "u": rec[k]["unit"], "cores": rec[k]["cores"], "kind": rec[k]["kind"],
+                      "sample": rec[k]["sample"]}
+    return row
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--quick", action="store_true", help="headline only (no 'also' list)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -409,27 +433,31 @@ def main():
     del _a, _b
 
     S, W, cpu = args.steps, args.warmup, not args.no_cpu
-    also = []
-    if args.workload in ("quant", "quant_ue8m0"):
-        rec = bench_quant(S, W, args.workload == "quant_ue8m0", cpu)
-    elif args.workload == "copy":
+    also, quant = [], []
+    wl = args.workload
+    if wl in ("quant", "quant_ue8m0"):
+        rec = bench_quant(S, W, wl == "quant_ue8m0", cpu)
+    elif wl == "copy":
         rec = bench_copy(S, W)
-    elif args.workload == "fp8_decode":
+    elif wl == "fp8_decode":
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 1, K, N, S, W, cpu)
-    elif args.workload == "int8_gemm":
+    elif wl == "int8_gemm":
         K, N = LLAMA3_8B["gate_up"]
-        rec = bench_int8_gemm("gate_up", 4096, K, N, S, W)
+        rec = bench_int8_gemm("gate_up", 4096, K, N, S, W, cpu)
+    elif wl.startswith("fp8:") or wl.startswith("int8:"):
+        kind, M, K, N = wl.split(":")
+        fn = bench_fp8_gemm if kind == "fp8" else bench_int8_gemm
+        rec = fn("shape", int(M), int(K), int(N), S, W, cpu)
     else:
-        quant_recs = []
-        if args.workload == "all" and not args.quick:
+        full = wl == "all" and not args.quick
+        if full:
             # the bandwidth-bound quantizer is measured first: right after the MFMA-heavy GEMMs the chip's power state
             # makes a 60 us streaming kernel read ~15 % slow
-            quant_recs = [bench_quant(S, W, False, cpu), bench_quant(S, W, True, False)]
+            quant = [bench_quant(S, W, False, cpu), bench_quant(S, W, True, False)]
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 4096, K, N, S, W, cpu)
-        if args.workload == "all" and not args.quick:
-            also.extend(quant_recs)
+        if full:
             K, N = DSV3_MLP["down"]
             also.append(bench_fp8_gemm("down", 4096, K, N, S, W, False))
             for nm, (K, N) in DSV3_MLA.items():
@@ -437,35 +465,34 @@ def main():
             for M in (1, 8, 32, 128):
                 for nm, (K, N) in DSV3_MLP.items():
                     also.append(bench_fp8_gemm(nm, M, K, N, S, W, False))
-            also.append(bench_fp8_gemm("single_linear", 16, 7168, 2048, S, W, cpu))
+            also.append(bench_fp8_gemm("single_linear", 16, 7168, 2048, S, W, cpu, w8a16_cpu=cpu))
             for M in (1, 256, 4096):
                 for nm, (K, N) in LLAMA3_8B.items():
-                    also.append(bench_int8_gemm(nm, M, K, N, S, W))
+                    also.append(bench_int8_gemm(nm, M, K, N, S, W, with_cpu=(cpu and M == 4096 and nm == "gate_up")))
 
     traffic = _measured_traffic()
-    for r in [rec] + also:
-        head = r["workload"].split(" (")[0].split(",")[0]  # e.g. "fp8_gemm gate_up M=4096 K=7168 N=36864"
-        parts = head.split()
-        key = "_".join(x for x in parts if "=" not in x) + "".join("_" + x.replace("=", "") for x in parts if x.startswith("M="))
-        if parts[0].startswith("quant"):
-            key = parts[0]
+    for r in [rec] + also + quant:
+        key = _traffic_key(r)
         if key in traffic:
             r["roofline"]["traffic"] = traffic[key]
 
     line = {
         "metric": METRIC, "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": S, "warmup": W,
         "ms_per_step": rec["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": rec["dtype"],
-        "data": "synthetic, seeded; resident in HBM before the timed region",
-        "config": {"workload": rec["workload"]},
+        "dtype": rec["dtype"], "data": DATA, "config": {"workload": rec["workload"]},
         "roofline": rec["roofline"], "kernel_ms": rec["kernel_ms"],
     }
-    for k in ("cpu_baseline", "cpu_baseline_torch_native", "gbytes_per_s"):
+    for k in ("kernel", "cpu_baseline", "cpu_torch_native"):
         if k in rec:
             line[k] = rec[k]
     if also:
-        line["also"] = also
-    print(json.dumps(line))
+        line["also"] = [_short(r) for r in also]
+    if quant:
+        # last in the line, so that a reader who only keeps the end of the output still has them
+        line["quant"] = [{"workload": q["workload"], "value": q["value"], "unit": q["unit"], "kernel_ms": q["kernel_ms"],
+                          "roofline": q["roofline"], **({"cpu_baseline": q["cpu_baseline"]} if "cpu_baseline" in q else {})}
+                         for q in quant]
+    print(json.dumps(r4(line), separators=(",", ":")))
 
 
 if __name__ == "__main__":

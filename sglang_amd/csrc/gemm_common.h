@@ -92,10 +92,7 @@ int launch_fp8_pipelined(GemmParams& p, hipStream_t stream, const char* what);
 // Large-M blockwise FP8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases);
 // gemm_fp8_pp.hip.  Same requirements.
 int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what);
-// Its token scales must be M-major with a 16-byte friendly pitch; otherwise it copies them into p.ws first, which must
-// then hold fp8_pp_workspace_bytes(M, K) bytes.
-size_t fp8_pp_workspace_bytes(int64_t M, int64_t K);
-bool fp8_pp_scales_conform(const GemmParams& p);
+// Token scales must be M-major with a pitch that is a multiple of four floats and a 16-byte aligned base.
 
 
 // Mid-M blockwise FP8 GEMM (64/128 x 256 tile, 8 waves, three LDS stages, hand-issued direct-to-LDS loads);

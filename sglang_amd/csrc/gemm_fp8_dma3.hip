@@ -14,7 +14,8 @@
 //     overwritten only after the barrier that follows its last read.
 // Operand roles, swizzle, chunk mapping and promotion FMA are those of gemm_w8a8.hip; a step is {MFMA of tile t, FMAs of
 // tile t-1}.  Optional split along K (partials to the workspace, ordered reduce afterwards).
-// Requires K % 128 == 0, 16-byte aligned rows, row offsets below 4 GiB.
+// Requires K % 128 == 0, 16-byte aligned rows, row offsets below 4 GiB, and token scales laid out M-major with a pitch that is
+// a multiple of four floats (fp8_scales_conform; the dispatcher re-lays other layouts out into the workspace first).
 #include "gemm_common.h"
 
 namespace mi355 {
@@ -28,7 +29,7 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
 typedef const __attribute__((address_space(4))) float* cfloat_ptr;
 
-// three stages: tiles (rows 0..BM-1 tokens, BM.. channels) and token scales (8 waves x 64 floats, see below)
+// three stages: tiles (rows 0..BM-1 tokens, BM.. channels) and the tile's BM token scales
 __shared__ __attribute__((aligned(1024))) uint8_t t_stage0[(128 + T_BN) * KSTEP];
 __shared__ __attribute__((aligned(1024))) uint8_t t_stage1[(128 + T_BN) * KSTEP];
 __shared__ __attribute__((aligned(1024))) uint8_t t_stage2[(128 + T_BN) * KSTEP];
@@ -52,7 +53,8 @@ struct Dma3State {
   const uint8_t* a_base;
   const uint8_t* b_base;
   uint32_t goff[LOADS];   // lane's byte offset from the matrix base (rows clamped); first BM/64 loads are token rows
-  const float* sa_ptr;    // &sa[m, 0] of the token whose scale this lane fetches (lanes beyond BM refetch a valid one)
+  const float* sa_base;   // token scales, M-major: element (m, kb) at sa_base[kb * sa_sk + m]
+  uint32_t sa_off;        // byte offset of the four scales this lane fetches (first BM / 32 lanes), clamped to the last valid quad
   cfloat_ptr sb_ptr;      // &sb[nb, 0] of this wave's 128-channel block
   int64_t sa_sk, sb_sk;
   int wave, kb_last;
@@ -72,9 +74,18 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM>& s, int i, uint8_t
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + (i * 64 + s.wave * 8) * KSTEP);
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(s.goff[i]), "s"(base), "s"(lds_addr) : "memory");
   } else {
-    const float* src = s.sa_ptr + (int64_t)kb * s.sa_sk;
-    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(scale + s.wave * 64);
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+    // the wave's BM / 8 token scales: BM / 32 lanes fetch 16 bytes each (a 4-byte-per-lane load in this stream costs far
+    // more than its size: measured 1.5x on the whole large-M kernel).  exec is narrowed and restored inside the statement.
+    const float* sbase = s.sa_base + (int64_t)kb * s.sa_sk;  // wave-uniform
+    asm volatile("" : "+s"(sbase));
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(scale + s.wave * (BM / 8));
+    uint64_t saved;
+    if constexpr (BM == 128)
+      asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xf\n\ts_mov_b32 m0, %3\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+                   : "=&s"(saved) : "v"(s.sa_off), "s"(sbase), "s"(lds_addr) : "memory");
+    else
+      asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0x3\n\ts_mov_b32 m0, %3\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+                   : "=&s"(saved) : "v"(s.sa_off), "s"(sbase), "s"(lds_addr) : "memory");
   }
 }
 
@@ -175,8 +186,9 @@ __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmPara
     }
     s.sc_off = (wave_m * WM + l16) * 4;
   }
-  // all eight waves fetch 64 token scales each (branch-free); the tile only has BM of them, the rest are refetched copies
-  s.sa_ptr = p.sa + (int64_t)min(m0 + (tid & (BM - 1)), p.M - 1) * p.sa_sm;
+  // every wave fetches BM / 8 token scales per K block, four per lane; quads past M refetch the last valid one
+  s.sa_base = p.sa;
+  s.sa_off = (uint32_t)min(m0 + wave * (BM / 8) + (lane & (BM / 32 - 1)) * 4, (p.M - 1) & ~3) * 4u;
   s.sa_sk = p.sa_sk;
   s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * T_WN, p.N - 1) / 128) * p.sb_sn);
   s.sb_sk = p.sb_sk;

@@ -29,7 +29,7 @@
 // Token scales: measured, ONE 4-byte-per-lane load per wave and K block (direct-to-LDS or to a register, whatever its
 // address or position in the stream) makes this kernel 1.5x slower, while 16-byte-per-lane loads stream freely.  So the
 // scales must be M-major (256 consecutive floats per tile and K block, the layout fp8_blockwise_scaled_mm prescribes),
-// and each wave fetches 32 of them with the first eight lanes of a 16-byte direct-to-LDS load; the launcher re-lays
+// and each wave fetches 32 of them with the first eight lanes of a 16-byte direct-to-LDS load; the dispatcher re-lays
 // other layouts out into the workspace first.  They use four small LDS stages so that they can travel with set A.
 // Loads, waits and barriers are written as instructions (the compiler would wait for all loads at every barrier).
 // Arithmetic, operand roles, LDS layout and swizzle are those of gemm_w8a8.hip.
@@ -327,53 +327,12 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
 
 
 
-// out[kb * ld_out + m] = sa[m * sa_sm + kb * sa_sk]: token scales re-laid out M-major with a row pitch that is a multiple
-// of four floats.  One 32 x 32 tile per workgroup through LDS, so that reads and writes are both contiguous for either
-// input layout.
-__global__ __launch_bounds__(256) void relayout_scales_kernel(const float* sa, int64_t sa_sm, int64_t sa_sk, float* out,
-                                                              int64_t ld_out, int M, int KB) {
-  __shared__ float tile[32][33];
-  const int m0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
-  const bool k_fast = sa_sk < sa_sm;                       // which index is contiguous in the input
-#pragma unroll
-  for (int r = ty; r < 32; r += 8) {
-    const int m = k_fast ? m0 + r : m0 + tx, kb = k_fast ? k0 + tx : k0 + r;
-    if (m < M && kb < KB) tile[kb - k0][m - m0] = sa[(int64_t)m * sa_sm + (int64_t)kb * sa_sk];
-  }
-  __syncthreads();
-#pragma unroll
-  for (int r = ty; r < 32; r += 8) {
-    const int m = m0 + tx, kb = k0 + r;
-    if (m < M && kb < KB) out[(int64_t)kb * ld_out + m] = tile[r][tx];
-  }
-}
-
 }  // namespace
 
-// The kernel reads token scales M-major with 16-byte loads.  Scales that are not laid out that way (K-major, as
-// per_token_group_quant_fp8 returns them by default; a pitch or base that is not a multiple of 16 bytes) are first copied
-// into the workspace.
-size_t fp8_pp_workspace_bytes(int64_t M, int64_t K) { return (size_t)((M + 3) & ~3ll) * (size_t)((K + KSTEP - 1) / KSTEP) * 4u; }
-
-bool fp8_pp_scales_conform(const GemmParams& p) {
-  return p.sa_sm == 1 && (p.sa_sk & 3) == 0 && p.sa_sk >= ((p.M + 3) & ~3) && (reinterpret_cast<uintptr_t>(p.sa) & 15) == 0;
-}
-
-// Needs 16-byte aligned rows and row offsets below 4 GiB; p.ws must hold fp8_pp_workspace_bytes() when the scales do not
-// conform.
+// Needs 16-byte aligned rows, row offsets below 4 GiB and conforming token scales (fp8_scales_conform).
 int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + G_BM - 1) / G_BM;
   p.tiles_n = (p.N + G_BN - 1) / G_BN;
-  if (!fp8_pp_scales_conform(p)) {
-    float* dst = static_cast<float*>(p.ws);
-    const int64_t ld = (p.M + 3) & ~3;
-    hipLaunchKernelGGL(relayout_scales_kernel, dim3((unsigned)((p.M + 31) / 32), (unsigned)((p.kb_total + 31) / 32)), dim3(256), 0,
-                       stream, p.sa, p.sa_sm, p.sa_sk, dst, ld, p.M, p.kb_total);
-    const int rc = check_launch(what);
-    if (rc != MI355_OK) return rc;
-    p.sa = dst, p.sa_sm = 1, p.sa_sk = ld;
-  }
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
   if (p.K % KSTEP == 0)
     hipLaunchKernelGGL(fp8_gemm_pp_kernel<true>, grid, dim3(G_THREADS), 0, stream, p);

@@ -336,6 +336,8 @@ Plan make_plan(int64_t M, int64_t N, int64_t K) {
   return pl;
 }
 
+size_t scale_relayout_bytes(int64_t M, int64_t K);
+
 // Upper bound over the kernels a shape may be routed to (the choice also depends on pointer alignment, which is not
 // known here).
 size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
@@ -352,10 +354,7 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
     const size_t dneed = ds > 1 ? (size_t)ds * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
   }
-  if (is_fp8 && M > 1024) {  // the large-M kernel may have to re-lay the token scales out
-    const size_t sneed = fp8_pp_workspace_bytes(M, K);
-    if (sneed > need) need = sneed;
-  }
+  if (is_fp8 && M > 16) need += scale_relayout_bytes(M, K);  // the direct-to-LDS kernels may have to re-lay the token scales out
   return need;
 }
 
@@ -450,11 +449,49 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   return r;
 }
 
-// Workspace bytes the chosen route needs for this call: split-K partial sums, or a re-laid-out copy of the token scales.
+// out[kb * ld_out + m] = sa[m * sa_sm + kb * sa_sk]: token scales re-laid out M-major with a row pitch that is a multiple
+// of four floats.  One 32 x 32 tile per workgroup through LDS, so that reads and writes are both contiguous for either
+// input layout.
+__global__ __launch_bounds__(256) void relayout_scales_kernel(const float* sa, int64_t sa_sm, int64_t sa_sk, float* out,
+                                                              int64_t ld_out, int M, int KB) {
+  __shared__ float tile[32][33];
+  const int m0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  const bool k_fast = sa_sk < sa_sm;                       // which index is contiguous in the input
+#pragma unroll
+  for (int r = ty; r < 32; r += 8) {
+    const int m = k_fast ? m0 + r : m0 + tx, kb = k_fast ? k0 + tx : k0 + r;
+    if (m < M && kb < KB) tile[kb - k0][m - m0] = sa[(int64_t)m * sa_sm + (int64_t)kb * sa_sk];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = ty; r < 32; r += 8) {
+    const int m = m0 + tx, kb = k0 + r;
+    if (m < M && kb < KB) out[(int64_t)kb * ld_out + m] = tile[r][tx];
+  }
+}
+
+
+// The direct-to-LDS kernels (two-phase large-M, three-stage mid-M) read token scales M-major with 16-byte loads.  Scales
+// that are not laid out that way (K-major, as per_token_group_quant_fp8 returns them by default; a pitch or base that is
+// not a multiple of 16 bytes) are first copied into the head of the workspace.
+size_t scale_relayout_bytes(int64_t M, int64_t K) {
+  const size_t b = (size_t)((M + 3) & ~3ll) * (size_t)((K + KSTEP - 1) / KSTEP) * 4u;
+  return (b + 255) & ~(size_t)255;  // what follows in the workspace stays 256-byte aligned
+}
+bool fp8_scales_conform(const GemmParams& p) {
+  return p.sa_sm == 1 && (p.sa_sk & 3) == 0 && p.sa_sk >= ((p.M + 3) & ~3) && (reinterpret_cast<uintptr_t>(p.sa) & 15) == 0;
+}
+bool route_wants_m_major_scales(bool is_fp8, const Route& r) {
+  return is_fp8 && (r.kernel == RK_PINGPONG || r.kernel == RK_DMA3);
+}
+
+// Workspace bytes the chosen route needs for this call: a re-laid-out copy of the token scales (first) and split-K
+// partial sums (after it).
 size_t route_workspace_need(bool is_fp8, const Route& r, const GemmParams& p) {
-  if (r.splits > 1) return (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u;
-  if (is_fp8 && r.kernel == RK_PINGPONG && !fp8_pp_scales_conform(p)) return fp8_pp_workspace_bytes(p.M, p.K);
-  return 0;
+  size_t need = r.splits > 1 ? (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u : 0;
+  if (route_wants_m_major_scales(is_fp8, r) && !fp8_scales_conform(p)) need += scale_relayout_bytes(p.M, p.K);
+  return need;
 }
 
 bool operands_aligned(const GemmParams& p) {
@@ -476,6 +513,16 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
     MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE,
                   "%s: workspace must be 16-byte aligned", what);
     p.ws = workspace;
+  }
+  if (route_wants_m_major_scales(IS_FP8, r) && !fp8_scales_conform(p)) {
+    float* dst = static_cast<float*>(workspace);
+    const int64_t ld = (p.M + 3) & ~3;
+    hipLaunchKernelGGL(relayout_scales_kernel, dim3((unsigned)((p.M + 31) / 32), (unsigned)((p.kb_total + 31) / 32)), dim3(256), 0,
+                       stream, p.sa, p.sa_sm, p.sa_sk, dst, ld, p.M, p.kb_total);
+    const int rc0 = check_launch(what);
+    if (rc0 != MI355_OK) return rc0;
+    p.sa = dst, p.sa_sm = 1, p.sa_sk = ld;
+    p.ws = static_cast<uint8_t*>(workspace) + scale_relayout_bytes(p.M, p.K);
   }
   int rc;
   switch (r.kernel) {
