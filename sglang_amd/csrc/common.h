@@ -64,6 +64,20 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv& f) {
   return (t + n) >> f.shift;  // n < 2^31, so t + n cannot overflow
 }
 
+// Separately rounded fp32 multiply and add, written as instructions: the INT8 epilogue contract is mul, mul, add, and no
+// compiler setting or code motion may fuse two of them into an FMA (a fused result differs in the last bit of the 16-bit
+// output about once in 10^5 elements).
+__device__ __forceinline__ float mul_rn(float a, float b) {
+  float r;
+  asm("v_mul_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float add_rn(float a, float b) {
+  float r;
+  asm("v_add_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {

@@ -61,6 +61,41 @@ __device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off
 }
 
 
+// ---- 256 x 256 output tile of 16-bit elements through LDS.
+// A lane's accumulators are four consecutive channels of one token: stored straight from registers, a wave instruction
+// writes 16 or 32 separate 32-byte pieces, and a tile takes ~12 us.  Instead every wave writes its results into a
+// [256 tokens][512 bytes] image of the tile in LDS (16-byte chunks XOR-swizzled with the row so that neither side has
+// bank conflicts), and after a barrier each wave stores 32 whole rows, two rows of 512 contiguous bytes per instruction.
+constexpr int OUT_TILE_BYTES = 256 * 512;
+
+__device__ __forceinline__ uint32_t pack2_16(int out_dtype, float lo, float hi) {
+  return out_dtype == MI355_BF16 ? (f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16))
+                                 : (f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16));
+}
+// four consecutive channels starting at tile column `col` (a multiple of 4) of tile row `row`
+__device__ __forceinline__ void out_tile_put4(uint8_t* tile, int row, int col, int out_dtype, const float* r) {
+  const int chunk = col >> 3, half = (col >> 2) & 1;
+  *reinterpret_cast<u32x2*>(tile + row * 512 + ((chunk ^ (row & 7)) << 4) + half * 8) =
+      u32x2{pack2_16(out_dtype, r[0], r[1]), pack2_16(out_dtype, r[2], r[3])};
+}
+// Called by all 512 threads after a barrier that follows the last out_tile_put4.  Needs ldo % 8 == 0, a 16-byte aligned
+// output base and n0 + 256 <= N; rows at or past M are skipped.
+__device__ __forceinline__ void out_tile_store(const uint8_t* tile, void* out, int64_t ldo, int m0, int n0, int M) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int chunk = lane & 31;
+  uint16_t* o = reinterpret_cast<uint16_t*>(out);
+#pragma unroll 4
+  for (int it = 0; it < 16; ++it) {
+    const int row = wave * 32 + it * 2 + (lane >> 5);
+    const u32x4 v = *reinterpret_cast<const u32x4*>(tile + row * 512 + ((chunk ^ (row & 7)) << 4));
+    if (m0 + row < M) *reinterpret_cast<u32x4*>(o + (int64_t)(m0 + row) * ldo + n0 + chunk * 8) = v;
+  }
+}
+__device__ __forceinline__ bool out_tile_ok(const void* out, int64_t ldo, int out_dtype, int n0, int N) {
+  return (out_dtype == MI355_BF16 || out_dtype == MI355_F16) && (ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+         n0 + 256 <= N;
+}
+
 struct TileCoord {
   int tile_m, tile_n, split;
 };
@@ -109,6 +144,10 @@ int launch_int8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, 32x32x32 MFMA); gemm_int8_dma.hip.
 // Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
 int launch_int8_dma(GemmParams& p, hipStream_t stream, const char* what);
+
+// Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases); gemm_int8_pp.hip.
+// Same requirements.
+int launch_int8_pp(GemmParams& p, hipStream_t stream, const char* what);
 
 // Small-M blockwise FP8 GEMM streaming the weight through wave-private LDS, no barriers; gemm_fp8_decode.hip.
 // decode_splits() is the split count it wants for a shape; the caller sets p.splits, p.kb_per_split and p.ws.

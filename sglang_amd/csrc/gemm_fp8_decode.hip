@@ -269,10 +269,10 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
           float r[4];
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
-            float t = __fmul_rn((float)acc[i][v], __fmul_rn(p.sb[n + v], sa_m));
+            float t = mul_rn((float)acc[i][v], mul_rn(p.sb[n + v], sa_m));
             if (p.bias) {
               const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
-              t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+              t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
             }
             r[v] = t;
           }

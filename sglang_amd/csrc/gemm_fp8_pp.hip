@@ -46,8 +46,11 @@ constexpr int G_ROWS = G_BM + G_BN;
 constexpr int G_LOADS = G_ROWS / 64;               // 8 direct-to-LDS tile loads per wave and K block
 constexpr int G_STAGE = G_ROWS * KSTEP;
 
-__shared__ __attribute__((aligned(1024))) uint8_t g_stage0[G_STAGE];
-__shared__ __attribute__((aligned(1024))) uint8_t g_stage1[G_STAGE];
+// the two stages are one array: after the K loop it holds the output tile on its way to memory
+__shared__ __attribute__((aligned(1024))) uint8_t g_stages[2 * G_STAGE];
+#define g_stage0 (g_stages)
+#define g_stage1 (g_stages + G_STAGE)
+static_assert(2 * G_STAGE >= OUT_TILE_BYTES, "the output tile is staged in the two input stages");
 // token scales: four stages (block b in stage b % 4) of 256 floats
 __shared__ __attribute__((aligned(256))) float g_scale[4 * G_BM];
 
@@ -311,6 +314,17 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   // ---- epilogue: lane holds channels n .. n+3 of token m
+  if (out_tile_ok(p.out, p.ldo, p.out_dtype, n0, p.N)) {
+    asm volatile("s_barrier" ::: "memory");  // every wave's stray loads have landed: the stages are free
+#pragma unroll
+    for (int j = 0; j < G_MT; ++j)
+#pragma unroll
+      for (int i = 0; i < G_NT; ++i)
+        out_tile_put4(g_stages, grp * G_WM + j * 16 + l16, wave_n * G_WN + i * 16 + 4 * q, p.out_dtype, acc[i][j]);
+    __syncthreads();
+    out_tile_store(g_stages, p.out, p.ldo, m0, n0, p.M);
+    return;
+  }
   const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
 #pragma unroll
   for (int j = 0; j < G_MT; ++j) {

@@ -189,10 +189,10 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             const int nn = min(n + v, p.N - 1);
-            float t = __fmul_rn((float)acc[i][j][4 * g + v], __fmul_rn(p.sb[nn], sa_m));
+            float t = mul_rn((float)acc[i][j][4 * g + v], mul_rn(p.sb[nn], sa_m));
             if (p.bias) {
               const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[nn];
-              t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+              t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
             }
             r[v] = t;
           }

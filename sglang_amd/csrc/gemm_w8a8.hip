@@ -237,10 +237,10 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const GemmParams p) {
           for (int v = 0; v < 4; ++v) {
             const int nn = min(n + v, p.N - 1);
             // separately rounded multiply and add: the contract is mul, mul, add, not a fused multiply-add
-            float t = __fmul_rn((float)acc[i][j][v], __fmul_rn(p.sb[nn], sa_m));
+            float t = mul_rn((float)acc[i][j][v], mul_rn(p.sb[nn], sa_m));
             if (p.bias) {
               const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[nn];
-              t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+              t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
             }
             r[v] = t;
           }
@@ -286,10 +286,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
     float r[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      float t = __fmul_rn((float)s[v], __fmul_rn(p.sb[n + v], sa_m));
+      float t = mul_rn((float)s[v], mul_rn(p.sb[n + v], sa_m));
       if (p.bias) {
         const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
-        t = __fadd_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+        t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
       }
       r[v] = t;
     }
@@ -534,7 +534,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
       break;
     case RK_PINGPONG: return launch_fp8_pp(p, stream, what);
     case RK_PIPELINED: return launch_fp8_pipelined(p, stream, what);
-    case RK_INT8_DMA256: return launch_int8_dma(p, stream, what);
+    case RK_INT8_DMA256: return launch_int8_pp(p, stream, what);
     default:
       // the generic kernel runs its own ordered reduce
       switch (r.bm) {
