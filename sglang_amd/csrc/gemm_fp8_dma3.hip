@@ -1,6 +1,7 @@
-// Mid-M blockwise-scaled FP8 GEMM for gfx950: (64 or 128) x 256 macro tile, 8 waves (two per SIMD), THREE LDS stages.
+// Blockwise-scaled FP8 GEMM for gfx950 with short token tiles: (64 or 128) x 256 macro tile, 8 waves (two per SIMD), THREE LDS stages.
 //
-// For 16 < M <= 1024 a linear layer is between weight streaming and MFMA-bound.  The tile is short in the token dimension
+// For 16 < M <= 1024 a linear layer is between weight streaming and MFMA-bound; prefill shapes with few output channels
+// (M = 4096, N = 576 or 1536) do not give 256 x 256 tiles enough workgroups.  Both take this kernel.  The tile is short in the token dimension
 // (64 or 128 tokens) and wide in channels (256), so a stage of LDS is (BM + 256) x 128 B <= 48 KB and three stages fit in
 // the CU's 160 KB.  With three stages the direct-to-LDS loads of K block k+2 are issued while block k is multiplied and
 // only have to land before block k+2 is multiplied, two barriers later: the wait that precedes the barrier at the end of
@@ -266,34 +267,40 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 
 }  // namespace
 
-// Token-tile height and split count for the mid-M kernel.  One workgroup per CU fits (three stages fill the LDS).
-// The estimate is a byte model, since this regime is bound by weight streaming: a split multiplies the number of
-// workgroups (better balance over 256 CUs when there are few tiles) but every extra split writes and re-reads an
-// M x N fp32 partial tile, and short K ranges pay the pipeline fill (two blocks) each.
-//   efficiency = balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2)
-// `efficiency` is returned so that the dispatcher can prefer another kernel when no split does well.
+// Token-tile height and split count for this kernel.  One workgroup per CU fits (three stages fill the LDS).
+// The estimate is a byte model for few tokens, where the kernel is bound by weight streaming: a split multiplies the
+// number of workgroups (better balance over 256 CUs when there are few tiles) but every extra split writes and re-reads
+// an M x N fp32 partial tile, and short K ranges pay the pipeline fill (two blocks) each:
+//   efficiency = balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2) * tile_factor
+// With many tokens (prefill shapes whose channel count is too small for 256 x 256 tiles) the same formula ranks the two
+// tile heights: 64-token tiles double the workgroups but do 0.65 of the work of a 128-token tile per unit of time
+// (measured on K=7168 -> N=1536 / N=576 at M=4096 and M=2048).
+// `efficiency` is returned so that the dispatcher can prefer another kernel when no choice does well.
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
   Dma3Plan pl;
-  pl.bm = M <= 64 ? 64 : 128;
   const int64_t kb_total = (K + KSTEP - 1) / KSTEP;
-  const int64_t tiles = ((M + pl.bm - 1) / pl.bm) * ((N + T_BN - 1) / T_BN);
   const double useful = (double)N * K + (double)M * K + 2.0 * M * N;
-  int best = 1;
-  double best_score = -1.0;
   const int max_split = (N % 4 == 0) ? 16 : 1;  // the reduce kernel works on aligned quads of one row
-  for (int sp = 1; sp <= max_split; ++sp) {
-    const int64_t per = (kb_total + sp - 1) / sp;
-    if (sp > 1 && per < 4) break;
-    if ((kb_total + per - 1) / per != sp) continue;  // some split would get no work
-    const int64_t wgs = tiles * sp;
-    const int64_t rounds = (wgs + 255) / 256;
-    const double balance = (double)wgs / (double)(rounds * 256);
-    const double partial = sp > 1 ? 8.0 * sp * M * N : 0.0;
-    const double score = balance * useful / (useful + partial) * (double)per / (double)(per + 2);
-    if (score > best_score) best_score = score, best = sp;
+  double best_score = -1.0;
+  pl.bm = 128, pl.splits = 1;
+  for (int bm = 64; bm <= 128; bm += 64) {
+    if (M <= 64 && bm == 128) break;                 // a second half tile of padding rows buys nothing
+    if (M > 64 && M <= 128 && bm == 64) continue;    // two token tiles would stream the weight twice
+    const double tile_factor = (bm == 64 && M > 128) ? 0.65 : 1.0;
+    const int64_t tiles = ((M + bm - 1) / bm) * ((N + T_BN - 1) / T_BN);
+    for (int sp = 1; sp <= max_split; ++sp) {
+      const int64_t per = (kb_total + sp - 1) / sp;
+      if (sp > 1 && per < 4) break;
+      if ((kb_total + per - 1) / per != sp) continue;  // some split would get no work
+      const int64_t wgs = tiles * sp;
+      const int64_t rounds = (wgs + 255) / 256;
+      const double balance = (double)wgs / (double)(rounds * 256);
+      const double partial = sp > 1 ? 8.0 * sp * M * N : 0.0;
+      const double score = balance * useful / (useful + partial) * (double)per / (double)(per + 2) * tile_factor;
+      if (score > best_score) best_score = score, pl.splits = sp, pl.bm = bm;
+    }
   }
-  pl.splits = best;
-  pl.kb_per_split = (int)((kb_total + best - 1) / best);
+  pl.kb_per_split = (int)((kb_total + pl.splits - 1) / pl.splits);
   pl.efficiency = best_score;
   return pl;
 }

@@ -344,8 +344,8 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const Plan pl = make_plan(M, N, K);
   size_t need = pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
-  if (M > 16 && M <= 1024 && K % KSTEP == 0) {
-    const Dma3Plan dp = dma3_plan(M, N, K);  // (an upper bound: the dispatcher may still pick the generic kernel)
+  if (M > 16 && K % KSTEP == 0) {
+    const Dma3Plan dp = dma3_plan(M, N, K);  // (an upper bound: the dispatcher may still pick another kernel)
     const size_t dneed = dp.splits > 1 ? (size_t)dp.splits * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
   }
@@ -417,8 +417,10 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
     r.groups_per_wg = decode_groups_per_wg(N, r.splits);
     return r;
   }
-  if (M > 16 && M <= 1024 && K % KSTEP == 0 && aligned && small_offsets) {
-    // mid-M: three-stage direct-to-LDS kernel, when its tiling fills the chip well enough
+  const int64_t tiles_256 = ((M + 255) / 256) * ((N + 255) / 256);
+  if (M > 16 && (M <= 1024 || tiles_256 < NUM_CUS) && K % KSTEP == 0 && aligned && small_offsets) {
+    // mid-M, or many tokens but too few channels for 256 x 256 tiles: three-stage direct-to-LDS kernel with 64- or 128-token
+    // tiles, when its tiling fills the chip well enough
     const Dma3Plan dp = dma3_plan(M, N, K);
     if (dp.efficiency >= DMA3_MIN_EFFICIENCY) {
       r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = 256, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
@@ -427,7 +429,6 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   }
   const Plan pl = make_plan(M, N, K);
   r.kernel = RK_GENERIC, r.bm = pl.bm, r.bn = pl.bn, r.splits = pl.splits, r.kb_per_split = pl.kb_per_split;
-  const int64_t tiles_256 = ((M + 255) / 256) * ((N + 255) / 256);
   const int64_t tiles_128 = ((M + 255) / 256) * ((N + 127) / 128);
   if (pl.bm == 256 && pl.splits == 1 && aligned && small_offsets) {
     if (is_fp8) {

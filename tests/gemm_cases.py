@@ -16,7 +16,7 @@ FP8_ROUTE_SHAPES = [
     (48, 16384, 2048), (33, 16384, 2176), (40, 65536, 512), (200, 16384, 2048), (100, 32768, 640), (130, 8192, 7168),
     (250, 8192, 7296),
     # 256 x 256 two-phase and 256 x 128 pipelined kernels, K a multiple of 128 and not
-    (4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 512), (4000, 2100, 272),
+    (4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 256), (4000, 2100, 272),
     # generic kernel: every token-tile height, aligned and byte-granular loads, whole-K and split
     (7, 1088, 512), (16, 576, 7168), (1, 1088, 3884), (17, 384, 2304), (20, 256, 264), (33, 512, 512), (64, 128, 3884),
     (50, 300, 520), (127, 128, 4096), (130, 640, 896), (1500, 640, 1000), (130, 200, 300), (2048, 4224, 264),
@@ -38,7 +38,7 @@ FP8_REQUIRED_VARIANTS = {
 INT8_ROUTE_SHAPES = [
     (16, 128, 512), (1, 6144, 4096), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432), (7, 33280, 4096),
     (5, 66048, 512), (2, 133120, 384),
-    (20, 8192, 4096), (40, 65536, 512), (200, 16384, 2048), (300, 4096, 14336), (130, 8192, 7168),
+    (20, 8192, 4096), (40, 65536, 512), (200, 16384, 2048), (200, 32768, 1024), (300, 4096, 14336), (130, 8192, 7168),
     (4096, 4096, 512), (4000, 4088, 1024),
     (1, 16, 512), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
 ]

@@ -189,7 +189,7 @@ def test_full_size_prefill_shape_properties(gpu, oracle):
 
 # Large-M kernels: 256x256 direct-to-LDS tiles (>= 256 such tiles) and 256x128 pipelined tiles, each with K a multiple of
 # 128 and not, and with ragged M and N edges.  The oracle checks a sample of rows (first, last, tile borders, random).
-@pytest.mark.parametrize("M,N,K", [(4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 512), (4000, 2100, 272),
+@pytest.mark.parametrize("M,N,K", [(4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 512), (4096, 2176, 256), (4000, 2100, 272),
                                    (8192, 2048, 1024)])
 def test_large_m_kernels(gpu, oracle, M, N, K):
     from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
