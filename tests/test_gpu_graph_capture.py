@@ -1,0 +1,74 @@
+"""The operators under HIP graph capture: quantize -> blockwise FP8 GEMM -> INT8 GEMM recorded once on a side stream and
+replayed with new input contents.
+
+What this pins: nothing on the path synchronizes, allocates outside torch's capture-aware allocator or depends on host
+state at replay time (the reference runs these operators inside its decode graphs,
+python/sglang/srt/model_executor/cuda_graph_runner.py:452-540).  Every replay is compared with the eager result of the
+same inputs (bit for bit: same kernels, deterministic reduce order) and the first one with the CPU oracle.  Replays are
+separated by eager work and synchronizations, and the graph holds no memset node of its own (split-K partial sums need no
+clearing).  Shapes cover a split-K decode plan (workspace from torch inside the capture), a mid-M plan with re-laid-out
+token scales, and an unsplit plan.
+"""
+import pytest
+import torch
+
+from sglang_amd.workloads import make_activation, make_fp8_weight, make_int8_weight
+
+pytestmark = pytest.mark.gpu
+
+
+def _linear_chain(x, w_q, w_s, wi_q, wi_s):
+    from sglang_amd.fp8_kernel import per_token_group_quant_fp8, w8a8_block_fp8_matmul
+    from sglang_amd.int8_kernel import per_token_quant_int8
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, int8_scaled_mm
+
+    x_q, x_s = per_token_group_quant_fp8(x, 128, column_major_scales=True)
+    y = fp8_blockwise_scaled_mm(x_q, w_q.t(), x_s, w_s.t(), torch.bfloat16)       # [M, N1]
+    x_q2, x_s2 = per_token_group_quant_fp8(x, 128)                                   # row-major scales: re-layout path
+    y2 = w8a8_block_fp8_matmul(x_q2, w_q, x_s2, w_s, [128, 128], torch.bfloat16)
+    a_q, a_s = per_token_quant_int8(y)
+    z = int8_scaled_mm(a_q, wi_q.t(), a_s, wi_s, torch.bfloat16)                    # [M, N2]
+    return x_q, x_s, y, y2, z
+
+
+@pytest.mark.parametrize("M", [4, 48, 300])
+def test_capture_and_replay_matches_eager(gpu, oracle, M):
+    from sglang_amd import _lib
+
+    K, N1, N2 = 2048, 1024, 512
+    plan = _lib.gemm_plan("fp8", M, N1, K)
+    print(f"case M={M}: fp8 {plan}  int8 {_lib.gemm_plan('int8', M, N2, N1)}", flush=True)
+    w_q, w_s = make_fp8_weight(N1, K, seed=11)
+    wi_q, wi_s = make_int8_weight(N2, N1, seed=12)
+    w_q, w_s, wi_q, wi_s = w_q.to(gpu), w_s.to(gpu), wi_q.to(gpu), wi_s.to(gpu)
+    inputs = [make_activation(M, K, seed=100 + i) for i in range(4)]
+    static_x = inputs[0].to(gpu).clone()
+
+    stream = torch.cuda.Stream()  # default priority
+    with torch.cuda.stream(stream):
+        for _ in range(2):  # warm up allocator, lazy initialisation and operator registration outside the capture
+            _linear_chain(static_x, w_q, w_s, wi_q, wi_s)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            static_out = _linear_chain(static_x, w_q, w_s, wi_q, wi_s)
+    torch.cuda.synchronize()
+
+    for i, x in enumerate(inputs[1:] + inputs[:1]):
+        static_x.copy_(x.to(gpu))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in static_out]
+        # eager work between replays, then the eager result of the same input
+        want = _linear_chain(x.to(gpu), w_q, w_s, wi_q, wi_s)
+        torch.cuda.synchronize()
+        for name, g_, w_ in zip(("x_q", "x_s", "y", "y2", "z"), got, want):
+            assert torch.equal(g_.view(torch.uint8) if g_.dtype == torch.float8_e4m3fn else g_,
+                               w_.view(torch.uint8) if w_.dtype == torch.float8_e4m3fn else w_), (i, name)
+        if i == 0:
+            q_o, s_o = oracle.group_quant(x, 128, mode="div", layout="col")
+            assert torch.equal(got[0].cpu().view(torch.uint8), q_o.view(torch.uint8)) and torch.equal(got[1].cpu(), s_o)
+            ref, mag = oracle.fp8_blockwise_mm(q_o, w_q.cpu(), s_o, w_s.cpu(), torch.float32, want_abs=True)
+            err = (got[2].float().cpu() - ref).abs()
+            assert bool((err <= 1e-2 * ref.abs() + 1e-4 * mag).all())
