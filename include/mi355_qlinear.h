@@ -163,6 +163,45 @@ int mi355_int8_scaled_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char
  */
 int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
 
+/*
+ * Per-token FP8 activation quantization: s[m] = max |x[m,:]| / 448 (no floor), q = e4m3fn(clamp(x * (1 / s[m]))) rounded to
+ * nearest even; a row of zeros gives s = 0 and zeros.
+ * Replaces sgl_per_token_quant_fp8 (sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:162-227, arithmetic of its
+ *          warp-per-token kernel :15-85; its small-batch kernel :91-160 omits the zero test and yields NaN for such a row).
+ *   x [M, K] contiguous F32/F16/BF16; q [M, K] e4m3fn contiguous; s [M] fp32.  K * sizeof(x element) % 16 == 0.
+ */
+int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
+
+/*
+ * Per-token x per-channel FP8 GEMM:  out[m,n] = cast( sa[m] * sb[n] * sum_k a[m,k] * b[n,k] + f32(bias[n]) ), fp32 accumulate.
+ * Replaces fp8_scaled_mm (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532, epilogue :529-547; caller apply_fp8_linear,
+ *          python/sglang/srt/layers/quantization/fp8_utils.py:565-853).
+ *   a [M, K] e4m3fn row stride lda;  b [N, K] e4m3fn row stride ldb (the reference's column-major mat_b [K, N]);
+ *   sa [M], sb [N] fp32 contiguous; bias NULL or [N] in the output dtype; out [M, N] BF16/F16 row stride ldo.
+ *   It runs on the blockwise kernels (token scale applied when a 128-wide K block is promoted, channel scale and bias
+ *   in the epilogue); workspace as for mi355_fp8_blockwise_mm.
+ */
+size_t mi355_fp8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_fp8_scaled_mm(const void* a, const void* b, const float* sa, const float* sb, const void* bias, void* out,
+                        int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldo,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * One block-FP8 linear layer in one call:  out = cast( blockwise_mm(quantize_1x128(x), w) + f32(bias) ).
+ * Replaces the call sequence of cutlass_w8a8_block_fp8_linear_with_fallback / triton_w8a8_block_fp8_linear
+ *          (python/sglang/srt/layers/quantization/fp8_utils.py:184-214, :281-301): per_token_group_quant_fp8, the blockwise
+ *          GEMM and `output += bias`.  The activation is quantized with q = x / s (s = max(amax, 1e-10) / 448) into the
+ *          workspace, with M-major scales, and the bias is added in fp32 in the GEMM epilogue (the reference adds it
+ *          after rounding the GEMM result to the output type).
+ *   x [M, K] contiguous F32/F16/BF16, K % 128 == 0; w [N, K] e4m3fn row stride ldw; w_scale element (nb, kb) at
+ *   w_scale[nb * ws_sn + kb * ws_sk]; bias NULL or [N] in the output dtype; out [M, N] BF16/F16 row stride ldo.
+ *   workspace: mi355_fp8_block_linear_workspace_bytes(M, N, K) bytes, 256-byte aligned.
+ */
+size_t mi355_fp8_block_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w, const float* w_scale, int64_t ws_sn, int64_t ws_sk,
+                           const void* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldw,
+                           int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

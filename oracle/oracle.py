@@ -57,6 +57,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_group_quant.restype = i32
         L.oracle_per_token_quant_int8.argtypes = [vp, i32, vp, vp, i64, i64]
         L.oracle_per_token_quant_int8.restype = i32
+        L.oracle_per_token_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64]
+        L.oracle_per_token_quant_fp8.restype = i32
+        L.oracle_fp8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32, vp] + [i64] * 6
+        L.oracle_fp8_scaled_mm.restype = i32
         L.oracle_fp8_blockwise_mm.argtypes = [vp, vp, vp, vp, vp, i32, vp] + [i64] * 10
         L.oracle_fp8_blockwise_mm.restype = i32
         L.oracle_int8_mm_acc.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64]
@@ -166,6 +170,37 @@ def per_token_quant_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     rc = lib().oracle_per_token_quant_int8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), M, K)
     assert rc == 0
     return q, s
+
+
+def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x [M,K] -> (e4m3fn [M,K], fp32 scales [M,1]); scale = max|x| / 448, zero rows give scale 0 and zeros."""
+    x = _cpu(x)
+    assert x.dim() == 2 and x.is_contiguous()
+    M, K = x.shape
+    q = torch.zeros(M, K, dtype=torch.uint8)
+    s = torch.zeros(M, 1, dtype=torch.float32)
+    rc = lib().oracle_per_token_quant_fp8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), M, K)
+    assert rc == 0
+    return q.view(torch.float8_e4m3fn), s
+
+
+def fp8_scaled_mm(a, w, sa, sb, out_dtype=torch.bfloat16, bias: Optional[torch.Tensor] = None, want_abs: bool = False):
+    """a [M,K] fp8, w [N,K] fp8 (weight as stored), sa [M], sb [N], bias [N] in the output dtype or None ->
+    out [M,N] = cast(sa[m] * (sb[n] * sum_k a*w) + bias[n]); with want_abs also the fp32 magnitude matrix."""
+    a, w, sa, sb = _cpu(a), _cpu(w), _cpu(sa).reshape(-1), _cpu(sb).reshape(-1)
+    M, K = a.shape
+    N = w.shape[0]
+    assert w.shape[1] == K and a.stride(1) == 1 and w.stride(1) == 1 and sa.numel() == M and sb.numel() == N
+    if bias is not None:
+        bias = _cpu(bias)
+        assert bias.dtype == out_dtype and bias.numel() == N
+    out = torch.zeros(M, N, dtype=out_dtype)
+    ab = torch.zeros(M, N, dtype=torch.float32) if want_abs else None
+    rc = lib().oracle_fp8_scaled_mm(
+        a.data_ptr(), w.data_ptr(), sa.data_ptr(), sb.data_ptr(), bias.data_ptr() if bias is not None else None,
+        out.data_ptr(), _DT[out_dtype], ab.data_ptr() if want_abs else None, M, N, K, a.stride(0), w.stride(0), out.stride(0))
+    assert rc == 0
+    return (out, ab) if want_abs else out
 
 
 def fp8_blockwise_mm(

@@ -23,6 +23,8 @@
  *                             sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:449-476 (sm90 order),
  *                             sgl-kernel/tests/test_int8_gemm.py:11-17 (torch order)
  *   oracle_per_token_quant_int8  python/sglang/srt/layers/quantization/int8_kernel.py:28-52
+ *   oracle_per_token_quant_fp8   sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85
+ *   oracle_fp8_scaled_mm         sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:529-547, :1450-1532
  *
  * Parity status: every function here is pinned by tests/test_oracle_*.py against
  * torch's CPU float8/bfloat16/half conversions, torch fp32/fp64 matmul, exact
@@ -168,6 +170,14 @@ static inline float load_as_f32(const void* p, int dtype, size_t i) {
   }
 }
 
+static inline void store_from_f32(void* p, int dtype, size_t i, float v) {
+  switch (dtype) {
+    case DT_F32: ((float*)p)[i] = v; break;
+    case DT_F16: ((uint16_t*)p)[i] = oracle_f32_to_f16(v); break;
+    default: ((uint16_t*)p)[i] = oracle_f32_to_bf16(v);
+  }
+}
+
 /* ceil(log2(x)) for a positive normal float, by its bits:
  * per_token_group_quant_8bit_v2.cu:61-66 (fast_log2_ceil). */
 static inline int log2_ceil_bits(float x) {
@@ -264,6 +274,59 @@ int oracle_per_token_quant_int8(const void* x, int x_dtype, int8_t* q, float* s,
     for (int64_t j = 0; j < K; ++j) {
       float t = load_as_f32(x, x_dtype, (size_t)row * K + j) * mul;
       q[(size_t)row * K + j] = (int8_t)roundf(t);
+    }
+  }
+  return 0;
+}
+
+/* x [M, K] -> q e4m3fn [M, K], s float [M]:  s = max|x| / 448 (no floor), q = RNE(clamp(x * (1 / s), -448, 448)),
+ * and a row of zeros gives s = 0, q = 0 (sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85, the warp-per-token kernel;
+ * its small-batch sibling :91-160 divides by the scale without the zero test and would produce NaN for such a row). */
+int oracle_per_token_quant_fp8(const void* x, int x_dtype, uint8_t* q, float* s, int64_t M, int64_t K) {
+#pragma omp parallel for schedule(static)
+  for (int64_t row = 0; row < M; ++row) {
+    float amax = 0.f;
+    for (int64_t j = 0; j < K; ++j) amax = fmaxf(amax, fabsf(load_as_f32(x, x_dtype, (size_t)row * K + j)));
+    const float scale = amax / 448.0f;
+    s[row] = scale;
+    const float inv = (scale == 0.f) ? 0.f : 1.0f / scale;
+    for (int64_t j = 0; j < K; ++j) {
+      float t = load_as_f32(x, x_dtype, (size_t)row * K + j) * inv;
+      t = fmaxf(fminf(t, 448.0f), -448.0f);
+      q[(size_t)row * K + j] = oracle_e4m3fn_encode(t);
+    }
+  }
+  return 0;
+}
+
+/*
+ * Per-token x per-channel FP8 GEMM:  out[m, n] = cast( sa[m] * (sb[n] * sum_k a[m,k] * b[n,k]) + bias[n] )
+ * (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532; epilogue order of its sm90 visitor tree :529-547: the weight scale
+ * multiplies the accumulator, the token scale multiplies that, the bias is added in the same fused step).  The sum over
+ * K is exact in double here; bias, if any, has the output dtype.  abs_out, if not NULL, receives
+ * |sa[m] * sb[n]| * sum_k |a * b| (fp32).
+ */
+int oracle_fp8_scaled_mm(const uint8_t* a, const uint8_t* b, const float* sa, const float* sb, const void* bias, void* out,
+                         int out_dtype, float* abs_out, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                         int64_t ldo) {
+  float lut[256];
+  for (int i = 0; i < 256; ++i) lut[i] = oracle_e4m3fn_decode((uint8_t)i);
+#pragma omp parallel for schedule(static) collapse(2)
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t n = 0; n < N; ++n) {
+      double acc = 0.0, mag = 0.0;
+      const uint8_t* ar = a + m * lda;
+      const uint8_t* br = b + n * ldb;
+      for (int64_t k = 0; k < K; ++k) {
+        const double prod = (double)lut[ar[k]] * (double)lut[br[k]];
+        acc += prod;
+        mag += fabs(prod);
+      }
+      float t = sb[n] * (float)acc;
+      t = sa[m] * t;
+      if (bias) t = t + load_as_f32(bias, out_dtype, (size_t)n);
+      store_from_f32(out, out_dtype, (size_t)(m * ldo + n), t);
+      if (abs_out) abs_out[m * N + n] = fabsf(sa[m] * sb[n]) * (float)mag;
     }
   }
   return 0;

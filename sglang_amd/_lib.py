@@ -31,6 +31,11 @@ EXPORTS = (
     "mi355_fp8_blockwise_mm_plan",
     "mi355_int8_scaled_mm_plan",
     "mi355_per_token_quant_int8",
+    "mi355_per_token_quant_fp8",
+    "mi355_fp8_scaled_mm_workspace_bytes",
+    "mi355_fp8_scaled_mm",
+    "mi355_fp8_block_linear_workspace_bytes",
+    "mi355_fp8_block_linear",
 )
 
 _lib = None
@@ -78,6 +83,16 @@ def lib() -> ctypes.CDLL:
         fn.restype = i32
     L.mi355_per_token_quant_int8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
     L.mi355_per_token_quant_int8.restype = i32
+    L.mi355_per_token_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
+    L.mi355_per_token_quant_fp8.restype = i32
+    L.mi355_fp8_scaled_mm_workspace_bytes.argtypes = [i64, i64, i64]
+    L.mi355_fp8_scaled_mm_workspace_bytes.restype = sz
+    L.mi355_fp8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32] + [i64] * 6 + [vp, sz, vp]
+    L.mi355_fp8_scaled_mm.restype = i32
+    L.mi355_fp8_block_linear_workspace_bytes.argtypes = [i64, i64, i64]
+    L.mi355_fp8_block_linear_workspace_bytes.restype = sz
+    L.mi355_fp8_block_linear.argtypes = [vp, i32, vp, vp, i64, i64, vp, vp, i32] + [i64] * 5 + [vp, sz, vp]
+    L.mi355_fp8_block_linear.restype = i32
     got = L.mi355_qlinear_abi_version()
     if got != ABI_VERSION:
         raise ImportError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}: rebuild it")

@@ -22,7 +22,8 @@ struct GemmParams {
   const uint8_t* b;  // channels [N, K], row stride ldb
   const float* sa;
   const float* sb;
-  const void* bias;
+  const void* bias;        // optional [N] in the output dtype (INT8 GEMM; per-channel FP8 epilogue)
+  const float* col_scale;  // FP8 only, optional [N]: per-channel scale applied in the epilogue (fp8_scaled_mm)
   void* out;
   void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
   int M, N, K;
@@ -94,6 +95,31 @@ __device__ __forceinline__ void out_tile_store(const uint8_t* tile, void* out, i
 __device__ __forceinline__ bool out_tile_ok(const void* out, int64_t ldo, int out_dtype, int n0, int N) {
   return (out_dtype == MI355_BF16 || out_dtype == MI355_F16) && (ldo & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
          n0 + 256 <= N;
+}
+
+// Optional per-channel epilogue of the FP8 kernels: r[v] = col_scale[n + v] * r[v] + bias[n + v] for the four consecutive
+// channels n .. n + 3 (channels at or past N repeat the last one; they are never stored).
+__device__ __forceinline__ void fp8_channel_epilogue(const GemmParams& p, int n, float* r) {
+  if (p.col_scale == nullptr && p.bias == nullptr) return;
+  const bool whole = n + 4 <= p.N;
+  if (p.col_scale) {
+    if (whole && (reinterpret_cast<uintptr_t>(p.col_scale + n) & 15) == 0) {
+      const v4f c = *reinterpret_cast<const v4f*>(p.col_scale + n);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) r[v] = c[v] * r[v];
+    } else {
+#pragma unroll
+      for (int v = 0; v < 4; ++v) r[v] = p.col_scale[min(n + v, p.N - 1)] * r[v];
+    }
+  }
+  if (p.bias) {
+    const uint16_t* b = reinterpret_cast<const uint16_t*>(p.bias);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const uint32_t h = b[min(n + v, p.N - 1)];
+      r[v] += (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+    }
+  }
 }
 
 struct TileCoord {

@@ -259,6 +259,7 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
 #pragma unroll
           for (int v = 0; v < 4; ++v) wsp[v] = acc[i][v];
         } else if constexpr (IS_FP8) {
+          fp8_channel_epilogue(p, n, acc[i]);
           store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, acc[i], 4, vec_ok);
         } else if (p.out_dtype == MI355_I32) {
           int* o = reinterpret_cast<int*>(p.out) + (int64_t)l16 * p.ldo + n;

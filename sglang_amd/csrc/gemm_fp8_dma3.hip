@@ -247,6 +247,7 @@ __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmPara
         for (int v = 0; v < 4; ++v)
           if (v < nvalid) wsp[v] = acc[i][j][v];
       } else {
+        fp8_channel_epilogue(p, n, acc[i][j]);
         store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
       }
     }

@@ -256,6 +256,7 @@ __global__ __launch_bounds__(THREADS) void fp8_gemm_pipelined_kernel(const GemmP
     for (int i = 0; i < P_NT; ++i) {
       const int n = n0 + wave_n * P_WN + i * 16 + 4 * q;
       if (n >= p.N) continue;
+      fp8_channel_epilogue(p, n, acc[i][j]);
       store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], min(4, p.N - n), vec_ok);
     }
   }

@@ -319,8 +319,10 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
 #pragma unroll
     for (int j = 0; j < G_MT; ++j)
 #pragma unroll
-      for (int i = 0; i < G_NT; ++i)
+      for (int i = 0; i < G_NT; ++i) {
+        fp8_channel_epilogue(p, n0 + wave_n * G_WN + i * 16 + 4 * q, acc[i][j]);
         out_tile_put4(g_stages, grp * G_WM + j * 16 + l16, wave_n * G_WN + i * 16 + 4 * q, p.out_dtype, acc[i][j]);
+      }
     __syncthreads();
     out_tile_store(g_stages, p.out, p.ldo, m0, n0, p.M);
     return;
@@ -334,6 +336,7 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
     for (int i = 0; i < G_NT; ++i) {
       const int n = n0 + wave_n * G_WN + i * 16 + 4 * q;
       if (n >= p.N) continue;
+      fp8_channel_epilogue(p, n, acc[i][j]);
       store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], min(4, p.N - n), vec_ok);
     }
   }

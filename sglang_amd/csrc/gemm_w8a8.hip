@@ -224,6 +224,7 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const GemmParams p) {
         for (int v = 0; v < 4; ++v)
           if (v < nvalid) w[v] = acc[i][j][v];
       } else if constexpr (IS_FP8) {
+        fp8_channel_epilogue(p, n, acc[i][j]);
         store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
       } else {
         if (p.out_dtype == MI355_I32) {
@@ -267,7 +268,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
       const v4f t = *reinterpret_cast<const v4f*>(w + (int64_t)k * total);
       s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
     }
-    const float r[4] = {s[0], s[1], s[2], s[3]};
+    float r[4] = {s[0], s[1], s[2], s[3]};
+    fp8_channel_epilogue(p, n, r);
     const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
     store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
   } else {
@@ -675,6 +677,109 @@ extern "C" int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, cons
   }
   // every partial sum that the reduce kernel reads is written by this call first, so nothing has to be cleared
   return run_gemm<true>(p, ws, need > 0 ? NOALLOC_SCRATCH_BYTES : 0, static_cast<hipStream_t>(stream), what);
+}
+
+namespace {
+
+// A weight-block scale of one for the per-token x per-channel FP8 GEMM, which runs on the blockwise kernels: every block
+// reads this same float (strides 0).  Device address looked up once per device, like the scratch array above.
+static __device__ __align__(16) float unit_scale[4] = {1.f, 1.f, 1.f, 1.f};
+void* unit_scale_ptr[MAX_DEVICES];  // guarded by scratch_mutex
+
+int unit_scale_of_current_device(const float** ptr, const char* what) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    set_error("%s: cannot identify the current device (%s, device %d)", what, hipGetErrorString(e), dev);
+    return MI355_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (unit_scale_ptr[dev] == nullptr) {
+    void* q = nullptr;
+    e = hipGetSymbolAddress(&q, HIP_SYMBOL(unit_scale));
+    if (e != hipSuccess || q == nullptr) {
+      set_error("%s: cannot resolve a device constant on device %d: %s", what, dev, hipGetErrorString(e));
+      return MI355_ERR_LAUNCH;
+    }
+    unit_scale_ptr[dev] = q;
+  }
+  *ptr = static_cast<const float*>(unit_scale_ptr[dev]);
+  return MI355_OK;
+}
+
+}  // namespace
+
+extern "C" size_t mi355_fp8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return workspace_bytes(M, N, K, true);
+}
+
+extern "C" int mi355_fp8_scaled_mm(const void* a, const void* b, const float* sa, const float* sb, const void* bias,
+                                   void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                   int64_t ldo, void* workspace, size_t workspace_bytes_given, void* stream) {
+  const char* what = "mi355_fp8_scaled_mm";
+  clear_error();
+  MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16, MI355_ERR_INVALID_ARGUMENT,
+                "%s: out_dtype must be bfloat16 or float16", what);
+  const float* one = nullptr;
+  if (M > 0 && N > 0) {
+    const int rc1 = unit_scale_of_current_device(&one, what);
+    if (rc1 != MI355_OK) return rc1;
+  }
+  GemmParams p;
+  bool empty;
+  // token scale: one value per token for every K block (stride 0 along K); weight-block scale: one
+  const int rc = fp8_mm_params(what, a, b, sa, one, out, out_dtype, M, N, K, lda, ldb, /*sa_sm*/ 1, /*sa_sk*/ 0, 0, 0, ldo, p, empty);
+  if (rc != MI355_OK || empty) return rc;
+  MI355_REQUIRE(sb != nullptr, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  p.col_scale = sb;
+  p.bias = bias;
+  return run_gemm<true>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
+}
+
+namespace {
+size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+}  // namespace
+
+extern "C" size_t mi355_fp8_block_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const size_t kb = (size_t)((K + KSTEP - 1) / KSTEP);
+  return align256((size_t)M * (size_t)K) + align256((size_t)((M + 3) & ~3ll) * kb * 4u) + workspace_bytes(M, N, K, true);
+}
+
+extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w, const float* w_scale, int64_t ws_sn,
+                                      int64_t ws_sk, const void* bias, void* out, int out_dtype, int64_t M, int64_t N,
+                                      int64_t K, int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes_given,
+                                      void* stream) {
+  const char* what = "mi355_fp8_block_linear";
+  clear_error();
+  MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
+  MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16, MI355_ERR_INVALID_ARGUMENT,
+                "%s: out_dtype must be bfloat16 or float16", what);
+  if (M == 0 || N == 0) return MI355_OK;
+  MI355_REQUIRE(K > 0 && K % KSTEP == 0, MI355_ERR_INVALID_ARGUMENT,
+                "%s: K must be a positive multiple of the quantization group (128)", what);
+  MI355_REQUIRE(x && w && w_scale && out, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  const size_t need = mi355_fp8_block_linear_workspace_bytes(M, N, K);
+  MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
+                "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
+  MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, MI355_ERR_WORKSPACE,
+                "%s: workspace must be 256-byte aligned", what);
+  // workspace: [codes M x K][token scales, M-major, pitch align4(M)][what the GEMM needs]
+  uint8_t* q = static_cast<uint8_t*>(workspace);
+  const size_t q_bytes = align256((size_t)M * (size_t)K);
+  float* sa = reinterpret_cast<float*>(q + q_bytes);
+  const int64_t pitch = (M + 3) & ~3ll;
+  const size_t sa_bytes = align256((size_t)pitch * (size_t)(K / KSTEP) * 4u);
+  // quantize with q = x / s, the arithmetic of the reference's column-major path (fp8_kernel.py:164-212 via fp8_utils.py:201-203)
+  int rc = mi355_group_quant_8bit(x, x_dtype, q, MI355_FP8_E4M3FN, sa, M, K, KSTEP, 1e-10f, -448.0f, 448.0f, MI355_QUANT_DIV,
+                                  MI355_SCALE_F32, 0.0f, 1, pitch, stream);
+  if (rc != MI355_OK) return rc;
+  GemmParams p;
+  bool empty;
+  rc = fp8_mm_params(what, q, w, sa, w_scale, out, out_dtype, M, N, K, K, ldw, 1, pitch, ws_sn, ws_sk, ldo, p, empty);
+  if (rc != MI355_OK || empty) return rc;
+  p.bias = bias;
+  return run_gemm<true>(p, q + q_bytes + sa_bytes, workspace_bytes_given - q_bytes - sa_bytes, static_cast<hipStream_t>(stream), what);
 }
 
 extern "C" size_t mi355_int8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {

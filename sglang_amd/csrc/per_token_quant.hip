@@ -1,8 +1,11 @@
-// Per-token (per-row) symmetric INT8 quantizer for gfx950.
+// Per-token (per-row) symmetric 8-bit quantizers for gfx950.
 //
 // One workgroup per row: 16-byte loads, |x| max over the row (DPP inside a wave, LDS across the four
-// waves), then q = round-half-away(x * (127 / absmax)) with absmax floored at 1e-10 and
-// scale = absmax / 127, as in python/sglang/srt/layers/quantization/int8_kernel.py:47-50.
+// waves), then
+//   INT8: q = round-half-away(x * (127 / absmax)) with absmax floored at 1e-10 and scale = absmax / 127, as in
+//         python/sglang/srt/layers/quantization/int8_kernel.py:47-50;
+//   FP8:  scale = absmax / 448 (no floor), q = e4m3fn(clamp(x * (1 / scale))) rounded to nearest even, a row of zeros
+//         gives scale 0 and zeros, as in sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85.
 // Rows of up to 8192 two-byte elements stay in registers between the two phases; longer rows are
 // re-read (from L2).
 #include "common.h"
@@ -47,8 +50,8 @@ __device__ __forceinline__ float wave_allreduce_max(float v) {
   return r;
 }
 
-template <int DT>
-__global__ __launch_bounds__(256) void per_token_quant_int8_kernel(const void* x, int8_t* q, float* s, int64_t K) {
+template <int DT, bool FP8_OUT>
+__global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int8_t* q, float* s, int64_t K) {
   constexpr int VEC = (DT == MI355_F32) ? 4 : 8;
   constexpr int KEEP = 4;  // vectors per thread kept in registers
   __shared__ float wave_max[4];
@@ -56,7 +59,7 @@ __global__ __launch_bounds__(256) void per_token_quant_int8_kernel(const void* x
   const int64_t nvec = K / VEC;
   const u32x4* src = reinterpret_cast<const u32x4*>(x) + row * nvec;
   u32x4 keep[KEEP];
-  float amax = 1e-10f;
+  float amax = FP8_OUT ? 0.f : 1e-10f;
 #pragma unroll
   for (int i = 0; i < KEEP; ++i) {
     const int64_t v = threadIdx.x + 256 * i;
@@ -76,8 +79,15 @@ __global__ __launch_bounds__(256) void per_token_quant_int8_kernel(const void* x
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = amax;
   __syncthreads();
   amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-  if (threadIdx.x == 0) s[row] = amax / 127.0f;
-  const float mul = 127.0f / amax;
+  float mul;
+  if constexpr (FP8_OUT) {
+    const float scale = amax / 448.0f;
+    if (threadIdx.x == 0) s[row] = scale;
+    mul = (scale == 0.f) ? 0.f : 1.0f / scale;
+  } else {
+    if (threadIdx.x == 0) s[row] = amax / 127.0f;
+    mul = 127.0f / amax;
+  }
 
   auto emit = [&](const u32x4& raw, int64_t v) {
     float f[VEC];
@@ -86,8 +96,17 @@ __global__ __launch_bounds__(256) void per_token_quant_int8_kernel(const void* x
 #pragma unroll
     for (int j = 0; j < VEC / 4; ++j) {
       uint32_t pk = 0;
+      if constexpr (FP8_OUT) {
+        float t[4];
 #pragma unroll
-      for (int b = 0; b < 4; ++b) pk |= ((uint32_t)(int)roundf(f[4 * j + b] * mul) & 0xffu) << (8 * b);
+        for (int b = 0; b < 4; ++b) t[b] = fmaxf(fminf(f[4 * j + b] * mul, 448.0f), -448.0f);
+        int c = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
+        c = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c, true);
+        pk = (uint32_t)c;
+      } else {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) pk |= ((uint32_t)(int)roundf(f[4 * j + b] * mul) & 0xffu) << (8 * b);
+      }
       w[j] = pk;
     }
     int8_t* d = q + row * K + v * VEC;
@@ -107,10 +126,11 @@ __global__ __launch_bounds__(256) void per_token_quant_int8_kernel(const void* x
 }  // namespace
 }  // namespace mi355
 
-extern "C" int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K,
-                                          void* stream) {
-  using namespace mi355;
-  const char* what = "mi355_per_token_quant_int8";
+namespace mi355 {
+namespace {
+
+template <bool FP8_OUT>
+int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream) {
   clear_error();
   MI355_REQUIRE(M >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
   MI355_REQUIRE(x_dtype == MI355_F32 || x_dtype == MI355_F16 || x_dtype == MI355_BF16, MI355_ERR_INVALID_ARGUMENT,
@@ -126,13 +146,26 @@ extern "C" int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, f
   int8_t* qq = static_cast<int8_t*>(q);
   switch (x_dtype) {
     case MI355_F32:
-      hipLaunchKernelGGL(per_token_quant_int8_kernel<MI355_F32>, dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F32, FP8_OUT>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
       break;
     case MI355_F16:
-      hipLaunchKernelGGL(per_token_quant_int8_kernel<MI355_F16>, dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F16, FP8_OUT>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
       break;
     default:
-      hipLaunchKernelGGL(per_token_quant_int8_kernel<MI355_BF16>, dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_BF16, FP8_OUT>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
   }
   return check_launch(what);
+}
+
+}  // namespace
+}  // namespace mi355
+
+extern "C" int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K,
+                                          void* stream) {
+  return mi355::per_token_quant<false>("mi355_per_token_quant_int8", x, x_dtype, q, s, M, K, stream);
+}
+
+extern "C" int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K,
+                                         void* stream) {
+  return mi355::per_token_quant<true>("mi355_per_token_quant_fp8", x, x_dtype, q, s, M, K, stream);
 }

@@ -179,6 +179,17 @@ def sglang_per_token_group_quant_fp8(
     return x_q, x_s
 
 
+def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
+    """fp8_kernel.py:573-589: one scale per row, ``(x_q, x_s [M, 1])``."""
+    assert x.is_contiguous(), "`x` is not contiguous"
+    x_q = torch.empty_like(x, device=x.device, dtype=dtype)
+    x_s = torch.empty(x.shape[0], 1, device=x.device, dtype=torch.float32)
+    from .sgl_kernel import sgl_per_token_quant_fp8
+
+    sgl_per_token_quant_fp8(x, x_q, x_s)
+    return x_q, x_s
+
+
 def sglang_per_token_group_quant_int8(
     x: torch.Tensor,
     group_size: int,

@@ -36,6 +36,9 @@ SCHEMAS = {
     "sgl_per_token_group_quant_8bit_v2": "sgl_per_token_group_quant_8bit_v2(Tensor input, Tensor output_q, "
     "Tensor output_s, int group_size, float eps, float fp8_min, float fp8_max, bool scale_ue8m0, "
     "bool fuse_silu_and_mul, Tensor? masked_m) -> ()",
+    "fp8_scaled_mm": "fp8_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, "
+    "Tensor? bias) -> Tensor",
+    "sgl_per_token_quant_fp8": "sgl_per_token_quant_fp8(Tensor input, Tensor output_q, Tensor output_s) -> ()",
 }
 
 
@@ -176,6 +179,99 @@ def block_fp8_matmul(A2d, B, As2d, Bs, out2d):
     return out2d
 
 
+def _workspace(nbytes: int, device) -> Optional[torch.Tensor]:
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+
+
+# ---------------------------------------------------------------- per-token x per-channel FP8 linear
+
+def sgl_per_token_quant_fp8(input, output_q, output_s):
+    """sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:162-227."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _check_input(output_s, "output_s")
+    _require(input.dim() == 2, "sgl_per_token_quant_fp8: input must be 2-D")
+    M, K = input.shape
+    _require(K % 8 == 0, f"Hidden dimension must be divisible by 8, but got {K}")
+    _require(input.dtype in (torch.float32, torch.float16, torch.bfloat16), "sgl_per_token_quant_fp8: unsupported input dtype")
+    _require(output_q.dtype == torch.float8_e4m3fn and output_q.numel() == input.numel(), "sgl_per_token_quant_fp8: output_q mismatch")
+    _require(output_s.dtype == torch.float32 and output_s.numel() == M, "sgl_per_token_quant_fp8: output_s mismatch")
+    if M:
+        check(lib().mi355_per_token_quant_fp8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), output_s.data_ptr(),
+                                              M, K, _stream()))
+
+
+def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[torch.Tensor] = None):
+    """sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532."""
+    _require(mat_a.is_cuda, "mat_a must be a CUDA tensor")
+    _require(mat_b.is_cuda, "mat_b must be a CUDA tensor")
+    _require(mat_a.dim() == 2, "mat_a must be a 2D tensor")
+    _require(mat_b.dim() == 2, "mat_b must be a 2D tensor")
+    _require(mat_a.stride(1) == 1, "mat_a must be a row major tensor")
+    _require(mat_b.stride(0) == 1, "mat_b must be a column major tensor")
+    _require(mat_a.size(1) == mat_b.size(0), "mat_a and mat_b shapes cannot be multiplied")
+    _require((mat_a.size(1) * mat_a.element_size()) % 16 == 0, "mat_a must be multiple of 16 bytes for memory alignment")
+    _require((mat_b.size(0) * mat_b.element_size()) % 16 == 0, "mat_b must be multiple of 16 bytes for memory alignment")
+    _require(mat_a.dtype == torch.float8_e4m3fn, "mat_a must be Float8_e4m3fn")
+    _require(mat_b.dtype == torch.float8_e4m3fn, "mat_b must be Float8_e4m3fn")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be Half or BFloat16")
+    M, K = mat_a.shape
+    N = mat_b.size(1)
+    _require(scales_a.numel() == M, "size of scales_a is not matched")
+    _require(scales_b.numel() == N, "size of scales_b is not matched")
+    _require(scales_a.is_contiguous(), "scales_a must be contiguous")
+    _require(scales_b.is_contiguous(), "scales_b msut be contiguous")
+    _require(scales_a.dtype == torch.float32, "scales_a must be Float32")
+    _require(scales_b.dtype == torch.float32, "scales_b must be Float32")
+    if bias is not None:
+        _require(bias.numel() == N, "size of bias is not matched")
+        _require(bias.is_contiguous(), "bias must be contiguous")
+        _require(bias.dtype == out_dtype, "bias dtype must match output dtype")
+    out = torch.empty((M, N), dtype=out_dtype, device=mat_a.device)
+    _require((N * out.element_size()) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    if M == 0:
+        return out
+    L = lib()
+    ws_bytes = L.mi355_fp8_scaled_mm_workspace_bytes(M, N, K)
+    ws = _workspace(ws_bytes, mat_a.device)
+    check(L.mi355_fp8_scaled_mm(mat_a.data_ptr(), mat_b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(),
+                                bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype], M, N, K,
+                                mat_a.stride(0), mat_b.stride(1), out.stride(0),
+                                ws.data_ptr() if ws is not None else None, ws_bytes, _stream()))
+    return out
+
+
+def block_fp8_linear(x2d: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                     bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+    """One block-FP8 linear layer (1x128 activation groups, 128x128 weight blocks) in one C-ABI call: the activation is
+    quantized into the workspace, multiplied, and the bias is added in the GEMM epilogue.  x2d [M, K] contiguous
+    bf16/fp16/fp32 with K % 128 == 0, weight [N, K] e4m3fn, weight_scale [ceil(N/128), K/128] (any strides)."""
+    _require(x2d.is_cuda and weight.is_cuda, "block_fp8_linear: operands must be CUDA tensors")
+    _require(x2d.dim() == 2 and x2d.is_contiguous(), "block_fp8_linear: x must be a contiguous 2-D tensor")
+    _require(weight.dim() == 2 and weight.stride(1) == 1 and weight.dtype == torch.float8_e4m3fn,
+             "block_fp8_linear: weight must be a row-major Float8_e4m3fn matrix")
+    M, K = x2d.shape
+    N = weight.size(0)
+    _require(weight.size(1) == K and K % 128 == 0, "block_fp8_linear: K must match and be a multiple of 128")
+    _require(tuple(weight_scale.shape) == ((N + 127) // 128, K // 128) and weight_scale.dtype == torch.float32,
+             "block_fp8_linear: weight_scale must be float32 [ceil(N/128), K/128]")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "block_fp8_linear: out_dtype must be Half or BFloat16")
+    if bias is not None:
+        _require(bias.numel() == N and bias.is_contiguous() and bias.dtype == out_dtype,
+                 "block_fp8_linear: bias must be a contiguous [N] tensor of the output dtype")
+    out = torch.empty((M, N), dtype=out_dtype, device=x2d.device)
+    if M == 0:
+        return out
+    L = lib()
+    ws_bytes = L.mi355_fp8_block_linear_workspace_bytes(M, N, K)
+    ws = _workspace(ws_bytes, x2d.device)
+    check(L.mi355_fp8_block_linear(x2d.data_ptr(), _DT[x2d.dtype], weight.data_ptr(), weight_scale.data_ptr(),
+                                   weight_scale.stride(0), weight_scale.stride(1),
+                                   bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype],
+                                   M, N, K, weight.stride(0), out.stride(0), ws.data_ptr(), ws_bytes, _stream()))
+    return out
+
+
 # ---------------------------------------------------------------- INT8 GEMM
 
 def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[torch.Tensor] = None):
@@ -263,6 +359,8 @@ def register() -> None:
         "fp8_blockwise_scaled_mm": fp8_blockwise_scaled_mm,
         "sgl_per_token_group_quant_8bit": sgl_per_token_group_quant_8bit,
         "sgl_per_token_group_quant_8bit_v2": sgl_per_token_group_quant_8bit_v2,
+        "fp8_scaled_mm": fp8_scaled_mm,
+        "sgl_per_token_quant_fp8": sgl_per_token_quant_fp8,
     }
     for name, fn in impls.items():
         if not hasattr(torch.ops.sgl_kernel, name):
@@ -274,6 +372,8 @@ def register() -> None:
 
     torch.library.register_fake("sgl_kernel::int8_scaled_mm", _fake_mm, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::fp8_blockwise_scaled_mm", _fake_mm, lib=_torch_lib)
+    torch.library.register_fake("sgl_kernel::fp8_scaled_mm", _fake_mm, lib=_torch_lib)
+    torch.library.register_fake("sgl_kernel::sgl_per_token_quant_fp8", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit_v2", lambda *a: None, lib=_torch_lib)
     _registered = True

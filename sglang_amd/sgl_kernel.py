@@ -1,5 +1,5 @@
 """Python wrappers with the names, arguments and defaults of ``sgl_kernel`` for this path
-(sgl-kernel/python/sgl_kernel/gemm.py:14-32, :101-142).  Each goes through
+(sgl-kernel/python/sgl_kernel/gemm.py:14-43, :101-161).  Each goes through
 ``torch.ops.sgl_kernel.<op>.default`` exactly like the reference's wrappers do."""
 from __future__ import annotations
 
@@ -24,6 +24,14 @@ def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
 
 def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
     return torch.ops.sgl_kernel.fp8_blockwise_scaled_mm.default(mat_a, mat_b, scales_a, scales_b, out_dtype)
+
+
+def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    return torch.ops.sgl_kernel.fp8_scaled_mm.default(mat_a, mat_b, scales_a, scales_b, out_dtype, bias)
+
+
+def sgl_per_token_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor) -> None:
+    torch.ops.sgl_kernel.sgl_per_token_quant_fp8.default(input, output_q, output_s)
 
 
 def sgl_per_token_group_quant_8bit(

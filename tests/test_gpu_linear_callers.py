@@ -7,10 +7,13 @@ from sglang_amd.workloads import make_activation, make_fp8_weight, make_int8_wei
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("shape,N,K", [((2, 5), 384, 512), ((16,), 2048, 7168), ((3, 7), 576, 1024), ((300,), 1088, 384)])
+@pytest.mark.parametrize("shape,N,K", [((2, 5), 384, 512), ((16,), 2048, 7168), ((3, 7), 576, 1024), ((300,), 1088, 384),
+                                       ((1,), 7168, 2048), ((4100,), 1024, 256)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
-    from sglang_amd.fp8_utils import dispatch_w8a8_block_fp8_linear, triton_w8a8_block_fp8_linear
+    """One-call block-FP8 linear (quantize into the workspace, GEMM, bias in the epilogue) against the same pipeline on
+    the oracle: q = x / s activation codes, blockwise GEMM in fp32, bias added in fp32, one rounding to bf16."""
+    from sglang_amd import fp8_utils
 
     M = 1
     for d in shape:
@@ -19,18 +22,31 @@ def test_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
     w_q, w_s = make_fp8_weight(N, K)
     g = torch.Generator().manual_seed(1)
     bias = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
-    for fn, mode in ((dispatch_w8a8_block_fp8_linear(), "div" if N % 128 == 0 else "rcp"), (triton_w8a8_block_fp8_linear, "rcp")):
+    assert fp8_utils.dispatch_w8a8_block_fp8_linear() is fp8_utils.w8a8_block_fp8_linear
+    for fn in (fp8_utils.cutlass_w8a8_block_fp8_linear_with_fallback, fp8_utils.triton_w8a8_block_fp8_linear):
         out = fn(x.to(gpu), w_q.to(gpu), [128, 128], w_s.to(gpu), None, bias.to(gpu) if with_bias else None)
         assert out.dtype == torch.bfloat16 and tuple(out.shape) == (*shape, N)
-        xq, xs = oracle.group_quant(x.view(M, K), 128, mode=mode)
+        xq, xs = oracle.group_quant(x.view(M, K), 128, mode="div")
         ref, mag = oracle.fp8_blockwise_mm(xq, w_q, xs, w_s, torch.float32, want_abs=True)
-        want = ref.to(torch.bfloat16)
-        if with_bias:
-            want = want + bias  # bf16 += bf16, as the reference does after the GEMM
-        err = (out.float().cpu().view(M, N) - want.float()).abs()
-        # the GEMM result is rounded to bf16 before the bias is added, so its rounding is relative to |ref|, not to the sum
-        tol = 1e-2 * want.float().abs() + 1e-4 * mag + (2.0 ** -7 * (ref.abs() + bias.float().abs()[None, :]) if with_bias else 0)
+        want = ref + bias.float()[None, :] if with_bias else ref
+        err = (out.float().cpu().view(M, N) - want).abs()
+        tol = 1e-2 * want.abs() + 1e-4 * mag + (2.0 ** -8 * bias.float().abs()[None, :] if with_bias else 0)
         assert bool((err <= tol).all()), float((err - tol).max())
+        assert bool(torch.isfinite(out).all())
+
+
+def test_block_fp8_linear_ragged_k_falls_back(gpu, oracle):
+    """K not a multiple of 128 cannot be group-quantized; N ragged is fine."""
+    from sglang_amd.fp8_utils import w8a8_block_fp8_linear
+
+    x = make_activation(8, 512, seed=3)
+    w_q, w_s = make_fp8_weight(200, 512)
+    out = w8a8_block_fp8_linear(x.to(gpu), w_q.to(gpu), [128, 128], w_s.to(gpu))
+    xq, xs = oracle.group_quant(x, 128, mode="div")
+    ref, mag = oracle.fp8_blockwise_mm(xq, w_q, xs, w_s, torch.float32, want_abs=True)
+    assert bool(((out.float().cpu() - ref).abs() <= 1e-2 * ref.abs() + 1e-4 * mag).all())
+    with pytest.raises(NotImplementedError):
+        w8a8_block_fp8_linear(x.to(gpu), w_q.to(gpu), [64, 64], w_s.to(gpu))
 
 
 @pytest.mark.parametrize("shape,N,K", [((4, 3), 6144, 4096), ((1,), 4096, 14336), ((300,), 264, 512)])

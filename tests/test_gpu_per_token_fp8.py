@@ -1,0 +1,115 @@
+"""GPU parity of the per-token x per-channel FP8 linear: sgl_per_token_quant_fp8 (codes and scales bit-exact) and
+fp8_scaled_mm (floating point: |out - ref| <= 1e-2 * |ref| + 1e-4 * mag, mag = |sa * sb| * sum |a * b|, the slack the
+grouped additions of the fp8 MFMA need where large terms cancel, see tests/test_gpu_fp8_gemm.py; plus the reference's own
+criterion rtol 0.02 / atol 1 against its torch formula, sgl-kernel/tests/test_fp8_gemm.py:7-37)."""
+import pytest
+import torch
+
+from sglang_amd.workloads import make_activation
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K", [(1, 512), (7, 4096), (64, 7168), (33, 16384 + 512), (3, 8)])
+def test_per_token_quant_fp8_bits(gpu, oracle, dtype, M, K):
+    from sglang_amd.fp8_kernel import sglang_per_token_quant_fp8
+
+    if dtype == torch.float32 and K % 4:
+        pytest.skip("row must span a multiple of 16 bytes")
+    x = make_activation(M, K, seed=M * 7 + K, dtype=dtype)
+    if M > 2:
+        x[1] = 0  # a row of zeros: scale 0, codes 0, no NaN
+    q, s = sglang_per_token_quant_fp8(x.to(gpu))
+    q_o, s_o = oracle.per_token_quant_fp8(x)
+    assert q.dtype == FP8 and tuple(s.shape) == (M, 1)
+    assert torch.equal(s.cpu().view(torch.int32), s_o.view(torch.int32))
+    assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8))
+    if M > 2:
+        assert float(s[1]) == 0.0 and not bool(q[1].view(torch.uint8).any())
+
+
+def _rand_fp8(shape, g):
+    return ((torch.rand(*shape, generator=g) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
+
+
+# decode, mid-M (64- and 128-token tiles, split and whole), generic (ragged N), two-phase large-M
+SHAPES = [(1, 512, 1024), (16, 2048, 7168), (48, 16384, 2048), (130, 8192, 7168), (300, 1088, 512), (128, 16, 512),
+          (1024, 1024, 4096), (4096, 4352, 512), (4000, 576, 1024)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_fp8_scaled_mm(gpu, oracle, M, N, K, with_bias, out_dtype):
+    from sglang_amd import _lib
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
+
+    print(f"case M={M} N={N} K={K} bias={with_bias} {out_dtype} -> {_lib.gemm_plan('fp8', M, N, K)['kernel']}", flush=True)
+    g = torch.Generator().manual_seed(M + 3 * N + K)
+    a, w = _rand_fp8((M, K), g), _rand_fp8((N, K), g)
+    sa = torch.randn(M, generator=g) * 1e-3
+    sb = torch.randn(N, generator=g) * 1e-3
+    bias = torch.randn(N, generator=g).to(out_dtype) if with_bias else None
+    out = fp8_scaled_mm(a.to(gpu), w.to(gpu).t(), sa.to(gpu), sb.to(gpu), out_dtype, bias.to(gpu) if with_bias else None)
+    assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
+    rows = torch.arange(M) if M <= 512 else torch.cat([torch.tensor([0, 255, 256, M - 1]), torch.randperm(M, generator=g)[:44]])
+    ref, mag = oracle.fp8_scaled_mm(a[rows].contiguous(), w, sa[rows], sb, torch.float32, None, want_abs=True)
+    if with_bias:
+        ref = ref + bias.float()[None, :]
+    got = out[rows.to(gpu)].float().cpu()
+    assert bool(torch.isfinite(got).all())
+    err = (got - ref).abs()
+    tol = 1e-2 * ref.abs() + 1e-4 * mag + (2.0 ** -8 * bias.float().abs()[None, :] if with_bias else 0)
+    if out_dtype == torch.float16:
+        tol = tol + 2.0 ** -24  # one step of the fp16 subnormal grid: the products of two 1e-3 scales reach down there
+    assert bool((err <= tol).all()), float((err - tol).max())
+    # the reference's own test: torch formula, bias added after the cast
+    o = (a[rows].float() @ w.float().T) * sa[rows].view(-1, 1) * sb.view(1, -1)
+    o = o.to(out_dtype)
+    if with_bias:
+        o = o + bias.view(1, -1)
+    torch.testing.assert_close(out[rows.to(gpu)].cpu(), o, rtol=0.02, atol=1.0)
+
+
+def test_fp8_scaled_mm_exact_integers(gpu):
+    """Integer codes and power-of-two scales: every product, sum and scaling is exact, whatever the order."""
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
+
+    g = torch.Generator().manual_seed(6)
+    for M, N, K in [(9, 384, 640), (300, 256, 1152), (2048, 4096, 256)]:
+        ai = torch.randint(-8, 9, (M, K), generator=g)
+        wi = torch.randint(-8, 9, (N, K), generator=g)
+        sa = torch.exp2(torch.randint(-3, 4, (M,), generator=g).float())
+        sb = torch.exp2(torch.randint(-3, 4, (N,), generator=g).float())
+        bias = torch.randint(-16, 17, (N,), generator=g).float().to(torch.bfloat16)
+        out = fp8_scaled_mm(ai.float().to(FP8).to(gpu), wi.float().to(FP8).to(gpu).t(), sa.to(gpu), sb.to(gpu), torch.bfloat16,
+                            bias.to(gpu))
+        want = ((ai.double() @ wi.double().T) * sa.double()[:, None] * sb.double()[None, :] + bias.double()[None, :])
+        assert torch.equal(out.cpu().double(), want.to(torch.bfloat16).double()), (M, N, K)
+
+
+@pytest.mark.parametrize("shape,N,K", [((2, 5), 384, 512), ((1,), 6144, 4096), ((700,), 1024, 2048)])
+def test_apply_fp8_linear(gpu, oracle, shape, N, K):
+    """apply_fp8_linear: per-token quantization then fp8_scaled_mm, against the oracle's pipeline and the unquantized linear."""
+    from sglang_amd.fp8_utils import apply_fp8_linear
+
+    M = 1
+    for d in shape:
+        M *= d
+    x = make_activation(M, K, seed=5, outlier_frac=0.0).view(*shape, K)
+    g = torch.Generator().manual_seed(8)
+    w = torch.randn(N, K, generator=g) * 0.02
+    w_s = w.abs().amax(1) / 448.0
+    w_q = (w / w_s[:, None]).clamp(-448, 448).to(FP8)
+    bias = torch.randn(N, generator=g).to(torch.bfloat16)
+    out = apply_fp8_linear(x.to(gpu), w_q.to(gpu).t(), w_s.to(gpu), bias=bias.to(gpu))
+    assert tuple(out.shape) == (*shape, N) and out.dtype == torch.bfloat16
+    xq, xs = oracle.per_token_quant_fp8(x.view(M, K))
+    ref, mag = oracle.fp8_scaled_mm(xq, w_q, xs, w_s, torch.float32, None, want_abs=True)
+    ref = ref + bias.float()[None, :]
+    err = (out.float().cpu().view(M, N) - ref).abs()
+    assert bool((err <= 1e-2 * ref.abs() + 1e-4 * mag + 2.0 ** -8 * bias.float().abs()[None, :]).all())
+    full = x.view(M, K).float() @ w.T + bias.float()
+    assert float((out.float().cpu().view(M, N) - full).norm() / full.norm()) < 0.05

@@ -151,3 +151,34 @@ def test_int8_epilogue_orders(oracle, out_dtype, with_bias):
     for order in (oracle.EPI_ROW_COL_ACC, oracle.EPI_TORCH):
         assert int((outs[order].view(torch.int16).to(torch.int32) - base).abs().max()) <= 1
     assert torch.equal(oracle.int8_scaled_mm(a, w, sa, sb, out_dtype, bias), outs[oracle.EPI_COL_ROW])
+
+
+# ---------------------------------------------------------------- per-token x per-channel FP8 GEMM
+
+def test_fp8_scaled_mm_against_fp64_matmul(oracle):
+    """sgl-kernel/tests/test_fp8_gemm.py:7-15 in fp64: the oracle's exact sum, scaled as sa * (sb * acc) in fp32, may
+    differ from fp64 by fp32 rounding only."""
+    g = torch.Generator().manual_seed(11)
+    M, N, K = 13, 40, 1000
+    a = ((torch.rand(M, K, generator=g) - 0.5) * 896).to(torch.float8_e4m3fn)
+    w = ((torch.rand(N, K, generator=g) - 0.5) * 896).to(torch.float8_e4m3fn)
+    sa, sb = torch.randn(M, generator=g) * 1e-3, torch.randn(N, generator=g) * 1e-3
+    bias = torch.randn(N, generator=g)
+    out = oracle.fp8_scaled_mm(a, w, sa, sb, torch.float32, bias)
+    ref = (a.double() @ w.double().T) * sa.double()[:, None] * sb.double()[None, :] + bias.double()[None, :]
+    assert float(((out.double() - ref).abs() / (ref.abs() + 1e-30)).max()) < 1e-5
+    # and the magnitude matrix bounds the result
+    out2, mag = oracle.fp8_scaled_mm(a, w, sa, sb, torch.float32, None, want_abs=True)
+    assert bool((out2.abs() <= mag * (1 + 1e-5)).all())
+
+
+def test_fp8_scaled_mm_exact_integers_and_cast(oracle):
+    g = torch.Generator().manual_seed(12)
+    M, N, K = 9, 24, 384
+    ai, wi = torch.randint(-8, 9, (M, K), generator=g), torch.randint(-8, 9, (N, K), generator=g)
+    sa = torch.exp2(torch.randint(-3, 4, (M,), generator=g).float())
+    sb = torch.exp2(torch.randint(-3, 4, (N,), generator=g).float())
+    bias = torch.randint(-16, 17, (N,), generator=g).float().to(torch.bfloat16)
+    out = oracle.fp8_scaled_mm(ai.float().to(torch.float8_e4m3fn), wi.float().to(torch.float8_e4m3fn), sa, sb, torch.bfloat16, bias)
+    want = ((ai @ wi.T).double() * sa.double()[:, None] * sb.double()[None, :] + bias.double()[None, :]).to(torch.bfloat16)
+    assert torch.equal(out, want)

@@ -234,3 +234,40 @@ def test_per_token_quant_int8(oracle):
     want = (torch.sign(t) * torch.floor(t.abs() + 0.5)).to(torch.int8)  # round half away from zero
     assert torch.equal(q, want) and torch.equal(s, amax / 127.0)
     assert int(q.abs().max()) == 127
+
+
+# ---------------------------------------------------------------- per-token FP8 quantizer (one scale per row)
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_per_token_quant_fp8_against_torch_fp32(oracle, dtype):
+    """sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85 restated with torch CPU fp32 ops (IEEE `/` and `*`) and torch's
+    own e4m3fn cast: scale = amax / 448, q = clamp(x * (1 / scale)), zero rows -> scale 0, codes 0."""
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(37, 1024, generator=g) * torch.rand(37, 1, generator=g) * 20).to(dtype)
+    x[5] = 0
+    x[6, 17] = 3.0e4 if dtype != torch.float16 else 6.0e4  # an outlier that sets the row's scale
+    q, s = oracle.per_token_quant_fp8(x)
+    xf = x.float()
+    s_ref = xf.abs().amax(dim=1, keepdim=True) / 448.0
+    inv = torch.where(s_ref == 0, torch.zeros(()), 1.0 / s_ref)
+    q_ref = (xf * inv).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    assert torch.equal(s.view(torch.int32), s_ref.view(torch.int32))
+    assert torch.equal(q.view(torch.uint8), q_ref.view(torch.uint8))
+    assert float(s[5]) == 0.0 and not bool(q[5].view(torch.uint8).any())
+    # the element that attains the row maximum encodes to +-448 (0x7e / 0xfe)
+    assert int(q[6, 17].view(torch.uint8)) == 0x7E
+
+
+def test_per_token_quant_fp8_known_answer(oracle):
+    """Codes that are exactly representable times a power-of-two scale must come back unchanged, with that scale."""
+    g = torch.Generator().manual_seed(4)
+    codes = torch.randint(0, 256, (16, 256), generator=g, dtype=torch.uint8)
+    codes = torch.where((codes & 0x7F) == 0x7F, codes & 0xF7, codes)
+    codes[:, 0] = 0x7E  # every row attains 448
+    scale = torch.exp2(torch.randint(-6, 7, (16, 1), generator=g).float())
+    x = codes.view(torch.float8_e4m3fn).float() * scale
+    q, s = oracle.per_token_quant_fp8(x)
+    assert torch.equal(s, scale)
+    back = q.view(torch.uint8)
+    want = torch.where(codes == 0x80, torch.zeros((), dtype=torch.uint8), codes)  # -0 * scale = -0 -> encodes as 0x80 again
+    assert torch.equal(back, codes) or torch.equal(back, want)
