@@ -112,20 +112,28 @@ __device__ __forceinline__ float div_shared(float x, float s, float r) {
 }
 
 // T: element tag; LPG lanes per group; ITERS 16-byte vectors per lane and group.
-template <typename T, int LPG, int ITERS, int MODE, bool UE8M0, bool FP8_OUT, int UNROLL>
+// QUAD (UNROLL == 4 only): the four groups of a thread are four CONSECUTIVE groups of one row, so their scales leave as
+// one 16-byte store (fp32, row-major) or one 32-bit word (packed UE8M0) instead of four 4-byte or 1-byte stores; the host
+// selects it when groups per row and the group count are multiples of four and the scale layout is one of those two.
+template <typename T, int LPG, int ITERS, int MODE, bool UE8M0, bool FP8_OUT, int UNROLL, bool QUAD>
 __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
+  static_assert(!QUAD || UNROLL == 4, "a quad is four groups");
   constexpr int VEC = Elem<T>::VEC;
   constexpr int GROUP = LPG * ITERS * VEC;
   constexpr int GROUPS_PER_PASS = 256 / LPG;
+  constexpr int G_STEP = QUAD ? 1 : GROUPS_PER_PASS;  // distance between a thread's consecutive groups
   const uint32_t lane = threadIdx.x % LPG;
-  const uint32_t g_first = blockIdx.x * (GROUPS_PER_PASS * UNROLL) + threadIdx.x / LPG;
+  // QUAD: quads past the end redo the last quad (same values to the same addresses), like single groups do below
+  const uint32_t g_first = QUAD ? min(blockIdx.x * GROUPS_PER_PASS + threadIdx.x / LPG, p.num_groups / 4 - 1) * 4
+                                : blockIdx.x * (GROUPS_PER_PASS * UNROLL) + threadIdx.x / LPG;
+  float quad_scale[QUAD ? 4 : 1];
 
   u32x4 raw[UNROLL][ITERS];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     // Past the last group the lanes redo the last group (same values to the same addresses): the body stays free of
     // branches, which keeps the stores nontemporal and the loop fully unrolled.
-    const uint32_t g = min(g_first + u * GROUPS_PER_PASS, p.num_groups - 1);
+    const uint32_t g = min(g_first + u * G_STEP, p.num_groups - 1);
     const u32x4* src = reinterpret_cast<const u32x4*>(p.x) + (size_t)g * (LPG * ITERS) + lane;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
@@ -135,7 +143,7 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
 
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
-    const uint32_t g = min(g_first + u * GROUPS_PER_PASS, p.num_groups - 1);
+    const uint32_t g = min(g_first + u * G_STEP, p.num_groups - 1);
     float v[ITERS][VEC];
     float amax = p.eps;
 #pragma unroll
@@ -198,7 +206,9 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
         else
           store_nt(d, w[0]);
       }
-      if (lane == 0) {
+      if constexpr (QUAD) {
+        quad_scale[u] = s_val;
+      } else if (lane == 0) {
         const uint32_t row = fastdiv(g, p.groups_per_row);
         const uint32_t kg = g - row * p.groups_per_row.div;
         if constexpr (UE8M0) {
@@ -213,6 +223,23 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const QuantParams p) {
       }
     }
   }
+  if constexpr (QUAD) {
+    if (lane == 0) {
+      if constexpr (UE8M0) {
+        const uint32_t row = fastdiv(g_first, p.groups_per_row);
+        const uint32_t kg = g_first - row * p.groups_per_row.div;  // a multiple of four
+        uint32_t word = 0;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) word |= (__float_as_uint(quad_scale[u]) >> 23) << (8 * u);
+        *reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(p.s) + (size_t)(kg >> 2) * (size_t)p.s_stride_col * 4u +
+                                     (size_t)row * 4u) = word;
+      } else {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.s) + g_first) =
+            f32x4{quad_scale[0], quad_scale[1], quad_scale[2], quad_scale[3]};
+      }
+    }
+  }
 }
 
 template <typename T, int LPG, int ITERS, int MODE, bool UE8M0, bool FP8_OUT>
@@ -221,7 +248,20 @@ int launch(const QuantParams& p, hipStream_t stream) {
   constexpr int UNROLL = (ITERS >= 4) ? 1 : (ITERS == 2 ? 2 : 4);
   constexpr int GROUPS_PER_BLOCK = (256 / LPG) * UNROLL;
   const uint32_t blocks = (p.num_groups + GROUPS_PER_BLOCK - 1) / GROUPS_PER_BLOCK;
-  hipLaunchKernelGGL((group_quant_kernel<T, LPG, ITERS, MODE, UE8M0, FP8_OUT, UNROLL>), dim3(blocks), dim3(256), 0,
+  if constexpr (UNROLL == 4) {
+    // four consecutive groups of a row per thread when their scales are adjacent in memory: fp32 scales indexed by the
+    // flat group number, or packed exponents (four k-groups per word)
+    const uint32_t gpr = p.groups_per_row.div;
+    const bool flat_f32 = !UE8M0 && p.s_stride_col == 1 && p.s_stride_row == (int64_t)gpr &&
+                          (reinterpret_cast<uintptr_t>(p.s) & 15) == 0;
+    const bool packed = UE8M0 && (reinterpret_cast<uintptr_t>(p.s) & 3) == 0;
+    if (gpr % 4 == 0 && p.num_groups % 4 == 0 && (flat_f32 || packed)) {
+      hipLaunchKernelGGL((group_quant_kernel<T, LPG, ITERS, MODE, UE8M0, FP8_OUT, UNROLL, true>), dim3(blocks), dim3(256), 0,
+                         stream, p);
+      return check_launch("mi355_group_quant_8bit");
+    }
+  }
+  hipLaunchKernelGGL((group_quant_kernel<T, LPG, ITERS, MODE, UE8M0, FP8_OUT, UNROLL, false>), dim3(blocks), dim3(256), 0,
                      stream, p);
   return check_launch("mi355_group_quant_8bit");
 }
