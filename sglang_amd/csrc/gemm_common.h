@@ -167,12 +167,8 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K);
 int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);   // bm: 64 or 128, from dma3_plan()
 int launch_int8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
 
-// Large-M INT8 GEMM (256 x 256 tile, 8 waves, direct-to-LDS loads, 32x32x32 MFMA); gemm_int8_dma.hip.
-// Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
-int launch_int8_dma(GemmParams& p, hipStream_t stream, const char* what);
-
-// Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases); gemm_int8_pp.hip.
-// Same requirements.
+// Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases, direct-to-LDS loads,
+// 32x32x32 MFMA); gemm_int8_pp.hip.  Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
 int launch_int8_pp(GemmParams& p, hipStream_t stream, const char* what);
 
 // Small-M blockwise FP8 GEMM streaming the weight through wave-private LDS, no barriers; gemm_fp8_decode.hip.

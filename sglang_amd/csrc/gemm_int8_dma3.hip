@@ -3,7 +3,7 @@
 // The loop structure is the one of gemm_fp8_dma3.hip: the direct-to-LDS loads of K step k+2 are issued while step k is
 // multiplied, the wait before the bare s_barrier that ends iteration k covers step k+1 only (s_waitcnt vmcnt(LOADS), the
 // loads per wave and iteration being a constant), loads, wait and barrier are written as instructions.  The arithmetic
-// is the one of gemm_int8_dma.hip: v_mfma_i32_32x32x32_i8, four per 32 x 32 tile and 128-byte K step, exact int32
+// is the one of gemm_int8_pp.hip: v_mfma_i32_32x32x32_i8, four per 32 x 32 tile and 128-byte K step, exact int32
 // accumulation, fragments of 32 rows x 2 K halves read with the (row >> 1) & 7 swizzle.  A wave owns (BM / 2) x 64 outputs.
 // Optional split along K: int32 partials to the workspace, the ordered reduce applies the epilogue.
 // Requires K % 128 == 0, 16-byte aligned rows, row offsets below 4 GiB.

@@ -395,8 +395,8 @@ int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* wha
 
 // Which kernel serves a problem, with which tiling.  One function decides for the launcher and for the plan query, so
 // what the query reports is what runs.
-enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_PINGPONG, RK_PIPELINED, RK_INT8_DMA256, RK_GENERIC };
-const char* const ROUTE_NAMES[] = {"decode", "dma3", "pingpong", "pipelined", "int8_dma256", "generic"};
+enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_PINGPONG, RK_PIPELINED, RK_GENERIC };
+const char* const ROUTE_NAMES[] = {"decode", "dma3", "pingpong", "pipelined", "generic"};
 
 struct Route {
   int kernel;
@@ -444,7 +444,7 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
         return r;
       }
     } else if (K % KSTEP == 0 && tiles_256 >= NUM_CUS / 2) {
-      r.kernel = RK_INT8_DMA256, r.bn = 256;
+      r.kernel = RK_PINGPONG, r.bn = 256;
       return r;
     }
   }
@@ -535,9 +535,8 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
     case RK_DMA3:
       rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, stream, what) : launch_int8_dma3(p, r.bm, stream, what);
       break;
-    case RK_PINGPONG: return launch_fp8_pp(p, stream, what);
+    case RK_PINGPONG: return IS_FP8 ? launch_fp8_pp(p, stream, what) : launch_int8_pp(p, stream, what);
     case RK_PIPELINED: return launch_fp8_pipelined(p, stream, what);
-    case RK_INT8_DMA256: return launch_int8_pp(p, stream, what);
     default:
       // the generic kernel runs its own ordered reduce
       switch (r.bm) {

@@ -85,17 +85,6 @@ def make_fp8_weight(N: int, K: int, seed: int | None = None, std: float = 0.02):
     return block_cast_to_fp8(w)
 
 
-def make_fp8_weight_fast(N: int, K: int, seed: int | None = None):
-    """Benchmark-only weight of the same format: uniformly random finite e4m3fn codes and
-    block scales near 2e-4, without drawing N*K Gaussians on the host (which takes minutes
-    at N*K = 2.6e8).  Timing does not depend on the values."""
-    g = _gen(N * 10007 + K if seed is None else seed)
-    codes = torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8)
-    codes = torch.where((codes & 0x7F) == 0x7F, codes & 0xF7, codes)  # no NaN codes
-    s = (torch.rand(cdiv(N, 128), cdiv(K, 128), generator=g) + 0.5) * 2e-4
-    return codes.view(FP8), s.contiguous()
-
-
 def make_int8_activation(M: int, K: int, seed: int | None = None):
     """bf16 N(0,1) activations quantized per token: (int8 [M,K], fp32 scales [M,1])."""
     g = _gen(M * 10000 + K + 1 if seed is None else seed)

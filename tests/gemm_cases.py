@@ -47,7 +47,7 @@ INT8_REQUIRED_VARIANTS = {
     ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
     ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
-    ("int8_dma256",),
+    ("pingpong", "kfull"),
     ("generic", 16, "aligned", "whole"), ("generic", 32, "aligned", "split"), ("generic", 64, "aligned", "whole"),
     ("generic", 128, "aligned", "whole"), ("generic", 128, "aligned", "split"), ("generic", 256, "aligned", "whole"),
 }
@@ -72,8 +72,6 @@ def variant_of(plan: dict, K: int):
         return (k, plan["bm"], sp)
     if k in ("pingpong", "pipelined"):
         return (k, "kfull" if K % 128 == 0 else "ktail")
-    if k == "int8_dma256":
-        return (k,)
     return (k, plan["bm"], "aligned" if plan["aligned"] else "bytes", sp)
 
 
