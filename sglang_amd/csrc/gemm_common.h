@@ -48,13 +48,14 @@ __device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off
     }
     return;
   }
-  uint32_t h[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) h[i] = (out_dtype == MI355_BF16) ? f32_to_bf16_bits(r[i]) : f32_to_f16_bits(r[i]);
+  const bool bf = out_dtype == MI355_BF16;
+  const uint32_t w0 = bf ? pack_bf16x2(r[0], r[1]) : pack_f16x2(r[0], r[1]);
+  const uint32_t w1 = bf ? pack_bf16x2(r[2], r[3]) : pack_f16x2(r[2], r[3]);
   uint16_t* o = reinterpret_cast<uint16_t*>(out) + off;
   if (nvalid == 4 && vec_ok) {
-    *reinterpret_cast<u32x2*>(o) = u32x2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+    *reinterpret_cast<u32x2*>(o) = u32x2{w0, w1};
   } else {
+    const uint32_t h[4] = {w0 & 0xffffu, w0 >> 16, w1 & 0xffffu, w1 >> 16};
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       if (i < nvalid) o[i] = (uint16_t)h[i];
@@ -70,8 +71,7 @@ __device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off
 constexpr int OUT_TILE_BYTES = 256 * 512;
 
 __device__ __forceinline__ uint32_t pack2_16(int out_dtype, float lo, float hi) {
-  return out_dtype == MI355_BF16 ? (f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16))
-                                 : (f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16));
+  return out_dtype == MI355_BF16 ? pack_bf16x2(lo, hi) : pack_f16x2(lo, hi);
 }
 // four consecutive channels starting at tile column `col` (a multiple of 4) of tile row `row`
 __device__ __forceinline__ void out_tile_put4(uint8_t* tile, int row, int col, int out_dtype, const float* r) {
