@@ -423,8 +423,10 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   if (M > 16 && (M <= 1024 || tiles_256 < NUM_CUS) && K % KSTEP == 0 && aligned && small_offsets) {
     // mid-M, or many tokens but too few channels for 256 x 256 tiles: three-stage direct-to-LDS kernel with 64- or 128-token
     // tiles, when its tiling fills the chip well enough
+    // Between 256 and 1024 tokens it beats the generic kernel even where its tiling fills the chip badly (measured on K=4096..7168 ->
+    // N=1536..6144: 25 us against 35..63 us); below that the generic kernel's small tiles win for few channels.
     const Dma3Plan dp = dma3_plan(M, N, K);
-    if (dp.efficiency >= DMA3_MIN_EFFICIENCY) {
+    if ((M >= 256 && M <= 1024) || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
       r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = 256, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
       return r;
     }
