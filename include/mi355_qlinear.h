@@ -143,16 +143,6 @@ int mi355_int8_scaled_mm(const void* a, const void* b, const float* sa, const fl
                          void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Split K in one launch.  The small-M kernels split K over several workgroups; by default the workgroup that finishes
- * last adds the partial sums (same fixed order as the separate reduce kernel, so results are bit-identical), using
- * arrival counters in device memory that the library owns, one block of counters per (device, stream, graph-capture
- * sequence): launches that can run concurrently never share one.  mi355_set_single_launch_split_k(0) switches back to a
- * second (reduce) launch for every later call of this process; returns the previous setting.  The reference has no
- * counterpart: its split-K lives inside CUTLASS/Triton.  Not a compute call.
- */
-int mi355_set_single_launch_split_k(int enabled);
-
-/*
  * Host-only query: which kernel and tiling mi355_fp8_blockwise_mm / mi355_int8_scaled_mm would run for a shape.
  * Stands in for the reference's shape dispatchers, which are compile-time ladders nobody can ask
  * (sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:181-195, sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:603-661);

@@ -36,7 +36,6 @@ EXPORTS = (
     "mi355_fp8_scaled_mm",
     "mi355_fp8_block_linear_workspace_bytes",
     "mi355_fp8_block_linear",
-    "mi355_set_single_launch_split_k",
 )
 
 _lib = None
@@ -63,11 +62,14 @@ def lib() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build it with `make -C {_CSRC}` (or __graft_entry__.build()). "
             "The quantized-linear operators have no other implementation."
         )
+    # The library links against libamdhip64; a process that also runs PyTorch must end up with ONE HIP runtime, the one
+    # torch ships, so torch is loaded first (a library loaded before it would pull in the system copy as a second
+    # runtime, which then sees no device).
+    import torch  # noqa: F401
+
     L = ctypes.CDLL(LIB_PATH)
     i64, i32, f32, vp, sz = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
     L.mi355_qlinear_abi_version.restype = i32
-    L.mi355_set_single_launch_split_k.argtypes = [i32]
-    L.mi355_set_single_launch_split_k.restype = i32
     L.mi355_last_error.restype = ctypes.c_char_p
     L.mi355_group_quant_8bit.argtypes = [vp, i32, vp, i32, vp, i64, i64, i32, f32, f32, f32, i32, i32, f32, i64, i64, vp]
     L.mi355_group_quant_8bit.restype = i32

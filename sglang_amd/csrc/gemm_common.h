@@ -26,7 +26,6 @@ struct GemmParams {
   const float* col_scale;  // FP8 only, optional [N]: per-channel scale applied in the epilogue (fp8_scaled_mm)
   void* out;
   void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
-  uint32_t* arrive;  // split K in one launch: zeroed arrival counters, one per workgroup column (else nullptr: separate reduce)
   int M, N, K;
   int64_t lda, ldb, ldo;
   int64_t sa_sm, sa_sk, sb_sn, sb_sk;
@@ -120,50 +119,6 @@ __device__ __forceinline__ void fp8_channel_epilogue(const GemmParams& p, int n,
       const uint32_t h = b[min(n + v, p.N - 1)];
       r[v] += (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
     }
-  }
-}
-
-// Output elements (m, n .. n + 3) from the split-K partial tiles: sum in ascending split order, epilogue, store.
-// n % 4 == 0 and N % 4 == 0 (the split path requires it), so the four elements share a row.
-template <bool IS_FP8>
-__device__ __forceinline__ void splitk_reduce_quad(const GemmParams& p, int m, int n) {
-  const int64_t total = (int64_t)p.M * p.N;
-  const int64_t idx = (int64_t)m * p.N + n;
-  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-  if constexpr (IS_FP8) {
-    const float* w = reinterpret_cast<const float*>(p.ws) + idx;
-    v4f s = *reinterpret_cast<const v4f*>(w);
-    for (int k = 1; k < p.splits; ++k) {
-      const v4f t = *reinterpret_cast<const v4f*>(w + (int64_t)k * total);
-      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
-    }
-    float r[4] = {s[0], s[1], s[2], s[3]};
-    fp8_channel_epilogue(p, n, r);
-    store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
-  } else {
-    const int* w = reinterpret_cast<const int*>(p.ws) + idx;
-    v4i s = *reinterpret_cast<const v4i*>(w);
-    for (int k = 1; k < p.splits; ++k) {
-      const v4i t = *reinterpret_cast<const v4i*>(w + (int64_t)k * total);
-      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
-    }
-    if (p.out_dtype == MI355_I32) {
-      int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
-      for (int v = 0; v < 4; ++v) o[v] = s[v];
-      return;
-    }
-    const float sa_m = p.sa[m];
-    float r[4];
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      float t = mul_rn((float)s[v], mul_rn(p.sb[n + v], sa_m));
-      if (p.bias) {
-        const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
-        t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
-      }
-      r[v] = t;
-    }
-    store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
   }
 }
 

@@ -19,9 +19,8 @@
 // one stage from reads of another and places exact vmcnt waits.  XOR swizzle and chunk mapping are those of the other
 // kernels (chunks q and q + 4 per lane quarter: full-rate LDS reads).
 //
-// Split along K: every K range writes a partial tile to the caller's workspace; they are added in a fixed order (for INT8
-// the partials are int32 and the epilogue follows the sum) either by the workgroup that finishes last (arrival counters, one
-// launch) or, when the caller has no counters to give, by splitk_reduce_kernel.  INT8 uses two
+// Split along K: every K range writes a partial tile to the caller's workspace and splitk_reduce_kernel adds them in a
+// fixed order (for INT8 the partials are int32 and the reduce kernel applies the epilogue).  INT8 uses two
 // v_mfma_i32_16x16x64_i8 per K block (chunk q of both operands, then chunk q + 4) and has no scales in the loop.
 // Requires K % 128 == 0, N % 128 == 0 and 16-byte aligned rows; other shapes take the generic kernel.
 #include "gemm_common.h"
@@ -280,32 +279,6 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
           }
           store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r, 4, vec_ok);
         }
-      }
-    }
-  }
-
-  if constexpr (SPLIT) {
-    if (p.arrive != nullptr) {
-      // One launch instead of two: the workgroups of all K ranges that share these channel groups count themselves at one
-      // counter; the one that arrives last finds every partial tile written and adds them up - in ascending range order, like
-      // the separate reduce kernel, so the result does not depend on who is last.  It leaves the counter at zero for the next
-      // launch.  Nobody waits for anybody.
-      __shared__ int r_last;
-      const int column = blockIdx.x - split * wg_per_split;
-      __syncthreads();  // the partial sums of all four waves are written
-      if (threadIdx.x == 0) {
-        __threadfence();  // ... and visible to the whole device before this workgroup is counted
-        const bool last = atomicAdd(p.arrive + column, 1u) == (uint32_t)p.splits - 1u;
-        if (last) p.arrive[column] = 0;
-        r_last = last;
-      }
-      __syncthreads();
-      if (!r_last) return;
-      __threadfence();  // what the other ranges wrote is read from memory, not from a stale cache line
-      const int quads = groups * (GROUP_N / 4);
-      for (int e = threadIdx.x; e < p.M * quads; e += 64 * WAVES) {
-        const int m = e / quads;
-        splitk_reduce_quad<IS_FP8>(p, m, g_first * GROUP_N + 4 * (e - m * quads));
       }
     }
   }

@@ -20,9 +20,7 @@
 //     workspace and a second kernel adds them in a fixed order (deterministic, no atomics);
 //   * workgroups are renumbered so that each of the 8 XCDs (own L2) works on a contiguous, M-grouped
 //     patch of output tiles.
-#include <atomic>
 #include <mutex>
-#include <vector>
 
 #include "gemm_common.h"
 
@@ -260,8 +258,46 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
   const int64_t total = (int64_t)p.M * p.N;
   const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (idx >= total) return;
+  // N % 4 == 0 is required for the split path, so the four elements share a row
   const int m = (int)(idx / p.N);
-  splitk_reduce_quad<IS_FP8>(p, m, (int)(idx - (int64_t)m * p.N));
+  const int n = (int)(idx - (int64_t)m * p.N);
+  if constexpr (IS_FP8) {
+    const float* w = reinterpret_cast<const float*>(p.ws) + idx;
+    v4f s = *reinterpret_cast<const v4f*>(w);
+    for (int k = 1; k < p.splits; ++k) {
+      const v4f t = *reinterpret_cast<const v4f*>(w + (int64_t)k * total);
+      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
+    }
+    float r[4] = {s[0], s[1], s[2], s[3]};
+    fp8_channel_epilogue(p, n, r);
+    const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+    store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
+  } else {
+    const int* w = reinterpret_cast<const int*>(p.ws) + idx;
+    v4i s = *reinterpret_cast<const v4i*>(w);
+    for (int k = 1; k < p.splits; ++k) {
+      const v4i t = *reinterpret_cast<const v4i*>(w + (int64_t)k * total);
+      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
+    }
+    if (p.out_dtype == MI355_I32) {
+      int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
+      for (int v = 0; v < 4; ++v) o[v] = s[v];
+      return;
+    }
+    const float sa_m = p.sa[m];
+    float r[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float t = mul_rn((float)s[v], mul_rn(p.sb[n + v], sa_m));
+      if (p.bias) {
+        const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
+        t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+      }
+      r[v] = t;
+    }
+    const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+    store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -468,64 +504,6 @@ bool operands_aligned(const GemmParams& p) {
          ((reinterpret_cast<uintptr_t>(p.b) & 15) == 0);
 }
 
-// ---- arrival counters for split K in one launch.
-// A kernel whose workgroups count themselves at a counter and let the last arriver do the reduction needs counters that are
-// zero when it starts; the last arriver puts them back to zero.  They live in device memory owned by this library (zero
-// when the code object is loaded, one copy per GPU), in blocks of ARRIVE_PER_BLOCK.  Two launches that may run at the same
-// time must not share a block.  Launches into one stream run one after the other, and so do the nodes one stream
-// contributes to a captured graph, so a block belongs to a (device, stream, capture sequence) triple; the table only
-// grows.  When it is full, when a launch needs more counters than a block holds, or when the capture state cannot be
-// read, the caller falls back to the separate reduce kernel.
-constexpr int MAX_DEVICES = 64;
-constexpr int ARRIVE_BLOCKS = 256, ARRIVE_PER_BLOCK = 1024;
-static __device__ __align__(256) uint32_t arrive_counters[ARRIVE_BLOCKS * ARRIVE_PER_BLOCK];
-
-struct ArriveOwner {
-  int dev;
-  hipStream_t stream;
-  unsigned long long capture;  // 0: not capturing
-};
-std::mutex arrive_mutex;
-std::vector<ArriveOwner> arrive_owners;   // index = block; guarded by arrive_mutex
-uint32_t* arrive_base[MAX_DEVICES];       // guarded by arrive_mutex
-std::atomic<bool> single_launch_split_k{true};
-
-uint32_t* arrive_block_for(hipStream_t stream, int64_t counters) {
-  if (!single_launch_split_k.load(std::memory_order_relaxed) || counters > ARRIVE_PER_BLOCK) return nullptr;
-  int dev = -1;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
-  unsigned long long capture = 0;
-  if (stream != nullptr) {  // the legacy default stream cannot be captured
-    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    unsigned long long id = 0;
-    if (hipStreamGetCaptureInfo(stream, &status, &id) != hipSuccess) {
-      (void)hipGetLastError();
-      return nullptr;
-    }
-    if (status == hipStreamCaptureStatusInvalidated) return nullptr;
-    if (status == hipStreamCaptureStatusActive) capture = id + 1;  // distinct from "not capturing" whatever ids the runtime uses
-  }
-  std::lock_guard<std::mutex> lock(arrive_mutex);
-  if (arrive_base[dev] == nullptr) {
-    void* q = nullptr;
-    if (hipGetSymbolAddress(&q, HIP_SYMBOL(arrive_counters)) != hipSuccess || q == nullptr) {
-      (void)hipGetLastError();
-      return nullptr;
-    }
-    arrive_base[dev] = static_cast<uint32_t*>(q);
-  }
-  size_t block = 0;
-  for (; block < arrive_owners.size(); ++block) {
-    const ArriveOwner& o = arrive_owners[block];
-    if (o.dev == dev && o.stream == stream && o.capture == capture) break;
-  }
-  if (block == arrive_owners.size()) {
-    if (block >= (size_t)ARRIVE_BLOCKS) return nullptr;
-    arrive_owners.push_back(ArriveOwner{dev, stream, capture});
-  }
-  return arrive_base[dev] + block * ARRIVE_PER_BLOCK;
-}
-
 template <bool IS_FP8>
 int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipStream_t stream, const char* what) {
   p.kb_total = (p.K + KSTEP - 1) / KSTEP;
@@ -554,10 +532,6 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
   int rc;
   switch (r.kernel) {
     case RK_DECODE:
-      if (p.splits > 1) {  // one counter per workgroup column
-        const int64_t groups_n = p.N / 128;
-        p.arrive = arrive_block_for(stream, (groups_n + r.groups_per_wg - 1) / r.groups_per_wg);
-      }
       rc = IS_FP8 ? launch_fp8_decode(p, r.groups_per_wg, stream, what) : launch_int8_decode(p, r.groups_per_wg, stream, what);
       break;
     case RK_DMA3:
@@ -575,7 +549,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
         default: rc = launch_tile<IS_FP8, 256, 128, 2, 2>(p, aligned, stream, what); break;
       }
   }
-  if (rc != MI355_OK || p.splits == 1 || p.arrive != nullptr) return rc;
+  if (rc != MI355_OK || p.splits == 1) return rc;
   const int64_t quads = ((int64_t)p.M * p.N + 3) / 4;
   hipLaunchKernelGGL(splitk_reduce_kernel<IS_FP8>, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
   return check_launch(what);
@@ -598,10 +572,6 @@ int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, ch
 }  // namespace mi355
 
 using namespace mi355;
-
-extern "C" int mi355_set_single_launch_split_k(int enabled) {
-  return single_launch_split_k.exchange(enabled != 0) ? 1 : 0;
-}
 
 extern "C" size_t mi355_fp8_blockwise_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return workspace_bytes(M, N, K, true);
@@ -646,6 +616,7 @@ int fp8_mm_params(const char* what, const void* a, const void* b, const float* s
 constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)MI355_NOALLOC_SCRATCH_BYTES;
 static __device__ __align__(256) uint8_t scratch[NOALLOC_SCRATCH_BYTES];
 
+constexpr int MAX_DEVICES = 64;
 std::mutex scratch_mutex;
 void* scratch_ptr[MAX_DEVICES];  // guarded by scratch_mutex
 
