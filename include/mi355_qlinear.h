@@ -173,6 +173,20 @@ int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, in
 int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
 
 /*
+ * Per-tensor FP8 activation quantization: ONE fp32 scale for the whole tensor, q = e4m3fn(clamp(x * (1 / scale))).
+ *   is_static == 0: scale = max |x| / 448 is computed first.  *scale must hold 0.0f on entry (block maxima are merged into
+ *                   it with an atomic max; the reference's wrapper passes torch.zeros(1) the same way).
+ *   is_static != 0: *scale is given.  scale_rows, if not NULL, receives `rows` copies of it (the per-token shape that
+ *                   fp8_scaled_mm wants for a per-tensor scale).
+ * Replaces sgl_per_tensor_quant_fp8 (sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:102-130, kernels :10-100) and the
+ * Triton static_quant_fp8 (python/sglang/srt/layers/quantization/fp8_kernel.py:593-665), whose arithmetic is the same.
+ * A tensor of zeros quantized dynamically gets scale 0 and, like in the reference, codes of +448 (0 * inf = NaN meets
+ * fmin/fmax).  x: numel contiguous F32/F16/BF16 elements, 16-byte aligned; q: numel e4m3fn bytes, 8-byte aligned.
+ */
+int mi355_per_tensor_quant_fp8(const void* x, int x_dtype, void* q, float* scale, int64_t numel, int is_static,
+                               float* scale_rows, int64_t rows, void* stream);
+
+/*
  * Per-token x per-channel FP8 GEMM:  out[m,n] = cast( sa[m] * sb[n] * sum_k a[m,k] * b[n,k] + f32(bias[n]) ), fp32 accumulate.
  * Replaces fp8_scaled_mm (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532, epilogue :529-547; caller apply_fp8_linear,
  *          python/sglang/srt/layers/quantization/fp8_utils.py:565-853).

@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_per_token_quant_int8.restype = i32
         L.oracle_per_token_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64]
         L.oracle_per_token_quant_fp8.restype = i32
+        L.oracle_per_tensor_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i32]
+        L.oracle_per_tensor_quant_fp8.restype = i32
         L.oracle_fp8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32, vp] + [i64] * 6
         L.oracle_fp8_scaled_mm.restype = i32
         L.oracle_fp8_blockwise_mm.argtypes = [vp, vp, vp, vp, vp, i32, vp] + [i64] * 10
@@ -180,6 +182,16 @@ def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     q = torch.zeros(M, K, dtype=torch.uint8)
     s = torch.zeros(M, 1, dtype=torch.float32)
     rc = lib().oracle_per_token_quant_fp8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), M, K)
+    assert rc == 0
+    return q.view(torch.float8_e4m3fn), s
+
+
+def per_tensor_quant_fp8(x: torch.Tensor, scale: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x (any shape) -> (e4m3fn like x, fp32 scale [1]); scale = max|x| / 448 unless given (static)."""
+    x = _cpu(x).contiguous()
+    q = torch.zeros(x.shape, dtype=torch.uint8)
+    s = torch.zeros(1, dtype=torch.float32) if scale is None else _cpu(scale).reshape(1).to(torch.float32).clone()
+    rc = lib().oracle_per_tensor_quant_fp8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), x.numel(), int(scale is not None))
     assert rc == 0
     return q.view(torch.float8_e4m3fn), s
 

@@ -24,6 +24,8 @@
  *                             sgl-kernel/tests/test_int8_gemm.py:11-17 (torch order)
  *   oracle_per_token_quant_int8  python/sglang/srt/layers/quantization/int8_kernel.py:28-52
  *   oracle_per_token_quant_fp8   sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85
+ *   oracle_per_tensor_quant_fp8  sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:10-100,
+ *                                python/sglang/srt/layers/quantization/fp8_kernel.py:593-632 (static_quant_fp8)
  *   oracle_fp8_scaled_mm         sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:529-547, :1450-1532
  *
  * Parity status: every function here is pinned by tests/test_oracle_*.py against
@@ -295,6 +297,27 @@ int oracle_per_token_quant_fp8(const void* x, int x_dtype, uint8_t* q, float* s,
       t = fmaxf(fminf(t, 448.0f), -448.0f);
       q[(size_t)row * K + j] = oracle_e4m3fn_encode(t);
     }
+  }
+  return 0;
+}
+
+/* x (n elements) -> q e4m3fn, one scale for the tensor.  Dynamic (is_static == 0): *scale = max|x| / 448 (the reference
+ * merges per-block quotients with an atomic max into a zeroed word: the same value, division by 448 being monotonic);
+ * then in both modes q = RNE(fmax(fmin(x * (1 / *scale), 448), -448))  (sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:10-100;
+ * python/sglang/srt/layers/quantization/fp8_kernel.py:593-632 has the same arithmetic for a given scale).  fmin/fmax return
+ * the other operand for a NaN, so a zero tensor quantized dynamically (0 * inf) comes out as +448, as in the reference. */
+int oracle_per_tensor_quant_fp8(const void* x, int x_dtype, uint8_t* q, float* scale, int64_t n, int is_static) {
+  if (!is_static) {
+    float amax = 0.f;
+    for (int64_t i = 0; i < n; ++i) amax = fmaxf(amax, fabsf(load_as_f32(x, x_dtype, (size_t)i)));
+    *scale = amax / 448.0f;
+  }
+  const float inv = 1.0f / *scale;
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float t = load_as_f32(x, x_dtype, (size_t)i) * inv;
+    t = fmaxf(fminf(t, 448.0f), -448.0f);
+    q[i] = oracle_e4m3fn_encode(t);
   }
   return 0;
 }

@@ -190,6 +190,52 @@ def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
     return x_q, x_s
 
 
+def static_quant_fp8(x: torch.Tensor, x_s: torch.Tensor, repeat_scale: bool = False):
+    """fp8_kernel.py:635-665: quantize with a given per-tensor scale; with ``repeat_scale`` the returned scale is a
+    ``[M, 1]`` tensor holding it once per row (the shape fp8_scaled_mm takes)."""
+    assert x.is_contiguous(), "`x` is not contiguous"
+    assert x_s.numel() == 1, "only supports per-tensor scale"
+    x_q = torch.empty_like(x, device=x.device, dtype=fp8_dtype)
+    scale = x_s.reshape(1).to(torch.float32)
+    if repeat_scale:
+        M = x.numel() // x.shape[-1]
+        x_s_repeat = torch.empty((M, 1), device=x.device, dtype=torch.float32)
+        ops.static_quant_fp8_repeat(x, x_q, scale, x_s_repeat)
+        return x_q, x_s_repeat
+    from .sgl_kernel import sgl_per_tensor_quant_fp8
+
+    sgl_per_tensor_quant_fp8(x, x_q, scale, True)
+    return x_q, x_s
+
+
+def scaled_fp8_quant(
+    input: torch.Tensor,
+    scale: Optional[torch.Tensor] = None,
+    num_token_padding: Optional[int] = None,
+    use_per_token_if_dynamic: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp8_kernel.py:1429-1463: dynamic per-tensor (scale None), dynamic per-token, or static per-tensor quantization.
+    Rows added by ``num_token_padding`` are left unwritten, as in the reference."""
+    from .sgl_kernel import sgl_per_tensor_quant_fp8, sgl_per_token_quant_fp8
+
+    assert input.ndim == 2, f"Expected 2D input tensor, got {input.ndim}D"
+    shape = input.shape
+    if num_token_padding:
+        shape = (max(num_token_padding, input.shape[0]), shape[1])
+    output = torch.empty(shape, device=input.device, dtype=fp8_dtype)
+    if scale is None:
+        if use_per_token_if_dynamic:
+            scale = torch.empty((shape[0], 1), device=input.device, dtype=torch.float32)
+            sgl_per_token_quant_fp8(input, output[: input.shape[0]], scale[: input.shape[0]])
+        else:
+            scale = torch.zeros(1, device=input.device, dtype=torch.float32)
+            sgl_per_tensor_quant_fp8(input, output, scale, is_static=False)
+    else:
+        assert scale.numel() == 1, f"Expected scalar scale, got numel={scale.numel()}"
+        sgl_per_tensor_quant_fp8(input, output, scale, is_static=True)
+    return output, scale
+
+
 def sglang_per_token_group_quant_int8(
     x: torch.Tensor,
     group_size: int,

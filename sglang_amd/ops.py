@@ -39,6 +39,7 @@ SCHEMAS = {
     "fp8_scaled_mm": "fp8_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, "
     "Tensor? bias) -> Tensor",
     "sgl_per_token_quant_fp8": "sgl_per_token_quant_fp8(Tensor input, Tensor output_q, Tensor output_s) -> ()",
+    "sgl_per_tensor_quant_fp8": "sgl_per_tensor_quant_fp8(Tensor input, Tensor output_q, Tensor output_s, bool is_static) -> ()",
 }
 
 
@@ -201,6 +202,30 @@ def sgl_per_token_quant_fp8(input, output_q, output_s):
                                               M, K, _stream()))
 
 
+def sgl_per_tensor_quant_fp8(input, output_q, output_s, is_static):
+    """sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:102-130.  Dynamic mode merges block maxima into `output_s` with an
+    atomic max, so the caller passes zeros (the reference's scaled_fp8_quant does)."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _check_input(output_s, "output_s")
+    _require(input.dtype in (torch.float32, torch.float16, torch.bfloat16), "sgl_per_tensor_quant_fp8: unsupported input dtype")
+    _require(output_q.dtype == torch.float8_e4m3fn and output_q.numel() >= input.numel(), "sgl_per_tensor_quant_fp8: output_q mismatch")
+    _require(output_s.dtype == torch.float32 and output_s.numel() >= 1, "sgl_per_tensor_quant_fp8: output_s mismatch")
+    check(lib().mi355_per_tensor_quant_fp8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), output_s.data_ptr(),
+                                           input.numel(), int(bool(is_static)), None, 0, _stream()))
+
+
+def static_quant_fp8_repeat(input, output_q, scale, scale_rows):
+    """Static per-tensor quantization that also writes the scale once per row (static_quant_fp8 with repeat_scale,
+    python/sglang/srt/layers/quantization/fp8_kernel.py:635-665)."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _require(scale.numel() == 1 and scale.dtype == torch.float32 and scale.is_cuda, "only supports per-tensor scale")
+    _require(scale_rows.dtype == torch.float32 and scale_rows.is_contiguous(), "scale_rows must be contiguous float32")
+    check(lib().mi355_per_tensor_quant_fp8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), scale.data_ptr(),
+                                           input.numel(), 1, scale_rows.data_ptr(), scale_rows.numel(), _stream()))
+
+
 def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[torch.Tensor] = None):
     """sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532."""
     _require(mat_a.is_cuda, "mat_a must be a CUDA tensor")
@@ -361,6 +386,7 @@ def register() -> None:
         "sgl_per_token_group_quant_8bit_v2": sgl_per_token_group_quant_8bit_v2,
         "fp8_scaled_mm": fp8_scaled_mm,
         "sgl_per_token_quant_fp8": sgl_per_token_quant_fp8,
+        "sgl_per_tensor_quant_fp8": sgl_per_tensor_quant_fp8,
     }
     for name, fn in impls.items():
         if not hasattr(torch.ops.sgl_kernel, name):
@@ -374,6 +400,7 @@ def register() -> None:
     torch.library.register_fake("sgl_kernel::fp8_blockwise_scaled_mm", _fake_mm, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::fp8_scaled_mm", _fake_mm, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_token_quant_fp8", lambda *a: None, lib=_torch_lib)
+    torch.library.register_fake("sgl_kernel::sgl_per_tensor_quant_fp8", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit_v2", lambda *a: None, lib=_torch_lib)
     _registered = True

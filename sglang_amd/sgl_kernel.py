@@ -34,6 +34,11 @@ def sgl_per_token_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_
     torch.ops.sgl_kernel.sgl_per_token_quant_fp8.default(input, output_q, output_s)
 
 
+def sgl_per_tensor_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor, is_static: bool) -> None:
+    """sgl-kernel/python/sgl_kernel/gemm.py:145-153."""
+    torch.ops.sgl_kernel.sgl_per_tensor_quant_fp8.default(input, output_q, output_s, is_static)
+
+
 def sgl_per_token_group_quant_8bit(
     input: torch.Tensor,
     output_q: torch.Tensor,

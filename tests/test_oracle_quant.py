@@ -271,3 +271,42 @@ def test_per_token_quant_fp8_known_answer(oracle):
     back = q.view(torch.uint8)
     want = torch.where(codes == 0x80, torch.zeros((), dtype=torch.uint8), codes)  # -0 * scale = -0 -> encodes as 0x80 again
     assert torch.equal(back, codes) or torch.equal(back, want)
+
+
+# ---------------------------------------------------------------- per-tensor FP8 quantizer (one scale for the tensor)
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_per_tensor_quant_fp8_against_torch_fp32(oracle, dtype):
+    """sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:10-100 restated with torch CPU fp32 ops and torch's e4m3fn cast:
+    scale = amax / 448 (dynamic) or given (static), q = clamp(x * (1 / scale))."""
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(29, 1000, generator=g) * 7).to(dtype)  # 29000 elements: not a multiple of a 16-byte vector
+    x[3, 7] = -2.5e4
+    q, s = oracle.per_tensor_quant_fp8(x)
+    xf = x.float()
+    s_ref = (xf.abs().max() / 448.0).reshape(1)
+    q_ref = (xf * (1.0 / s_ref)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    assert torch.equal(s.view(torch.int32), s_ref.view(torch.int32))
+    assert torch.equal(q.view(torch.uint8), q_ref.view(torch.uint8))
+    assert int(q[3, 7].view(torch.uint8)) == 0xFE  # the extreme element encodes to -448
+    # static: a scale that saturates part of the tensor and is not a power of two
+    given = torch.tensor([0.013], dtype=torch.float32)
+    q2, s2 = oracle.per_tensor_quant_fp8(x, given)
+    q2_ref = (xf * (1.0 / given)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    assert torch.equal(s2, given) and torch.equal(q2.view(torch.uint8), q2_ref.view(torch.uint8))
+    assert int((q2.view(torch.uint8) & 0x7F).max()) == 0x7E  # saturated, never NaN
+
+
+def test_per_tensor_quant_fp8_known_answer_and_zero_tensor(oracle):
+    """Representable codes times a power-of-two scale come back unchanged with that scale; a tensor of zeros gets
+    scale 0 and, because fmin/fmax drop the NaN of 0 * inf, codes of +448 (what the reference's kernel produces)."""
+    g = torch.Generator().manual_seed(12)
+    codes = torch.randint(0, 256, (8, 512), generator=g, dtype=torch.uint8)
+    codes = torch.where((codes & 0x7F) == 0x7F, codes & 0xF7, codes)
+    codes[0, 0] = 0x7E
+    x = codes.view(torch.float8_e4m3fn).float() * 0.25
+    q, s = oracle.per_tensor_quant_fp8(x)
+    assert float(s) == 0.25
+    assert torch.equal(q.view(torch.uint8), codes)
+    qz, sz = oracle.per_tensor_quant_fp8(torch.zeros(4, 64))
+    assert float(sz) == 0.0 and bool((qz.view(torch.uint8) == 0x7E).all())
