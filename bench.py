@@ -16,6 +16,7 @@ Infinity Cache.
   fp8_decode   FP8 gate_up at M=1          int8_gemm             INT8 gate_up (K=4096 -> N=28672) at M=4096
   fp8:M:K:N    any blockwise-FP8 linear    int8:M:K:N            any INT8 linear
   copy         a plain 256 MiB device copy (calibration of the HBM traffic counters)
+  silu_quant   silu(gate) * up fused in front of the group quantizer (packed UE8M0 scales)
 
 Per-launch durations are HIP events on the launch stream (torch's current stream, which is the stream
 handed to the C ABI).  `roofline.achieved` = algorithmic FLOPs (2*M*N*K) or bytes per launch / MEDIAN
@@ -353,6 +354,39 @@ def bench_int8_gemm(name, M, K, N, steps, warmup, with_cpu=False):
     return rec
 
 
+def bench_silu_quant(steps, warmup):
+    """silu(gate) * up fused in front of the group quantizer (packed UE8M0 scales), [32768, 2 x 2048] bf16."""
+    import torch
+
+    from sglang_amd import _lib, fp8_kernel
+
+    dev = torch.device("cuda:0")
+    T, H = 32768, 2048
+    nbuf = 3
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    xs = [torch.randn(T, 2 * H, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(nbuf)]
+    qs = [torch.empty(T, H, dtype=torch.float8_e4m3fn, device=dev) for _ in range(nbuf)]
+    ss = [fp8_kernel.create_per_token_group_quant_fp8_output_scale((T, H), dev, 128, True, True, True) for _ in range(nbuf)]
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    args = [(xs[i].data_ptr(), _lib.BF16, qs[i].data_ptr(), ss[i].data_ptr(), 1, T, H, None, 0, ss[i].stride(1), stream)
+            for i in range(nbuf)]
+
+    def step(i):
+        _lib.check(L.mi355_silu_mul_group_quant_fp8(*args[i]))
+
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms, b2b)
+    alg = T * H * (4 + 1) + T * (H // 128)
+    return {
+        "workload": f"silu_mul_quant M={T} H={H} g=128 bf16 [M,2H] -> e4m3fn [M,H], packed UE8M0 scales",
+        "value": alg / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "f32 arithmetic, e4m3fn out", "kernel": "silu_mul_quant",
+        "roofline": _roofline(0, alg, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
+    }
+
+
 def bench_copy(steps, warmup):
     """Plain device-to-device copy of a known size (256 MiB read + 256 MiB written per launch): the calibration
     workload for the FETCH_SIZE / WRITE_SIZE counters behind `roofline.traffic`."""
@@ -443,6 +477,8 @@ def main():
         rec = bench_quant(S, W, wl == "quant_ue8m0", cpu)
     elif wl == "copy":
         rec = bench_copy(S, W)
+    elif wl == "silu_quant":
+        rec = bench_silu_quant(S, W)
     elif wl == "fp8_decode":
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 1, K, N, S, W, cpu)
@@ -462,6 +498,7 @@ def main():
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 4096, K, N, S, W, cpu)
         if full:
+            also.append(bench_silu_quant(S, W))
             K, N = DSV3_MLP["down"]
             also.append(bench_fp8_gemm("down", 4096, K, N, S, W, False))
             for nm, (K, N) in DSV3_MLA.items():

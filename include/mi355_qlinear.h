@@ -173,6 +173,22 @@ int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, in
 int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
 
 /*
+ * silu(gate) * up fused in front of the 1 x 128 FP8 group quantizer (the MoE expert MLP's activation + quantization).
+ *   x [E, T, 2 * H] contiguous F16/BF16, each row gate | up;  q [E, T, H] e4m3fn contiguous;
+ *   v = T( float(T(silu(float(gate)))) * float(up) ) in the input's type T, then per 128 values amax = max(1e-10, max |v|),
+ *   e = ceil(log2(amax / 448)), q = e4m3fn(clamp(v * 2^-e)), scale byte e + 127.
+ *   s_words: int32 words of four exponent bytes (byte kg & 3 of word kg >> 2 for group kg of a row); word (e, t, kw) lies
+ *   at s_words[e * s_expert_stride + kw * s_k_stride + t] - token index fastest, the packed column-major layout of
+ *   create_per_token_group_quant_fp8_output_scale(scale_ue8m0=True).  Unused bytes of a row's last word are set to 0.
+ *   masked_m: NULL, or [E] int32 on the device: tokens t >= masked_m[e] of expert e are neither read nor written.
+ * Replaces sgl_per_token_group_quant_8bit_v2 with fuse_silu_and_mul (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:
+ * 394-514, kernel :250-392, masked scheduler :194-238), which exists for exactly this scale format.  exp is evaluated by a
+ * fixed sequence of fp32 operations, within 1 ulp (the reference uses the GPU's approximate intrinsic).  H % 128 == 0.
+ */
+int mi355_silu_mul_group_quant_fp8(const void* x, int x_dtype, void* q, void* s_words, int64_t E, int64_t T, int64_t H,
+                                   const int32_t* masked_m, int64_t s_expert_stride, int64_t s_k_stride, void* stream);
+
+/*
  * Per-tensor FP8 activation quantization: ONE fp32 scale for the whole tensor, q = e4m3fn(clamp(x * (1 / scale))).
  *   is_static == 0: scale = max |x| / 448 is computed first.  *scale must hold 0.0f on entry (block maxima are merged into
  *                   it with an atomic max; the reference's wrapper passes torch.zeros(1) the same way).

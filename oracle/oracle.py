@@ -60,6 +60,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_per_token_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64]
         L.oracle_per_token_quant_fp8.restype = i32
         L.oracle_per_tensor_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i32]
+        L.oracle_silu_mul.argtypes = [vp, i32, vp, i64, i64]
+        L.oracle_silu_mul.restype = i32
+        L.oracle_expf.argtypes = [ctypes.c_float]
+        L.oracle_expf.restype = ctypes.c_float
         L.oracle_per_tensor_quant_fp8.restype = i32
         L.oracle_fp8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32, vp] + [i64] * 6
         L.oracle_fp8_scaled_mm.restype = i32
@@ -184,6 +188,20 @@ def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     rc = lib().oracle_per_token_quant_fp8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), M, K)
     assert rc == 0
     return q.view(torch.float8_e4m3fn), s
+
+
+def silu_mul(x: torch.Tensor) -> torch.Tensor:
+    """x [..., 2H] bf16/fp16 -> [..., H] of the same dtype: T(silu(gate)) * up with the roundings of the v2 quantizer."""
+    x = _cpu(x).contiguous()
+    H = x.shape[-1] // 2
+    out = torch.zeros(*x.shape[:-1], H, dtype=x.dtype)
+    rc = lib().oracle_silu_mul(x.data_ptr(), _DT[x.dtype], out.data_ptr(), x.numel() // (2 * H), H)
+    assert rc == 0
+    return out
+
+
+def expf(v: float) -> float:
+    return float(lib().oracle_expf(float(v)))
 
 
 def per_tensor_quant_fp8(x: torch.Tensor, scale: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:

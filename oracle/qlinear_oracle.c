@@ -24,6 +24,8 @@
  *                             sgl-kernel/tests/test_int8_gemm.py:11-17 (torch order)
  *   oracle_per_token_quant_int8  python/sglang/srt/layers/quantization/int8_kernel.py:28-52
  *   oracle_per_token_quant_fp8   sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85
+ *   oracle_silu_mul              sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:32-40, :318-331 (the activation the v2
+ *                                quantizer fuses in front of oracle_group_quant: T(silu(float(gate))) * up, in T)
  *   oracle_per_tensor_quant_fp8  sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:10-100,
  *                                python/sglang/srt/layers/quantization/fp8_kernel.py:593-632 (static_quant_fp8)
  *   oracle_fp8_scaled_mm         sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:529-547, :1450-1532
@@ -296,6 +298,49 @@ int oracle_per_token_quant_fp8(const void* x, int x_dtype, uint8_t* q, float* s,
       float t = load_as_f32(x, x_dtype, (size_t)row * K + j) * inv;
       t = fmaxf(fminf(t, 448.0f), -448.0f);
       q[(size_t)row * K + j] = oracle_e4m3fn_encode(t);
+    }
+  }
+  return 0;
+}
+
+/* exp(x) in single precision from individually rounded fp32 operations only (multiply, round-to-integer, fused
+ * multiply-add, scaling by a power of two), so that a GPU evaluating the same sequence gets the same bits: n = rint(x *
+ * log2(e)), r = x - n * ln2 in two FMA steps (ln2 split so that n * hi is exact), Taylor polynomial of degree 7 in Horner
+ * form with FMAs (|r| <= 0.3466: truncation below 6e-9), times 2^n.  Within 1 ulp of exp on the whole range. */
+float oracle_expf(float x) {
+  if (x > 88.72284f) return INFINITY;
+  if (x < -103.97208f) return 0.0f;
+  const float n = rintf(x * 1.44269504f);
+  float r = fmaf(n, -0.693145751953125f, x);
+  r = fmaf(n, -1.42860682e-6f, r);
+  float p = 1.98412698e-4f; /* 1/5040 */
+  p = fmaf(p, r, 1.38888889e-3f); /* 1/720 */
+  p = fmaf(p, r, 8.33333333e-3f); /* 1/120 */
+  p = fmaf(p, r, 4.16666667e-2f); /* 1/24 */
+  p = fmaf(p, r, 1.66666667e-1f); /* 1/6 */
+  p = fmaf(p, r, 0.5f);
+  p = fmaf(p, r, 1.0f);
+  p = fmaf(p, r, 1.0f);
+  return ldexpf(p, (int)n);
+}
+
+/* x [rows, 2 * H] (gate | up halves of each row) -> out [rows, H] in the same 16-bit type T:
+ *   out = T( float(T(silu(float(gate)))) * float(up) ),  silu(g) = g / (1 + exp(-g))
+ * i.e. the activation is rounded to T, then multiplied by `up` in T (one rounding of the exact product), as
+ * per_token_group_quant_8bit_v2.cu:318-331 does with its element type.  The reference evaluates exp with the GPU's
+ * approximate intrinsic (:32-40), whose bits differ between its own kernels, and compares with a tolerance
+ * (sgl-kernel/tests/test_per_token_group_quant_8bit.py:153-168); here exp is oracle_expf. */
+int oracle_silu_mul(const void* x, int dtype, void* out, int64_t rows, int64_t H) {
+  if (dtype != DT_BF16 && dtype != DT_F16) return 1;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    for (int64_t j = 0; j < H; ++j) {
+      const float g = load_as_f32(x, dtype, (size_t)(r * 2 * H + j));
+      const float u = load_as_f32(x, dtype, (size_t)(r * 2 * H + H + j));
+      const float sl = g / (1.0f + oracle_expf(-g));
+      store_from_f32(out, dtype, (size_t)(r * H + j), sl);               /* T(silu) */
+      const float st = load_as_f32(out, dtype, (size_t)(r * H + j));
+      store_from_f32(out, dtype, (size_t)(r * H + j), st * u);           /* exact product, one rounding */
     }
   }
   return 0;

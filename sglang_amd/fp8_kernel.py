@@ -118,6 +118,37 @@ def _per_token_group_quant_8bit_raw(
 per_token_group_quant_fp8 = _per_token_group_quant_8bit_raw
 
 
+def _per_token_group_quant_8bit_fuse_silu_and_mul(
+    x: torch.Tensor,
+    group_size: int,
+    dst_dtype: torch.dtype,
+    column_major_scales: bool,
+    scale_tma_aligned: bool,
+    scale_ue8m0: bool,
+    masked_m: Optional[torch.Tensor],
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp8_kernel.py:325-397: silu(gate) * up, then the 1x128 quantizer with packed UE8M0 scales; ``x`` is [T, 2H] or,
+    with ``masked_m``, [E, T, 2H].  The reference goes through a Triton kernel and DeepGEMM's layout transform; its own
+    test holds that pair equal to the fused v2 kernel, which is what runs here.  Outputs start as zeros, as there
+    (rows past ``masked_m`` stay zero)."""
+    assert column_major_scales
+    assert scale_tma_aligned
+    assert scale_ue8m0
+    assert group_size == 128
+    out_shape = (*x.shape[:-1], x.shape[-1] // 2)
+    output = torch.zeros(out_shape, device=x.device, dtype=dst_dtype)
+    output_scale = create_per_token_group_quant_fp8_output_scale(
+        x_shape=out_shape, device=x.device, group_size=group_size, column_major_scales=True, scale_tma_aligned=True,
+        scale_ue8m0=True,
+    )
+    output_scale.zero_()
+    if x.numel() > 0:
+        sgl_per_token_group_quant_8bit(
+            x, output, output_scale, group_size, 1e-10, fp8_min, fp8_max, True, True, masked_m, enable_v2=True,
+        )
+    return output, output_scale
+
+
 def per_token_group_quant_8bit(
     x: torch.Tensor,
     group_size: int,
@@ -130,8 +161,13 @@ def per_token_group_quant_8bit(
     masked_m: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """fp8_kernel.py:400-430."""
-    if fuse_silu_and_mul or masked_m is not None:
-        raise NotImplementedError("fuse_silu_and_mul / masked_m belong to the MoE path, which is not built")
+    if fuse_silu_and_mul:
+        return _per_token_group_quant_8bit_fuse_silu_and_mul(
+            x=x, group_size=group_size, dst_dtype=dst_dtype, column_major_scales=column_major_scales,
+            scale_tma_aligned=scale_tma_aligned, scale_ue8m0=scale_ue8m0, masked_m=masked_m,
+        )
+    if masked_m is not None:
+        raise NotImplementedError("masked_m without fuse_silu_and_mul has no kernel in the reference either")
     return _per_token_group_quant_8bit_raw(
         x=x,
         group_size=group_size,

@@ -98,12 +98,45 @@ def sgl_per_token_group_quant_8bit(input, output_q, output_s, group_size, eps, f
                  _lib.QUANT_DIV, 1e-10, "sgl_per_token_group_quant_8bit")
 
 
+def _silu_mul_group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, masked_m, op):
+    """The fuse_silu_and_mul branch of per_token_group_quant_8bit_v2.cu:394-514: input [T, 2H] or, with masked_m,
+    [E, T, 2H]; the reference instantiates it for column-major packed UE8M0 scales only (:455-470)."""
+    if not (scale_ue8m0 and output_s.dtype == torch.int32 and output_s.dim() >= 2 and output_s.stride(-2) == 1 and group_size == 128
+            and output_q.dtype == torch.float8_e4m3fn):
+        raise NotImplementedError(f"{op}: fuse_silu_and_mul is built for group 128, e4m3fn codes and column-major packed "
+                                  "UE8M0 scales, the one combination the reference instantiates")
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _require(input.numel() > 0, f"{op}: input.numel() > 0")
+    _require(abs(1e-10 - eps) < 1e-13, f"{op}: eps must be 1e-10")
+    masked = masked_m is not None
+    _require(output_s.dim() == (3 if masked else 2), f"{op}: output_s.dim() == {3 if masked else 2}")
+    _require(input.dim() == output_s.dim(), f"{op}: input and output_s ranks differ")
+    _require(input.dtype in (torch.float16, torch.bfloat16), f"{op}: input must be float16 or bfloat16")
+    _require((fp8_min, fp8_max) == (-448.0, 448.0), f"{op}: CHECK_EQ(dst_dtype_info::MIN/MAX, min_8bit/max_8bit) failed")
+    H = output_q.size(-1)
+    T = output_q.size(-2)
+    E = input.size(0) if masked else 1
+    _require(input.size(-1) == 2 * H and input.size(-2) == T, f"{op}: input must be [..., tokens, 2 * hidden]")
+    _require(H % 128 == 0, f"{op}: hidden size must be a multiple of 128")
+    _require(output_s.size(-2) == T and output_s.size(-1) * 4 >= H // 128, f"{op}: output_s shape mismatch")
+    mm = None
+    if masked:
+        _require(masked_m.is_cuda and masked_m.dtype == torch.int32 and masked_m.numel() == E and masked_m.is_contiguous(),
+                 f"{op}: masked_m must be a contiguous int32 CUDA tensor with one entry per expert")
+        mm = masked_m.data_ptr()
+    check(lib().mi355_silu_mul_group_quant_fp8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), output_s.data_ptr(),
+                                               E, T, H, mm, output_s.stride(0) if masked else 0, output_s.stride(-1), _stream()))
+
+
 def sgl_per_token_group_quant_8bit_v2(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0,
                                       fuse_silu_and_mul, masked_m):
     """sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:394-514: q = x * (max / amax)."""
     op = "sgl_per_token_group_quant_8bit_v2"
-    if fuse_silu_and_mul or masked_m is not None:
-        raise NotImplementedError(f"{op}: fuse_silu_and_mul / masked_m (expert-parallel MoE layouts) are not built")
+    if fuse_silu_and_mul:
+        return _silu_mul_group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, masked_m, op)
+    if masked_m is not None:
+        raise NotImplementedError(f"{op}: masked_m without fuse_silu_and_mul has no kernel in the reference either")
     _require(input.numel() > 0, f"{op}: input.numel() > 0")
     _require(abs(1e-10 - eps) < 1e-13, f"{op}: eps must be 1e-10")
     _require(group_size in (16, 32, 64, 128), "Unsupported group_size")

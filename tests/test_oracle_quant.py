@@ -310,3 +310,44 @@ def test_per_tensor_quant_fp8_known_answer_and_zero_tensor(oracle):
     assert torch.equal(q.view(torch.uint8), codes)
     qz, sz = oracle.per_tensor_quant_fp8(torch.zeros(4, 64))
     assert float(sz) == 0.0 and bool((qz.view(torch.uint8) == 0x7E).all())
+
+
+# ---------------------------------------------------------------- silu(gate) * up in front of the v2 quantizer
+
+def test_oracle_expf_within_one_ulp(oracle):
+    """The oracle's exp is built from individually rounded fp32 operations (so that the GPU kernel can repeat it bit for
+    bit); against fp64 exp it must stay within 1 ulp over the whole range, with exact limits."""
+    import math
+
+    g = torch.Generator().manual_seed(21)
+    xs = torch.cat([torch.linspace(-104.0, 88.7, 20001), torch.randn(20000, generator=g) * 4, torch.tensor([0.0, -0.0, 1.0, -1.0])])
+    worst = 0.0
+    for v in xs.tolist():
+        got = oracle.expf(v)
+        want = math.exp(v)
+        want32 = float(torch.tensor(want, dtype=torch.float64).to(torch.float32))
+        if want32 == 0.0 or math.isinf(want32) or want < 1.2e-38:
+            continue  # subnormal results only need to vanish next to 1
+        ulp = abs(float(torch.nextafter(torch.tensor(want32), torch.tensor(float("inf")))) - want32)
+        worst = max(worst, abs(got - want) / ulp)
+    assert worst <= 1.0, worst
+    assert oracle.expf(0.0) == 1.0 and oracle.expf(100.0) == float("inf") and oracle.expf(-200.0) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_silu_mul_against_torch(oracle, dtype):
+    """per_token_group_quant_8bit_v2.cu:318-331: T(silu(float(gate))) * up in T.  torch's CPU silu uses a correctly
+    rounded-ish exp, the oracle its own 1-ulp exp, so after rounding to T the two may differ in isolated elements by one
+    unit of T; a wrong formula (activation not rounded to T first, halves swapped, product in fp32) differs everywhere."""
+    g = torch.Generator().manual_seed(22)
+    x = (torch.randn(64, 2 * 1024, generator=g) * 3).to(dtype)
+    x[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 100.0, -100.0, 1e-3, -1e-3]).to(dtype)
+    got = oracle.silu_mul(x)
+    gate, up = x[:, :1024], x[:, 1024:]
+    want = torch.nn.functional.silu(gate.float()).to(dtype) * up
+    assert got.shape == want.shape and got.dtype == dtype
+    diff = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+    assert int(diff.max()) <= 1 and float((diff != 0).float().mean()) < 2e-4, (int(diff.max()), float((diff != 0).float().mean()))
+    # discriminating alternatives must be far away
+    alt = (torch.nn.functional.silu(gate.float()) * up.float()).to(dtype)  # product before the first rounding
+    assert float((alt.view(torch.int16) != got.view(torch.int16)).float().mean()) > 0.05
