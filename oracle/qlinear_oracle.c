@@ -38,6 +38,10 @@
  * reference leaves it to the tensor cores, and compares with a tolerance only.
  * The oracle sums each block in double precision ("parity unpinned" for that
  * summation order; the GPU kernel is held to the reference's tolerance instead).
+ * Likewise "parity unpinned": the bits of exp inside oracle_silu_mul.  The reference calls the GPU's approximate
+ * __expf there (per_token_group_quant_8bit_v2.cu:32-40) and compares its kernels with a tolerance; oracle_expf is one
+ * fixed definition, pinned to fp64 exp within 1 ulp, and oracle_silu_mul is pinned against torch's silu up to isolated
+ * one-unit differences after the rounding to the 16-bit type.
  */
 #include <math.h>
 #include <stddef.h>
