@@ -48,6 +48,7 @@ __device__ __attribute__((aligned(16))) uint32_t r_zero16[4] = {0, 0, 0, 0};
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
+typedef const __attribute__((address_space(4))) float* cfloat_ptr;
 
 struct Frag {
   u32x4 lo, hi;
@@ -202,7 +203,10 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
   float sb_cur[KB_PER], sb_nxt[KB_PER];
   auto load_sb = [&](int g, float (&dst)[KB_PER]) {
     if constexpr (IS_FP8) {
-      const float* sb_row = p.sb + (int64_t)(g_first + min(g, groups - 1)) * p.sb_sn + (int64_t)kb_begin * p.sb_sk;
+      // uniform addresses through a constant-address-space pointer: scalar loads, which do not count in vmcnt, so the
+      // copy of these values at the end of a group never waits for the weight ring
+      const cfloat_ptr sb_row =
+          (cfloat_ptr)(p.sb + (int64_t)(g_first + min(g, groups - 1)) * p.sb_sn + (int64_t)kb_begin * p.sb_sk);
 #pragma unroll
       for (int d = 0; d < KB_PER; ++d) dst[d] = sb_row[(int64_t)min(d, kb_valid - 1) * p.sb_sk];
     } else {
