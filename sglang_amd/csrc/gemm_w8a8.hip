@@ -252,7 +252,9 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(const GemmParams p) {
   }
 }
 
-// Sums the split-K partial tiles in ascending split order and applies the epilogue.
+// Sums the split-K partial tiles in ascending split order and applies the epilogue.  The partial tiles are fetched eight at
+// a time before they are added: with one load per addition the kernel is a chain of memory latencies (4.6 us for 7 splits).
+constexpr int REDUCE_BATCH = 8;
 template <bool IS_FP8>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) {
   const int64_t total = (int64_t)p.M * p.N;
@@ -263,10 +265,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
   const int n = (int)(idx - (int64_t)m * p.N);
   if constexpr (IS_FP8) {
     const float* w = reinterpret_cast<const float*>(p.ws) + idx;
-    v4f s = *reinterpret_cast<const v4f*>(w);
-    for (int k = 1; k < p.splits; ++k) {
-      const v4f t = *reinterpret_cast<const v4f*>(w + (int64_t)k * total);
-      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
+    v4f s = {0.f, 0.f, 0.f, 0.f};  // 0 + first partial is exact, so the sum is the one that starts from the first partial
+    for (int k0 = 0; k0 < p.splits; k0 += REDUCE_BATCH) {
+      v4f t[REDUCE_BATCH];
+#pragma unroll
+      for (int j = 0; j < REDUCE_BATCH; ++j)
+        t[j] = *reinterpret_cast<const v4f*>(w + (int64_t)min(k0 + j, p.splits - 1) * total);
+#pragma unroll
+      for (int j = 0; j < REDUCE_BATCH; ++j)
+        if (k0 + j < p.splits) s[0] += t[j][0], s[1] += t[j][1], s[2] += t[j][2], s[3] += t[j][3];
     }
     float r[4] = {s[0], s[1], s[2], s[3]};
     fp8_channel_epilogue(p, n, r);
@@ -274,10 +281,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
     store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, r, 4, vec_ok);
   } else {
     const int* w = reinterpret_cast<const int*>(p.ws) + idx;
-    v4i s = *reinterpret_cast<const v4i*>(w);
-    for (int k = 1; k < p.splits; ++k) {
-      const v4i t = *reinterpret_cast<const v4i*>(w + (int64_t)k * total);
-      s[0] += t[0], s[1] += t[1], s[2] += t[2], s[3] += t[3];
+    v4i s = {0, 0, 0, 0};
+    for (int k0 = 0; k0 < p.splits; k0 += REDUCE_BATCH) {
+      v4i t[REDUCE_BATCH];
+#pragma unroll
+      for (int j = 0; j < REDUCE_BATCH; ++j)
+        t[j] = *reinterpret_cast<const v4i*>(w + (int64_t)min(k0 + j, p.splits - 1) * total);
+#pragma unroll
+      for (int j = 0; j < REDUCE_BATCH; ++j)
+        if (k0 + j < p.splits) s[0] += t[j][0], s[1] += t[j][1], s[2] += t[j][2], s[3] += t[j][3];
     }
     if (p.out_dtype == MI355_I32) {
       int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
