@@ -44,8 +44,8 @@ INT8_PEAK_TOPS = 5000.0   # dense int8 MFMA
 
 METRIC = "blockwise-FP8 GEMM TFLOPS & %MFMA peak; quant GB/s & %HBM peak (1 GPU)"
 DATA = ("synthetic, seeded, resident in HBM before the timed region; activations bf16 N(0,1) + 0.1% x50 outliers quantized "
-        "1x128 by the GPU quantizer; FP8 weights N(0,0.02) quantized per 128x128 block (drawn on the device); INT8 operands "
-        "uniform in [-127,127]")
+        "1x128 by the GPU quantizer; FP8 weights N(0,0.02) quantized per 128x128 block (drawn on the device); INT8 weights "
+        "N(0,0.02) quantized per channel, INT8 activations the same bf16 data quantized per token by the GPU quantizer")
 
 
 def r4(x):
@@ -307,14 +307,29 @@ def bench_int8_gemm(name, M, K, N, steps, warmup, with_cpu=False):
     gen = torch.Generator(device=dev)
     gen.manual_seed(N * 10009 + K)
     nbuf = max(2, min(6, int(600e6 // (N * K)) + 1))
-    ws = [torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev, generator=gen) for _ in range(nbuf)]
-    a = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev, generator=gen)
-    sa = torch.rand(M, 1, device=dev, generator=gen) * 0.05
-    sb = torch.rand(N, device=dev, generator=gen) * 1e-3
+    # operands as a W8A8 checkpoint and its activations have them: N(0, 0.02) weights quantized symmetrically per output
+    # channel, bf16 N(0, 1) activations (with outliers) quantized per token by the GPU quantizer.  Timing depends on the
+    # data through the chip's power state; uniformly random bytes would be the worst case, not a representative one.
+    from sglang_amd.int8_kernel import per_token_quant_int8
+    from sglang_amd.workloads import make_activation
+
+    ws, sbs = [], []
+    for _ in range(nbuf):
+        q = torch.empty(N, K, dtype=torch.int8, device=dev)
+        sc = torch.empty(N, dtype=torch.float32, device=dev)
+        for n0 in range(0, N, 4096):
+            w = torch.randn(min(4096, N - n0), K, generator=gen, device=dev) * 0.02
+            amax = w.abs().amax(dim=1, keepdim=True).clamp(min=1e-8)
+            q[n0:n0 + w.shape[0]] = torch.round(w * (127.0 / amax)).to(torch.int8)
+            sc[n0:n0 + w.shape[0]] = (amax / 127.0).view(-1)
+        ws.append(q)
+        sbs.append(sc)
+    sb = sbs[0]
+    a, sa = per_token_quant_int8(make_activation(M, K).to(dev))
     bias = torch.randn(N, device=dev, generator=gen).to(torch.bfloat16)
 
     def step(i):
-        return sgl_kernel.int8_scaled_mm(a, ws[i].t(), sa, sb, torch.bfloat16, bias)
+        return sgl_kernel.int8_scaled_mm(a, ws[i].t(), sa, sbs[i], torch.bfloat16, bias)
 
     direct = M <= 256 or N * K <= 16e6  # launches of tens of microseconds
     if direct:
@@ -323,7 +338,7 @@ def bench_int8_gemm(name, M, K, N, steps, warmup, with_cpu=False):
         wsbuf = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
         outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
         stream = torch.cuda.current_stream().cuda_stream
-        args = [(a.data_ptr(), ws[i].data_ptr(), sa.data_ptr(), sb.data_ptr(), bias.data_ptr(), outs[i].data_ptr(), _lib.BF16,
+        args = [(a.data_ptr(), ws[i].data_ptr(), sa.data_ptr(), sbs[i].data_ptr(), bias.data_ptr(), outs[i].data_ptr(), _lib.BF16,
                  M, N, K, a.stride(0), ws[i].stride(0), outs[i].stride(0), wsbuf.data_ptr(), wsb, stream) for i in range(nbuf)]
 
         def step(i):  # noqa: F811
