@@ -76,6 +76,7 @@ __device__ __forceinline__ void issue_set_b(const JState& s, uint8_t* stage, int
 
 __device__ __forceinline__ void compute_end() {
   __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_setprio(2);  // the memory phase that follows runs above the other group's MFMA stream (measured: ~1 %)
   asm volatile("s_barrier" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 }
@@ -84,6 +85,7 @@ __device__ __forceinline__ void memory_end() {
   static_assert(J_SET_A + J_SET_B == 8, "the wait is written for eight loads per K step");
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_s_setprio(0);
   __builtin_amdgcn_sched_barrier(0);
 }
 
