@@ -173,6 +173,18 @@ int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, in
 int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
 
 /*
+ * Weight-side 128 x 128 block quantization (load time: re-quantizing a block-FP8 checkpoint to power-of-two scales).
+ *   mi355_block_cast_to_fp8:  x [m, n] contiguous F32/F16/BF16 -> q [m, n] e4m3fn, s [ceil(m/128), ceil(n/128)] fp32
+ *       contiguous;  amax = max(1e-4, max |x| over the block), s = 2^ceil(log2(amax / 448)) exactly, q = e4m3fn(x * (1 / s)).
+ *       Replaces per_block_cast_to_fp8 + ceil_to_ue8m0 (python/sglang/srt/layers/quantization/fp8_utils.py:487-505), which
+ *       the reference writes in torch ops (zero padding to whole blocks included, which changes no maximum).
+ *   mi355_block_dequant_fp8:  q [n, k] e4m3fn, s [ceil(n/128), ceil(k/128)] fp32 contiguous -> out [n, k] = T(float(q) * s).
+ *       Replaces block_quant_dequant (fp8_utils.py:392-413) for 128 x 128 blocks.
+ */
+int mi355_block_cast_to_fp8(const void* x, int x_dtype, void* q, float* s, int64_t m, int64_t n, void* stream);
+int mi355_block_dequant_fp8(const void* q, const float* s, void* out, int out_dtype, int64_t n, int64_t k, void* stream);
+
+/*
  * silu(gate) * up fused in front of the 1 x 128 FP8 group quantizer (the MoE expert MLP's activation + quantization).
  *   x [E, T, 2 * H] contiguous F16/BF16, each row gate | up;  q [E, T, H] e4m3fn contiguous;
  *   v = T( float(T(silu(float(gate)))) * float(up) ) in the input's type T, then per 128 values amax = max(1e-10, max |v|),

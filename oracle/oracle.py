@@ -60,6 +60,10 @@ def lib() -> ctypes.CDLL:
         L.oracle_per_token_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64]
         L.oracle_per_token_quant_fp8.restype = i32
         L.oracle_per_tensor_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i32]
+        L.oracle_block_cast_to_fp8.argtypes = [vp, i32, vp, vp, i64, i64]
+        L.oracle_block_cast_to_fp8.restype = i32
+        L.oracle_block_dequant_fp8.argtypes = [vp, vp, vp, i32, i64, i64]
+        L.oracle_block_dequant_fp8.restype = i32
         L.oracle_silu_mul.argtypes = [vp, i32, vp, i64, i64]
         L.oracle_silu_mul.restype = i32
         L.oracle_expf.argtypes = [ctypes.c_float]
@@ -188,6 +192,26 @@ def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     rc = lib().oracle_per_token_quant_fp8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), M, K)
     assert rc == 0
     return q.view(torch.float8_e4m3fn), s
+
+
+def block_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x [m,n] -> (e4m3fn [m,n], fp32 power-of-two scales [ceil(m/128), ceil(n/128)])."""
+    x = _cpu(x).contiguous()
+    m, n = x.shape
+    q = torch.zeros(m, n, dtype=torch.uint8)
+    s = torch.zeros((m + 127) // 128, (n + 127) // 128, dtype=torch.float32)
+    rc = lib().oracle_block_cast_to_fp8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), m, n)
+    assert rc == 0
+    return q.view(torch.float8_e4m3fn), s
+
+
+def block_dequant_fp8(q: torch.Tensor, s: torch.Tensor, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    q, s = _cpu(q).contiguous(), _cpu(s).contiguous().to(torch.float32)
+    n, k = q.shape
+    out = torch.zeros(n, k, dtype=dtype)
+    rc = lib().oracle_block_dequant_fp8(q.view(torch.uint8).data_ptr(), s.data_ptr(), out.data_ptr(), _DT[dtype], n, k)
+    assert rc == 0
+    return out
 
 
 def silu_mul(x: torch.Tensor) -> torch.Tensor:

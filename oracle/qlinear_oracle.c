@@ -26,6 +26,8 @@
  *   oracle_per_token_quant_fp8   sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85
  *   oracle_silu_mul              sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:32-40, :318-331 (the activation the v2
  *                                quantizer fuses in front of oracle_group_quant: T(silu(float(gate))) * up, in T)
+ *   oracle_block_cast_to_fp8     python/sglang/srt/layers/quantization/fp8_utils.py:487-505 (per_block_cast_to_fp8, ceil_to_ue8m0)
+ *   oracle_block_dequant_fp8     python/sglang/srt/layers/quantization/fp8_utils.py:392-413 (block_quant_dequant)
  *   oracle_per_tensor_quant_fp8  sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:10-100,
  *                                python/sglang/srt/layers/quantization/fp8_kernel.py:593-632 (static_quant_fp8)
  *   oracle_fp8_scaled_mm         sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:529-547, :1450-1532
@@ -304,6 +306,42 @@ int oracle_per_token_quant_fp8(const void* x, int x_dtype, uint8_t* q, float* s,
       q[(size_t)row * K + j] = oracle_e4m3fn_encode(t);
     }
   }
+  return 0;
+}
+
+/* x [m, n] -> q e4m3fn [m, n], s fp32 [ceil(m/128), ceil(n/128)]: per 128 x 128 block amax = max(1e-4, max |x|),
+ * s = 2^ceil(log2(amax / 448)), q = RNE(x * (1 / s))  (fp8_utils.py:487-505; the reference zero-pads to whole blocks and
+ * takes log2 / ceil / pow in fp32 tensor ops - here ceil(log2) comes from the exponent and mantissa bits, the exact value). */
+int oracle_block_cast_to_fp8(const void* x, int x_dtype, uint8_t* q, float* s, int64_t m, int64_t n) {
+  const int64_t bm = (m + 127) / 128, bn = (n + 127) / 128;
+#pragma omp parallel for schedule(static) collapse(2)
+  for (int64_t i = 0; i < bm; ++i)
+    for (int64_t j = 0; j < bn; ++j) {
+      const int64_t r1 = (i + 1) * 128 < m ? (i + 1) * 128 : m, c1 = (j + 1) * 128 < n ? (j + 1) * 128 : n;
+      float amax = 0.f;
+      for (int64_t r = i * 128; r < r1; ++r)
+        for (int64_t c = j * 128; c < c1; ++c) amax = fmaxf(amax, fabsf(load_as_f32(x, x_dtype, (size_t)(r * n + c))));
+      amax = fmaxf(amax, 1e-4f);
+      const float t = amax / 448.0f;
+      int e;
+      const float mant = frexpf(t, &e); /* t = mant * 2^e, mant in [0.5, 1) */
+      const int ce = (mant == 0.5f) ? e - 1 : e; /* ceil(log2 t) */
+      const float sf = ldexpf(1.0f, ce), inv = ldexpf(1.0f, -ce);
+      s[i * bn + j] = sf;
+      for (int64_t r = i * 128; r < r1; ++r)
+        for (int64_t c = j * 128; c < c1; ++c)
+          q[r * n + c] = oracle_e4m3fn_encode(load_as_f32(x, x_dtype, (size_t)(r * n + c)) * inv);
+    }
+  return 0;
+}
+
+/* q [n, k] e4m3fn, s [ceil(n/128), ceil(k/128)] -> out [n, k] = T(float(q) * s)  (fp8_utils.py:392-413). */
+int oracle_block_dequant_fp8(const uint8_t* q, const float* s, void* out, int out_dtype, int64_t n, int64_t k) {
+  const int64_t bk = (k + 127) / 128;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < n; ++r)
+    for (int64_t c = 0; c < k; ++c)
+      store_from_f32(out, out_dtype, (size_t)(r * k + c), oracle_e4m3fn_decode(q[r * k + c]) * s[(r / 128) * bk + c / 128]);
   return 0;
 }
 

@@ -34,6 +34,8 @@ EXPORTS = (
     "mi355_per_token_quant_fp8",
     "mi355_per_tensor_quant_fp8",
     "mi355_silu_mul_group_quant_fp8",
+    "mi355_block_cast_to_fp8",
+    "mi355_block_dequant_fp8",
     "mi355_fp8_scaled_mm_workspace_bytes",
     "mi355_fp8_scaled_mm",
     "mi355_fp8_block_linear_workspace_bytes",
@@ -96,6 +98,10 @@ def lib() -> ctypes.CDLL:
     L.mi355_per_tensor_quant_fp8.restype = i32
     L.mi355_silu_mul_group_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp, i64, i64, vp]
     L.mi355_silu_mul_group_quant_fp8.restype = i32
+    L.mi355_block_cast_to_fp8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
+    L.mi355_block_cast_to_fp8.restype = i32
+    L.mi355_block_dequant_fp8.argtypes = [vp, vp, vp, i32, i64, i64, vp]
+    L.mi355_block_dequant_fp8.restype = i32
     L.mi355_fp8_scaled_mm_workspace_bytes.argtypes = [i64, i64, i64]
     L.mi355_fp8_scaled_mm_workspace_bytes.restype = sz
     L.mi355_fp8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32] + [i64] * 6 + [vp, sz, vp]

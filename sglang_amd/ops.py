@@ -235,6 +235,32 @@ def sgl_per_token_quant_fp8(input, output_q, output_s):
                                               M, K, _stream()))
 
 
+def block_cast_to_fp8(x: torch.Tensor):
+    """x [m, n] -> (e4m3fn [m, n], fp32 power-of-two scales [ceil(m/128), ceil(n/128)]): per_block_cast_to_fp8 of
+    python/sglang/srt/layers/quantization/fp8_utils.py:487-500 as one kernel."""
+    _require(x.is_cuda and x.dim() == 2, "block_cast_to_fp8: a 2-D CUDA tensor is expected")
+    _require(x.dtype in (torch.float32, torch.float16, torch.bfloat16), "block_cast_to_fp8: unsupported dtype")
+    x = x.contiguous()
+    m, n = x.shape
+    q = torch.empty((m, n), dtype=torch.float8_e4m3fn, device=x.device)
+    s = torch.empty(((m + 127) // 128, (n + 127) // 128), dtype=torch.float32, device=x.device)
+    check(lib().mi355_block_cast_to_fp8(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), m, n, _stream()))
+    return q, s
+
+
+def block_dequant_fp8(q: torch.Tensor, s: torch.Tensor, dtype: torch.dtype):
+    """q [n, k] e4m3fn, s [ceil(n/128), ceil(k/128)] -> [n, k] of `dtype`: block_quant_dequant (fp8_utils.py:392-413)."""
+    _require(q.is_cuda and q.dim() == 2 and q.dtype == torch.float8_e4m3fn, "block_dequant_fp8: a 2-D e4m3fn CUDA tensor is expected")
+    n, k = q.shape
+    _require(tuple(s.shape) == ((n + 127) // 128, (k + 127) // 128), "block_dequant_fp8: scale shape mismatch")
+    _require(dtype in (torch.float32, torch.float16, torch.bfloat16), "block_dequant_fp8: unsupported dtype")
+    q = q.contiguous()
+    s = s.to(torch.float32).contiguous()
+    out = torch.empty((n, k), dtype=dtype, device=q.device)
+    check(lib().mi355_block_dequant_fp8(q.data_ptr(), s.data_ptr(), out.data_ptr(), _DT[dtype], n, k, _stream()))
+    return out
+
+
 def sgl_per_tensor_quant_fp8(input, output_q, output_s, is_static):
     """sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:102-130.  Dynamic mode merges block maxima into `output_s` with an
     atomic max, so the caller passes zeros (the reference's scaled_fp8_quant does)."""

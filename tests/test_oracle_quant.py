@@ -351,3 +351,48 @@ def test_silu_mul_against_torch(oracle, dtype):
     # discriminating alternatives must be far away
     alt = (torch.nn.functional.silu(gate.float()) * up.float()).to(dtype)  # product before the first rounding
     assert float((alt.view(torch.int16) != got.view(torch.int16)).float().mean()) > 0.05
+
+
+# ---------------------------------------------------------------- weight side: 128 x 128 block cast / dequant
+
+def _ref_per_block_cast_to_fp8(x):
+    """per_block_cast_to_fp8 + ceil_to_ue8m0 of python/sglang/srt/layers/quantization/fp8_utils.py:487-505, in the same
+    torch operations (CPU)."""
+    m, n = x.shape
+    pm, pn = (m + 127) // 128 * 128, (n + 127) // 128 * 128
+    x_padded = torch.zeros((pm, pn), dtype=x.dtype)
+    x_padded[:m, :n] = x
+    x_view = x_padded.view(-1, 128, pn // 128, 128)
+    x_amax = x_view.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    sf = torch.pow(2.0, torch.ceil(torch.log2((x_amax / 448.0).abs())))
+    x_scaled = (x_view * (1.0 / sf)).to(torch.float8_e4m3fn)
+    return x_scaled.view_as(x_padded)[:m, :n].contiguous(), sf.view(x_view.size(0), x_view.size(2))
+
+
+@pytest.mark.parametrize("shape", [(256, 384), (130, 200), (128, 128), (5, 7), (384, 1000)])
+def test_block_cast_to_fp8_against_torch(oracle, shape):
+    g = torch.Generator().manual_seed(shape[0] * 7 + shape[1])
+    x = (torch.randn(*shape, generator=g) * torch.rand(*shape, generator=g).pow(4) * 3).to(torch.bfloat16)
+    x[0, 0] = 448.0 * 0.25  # amax / 448 exactly a power of two in the first block: ceil must not step up
+    q, s = oracle.block_cast_to_fp8(x)
+    q_ref, s_ref = _ref_per_block_cast_to_fp8(x)
+    assert torch.equal(s, s_ref)
+    assert torch.equal(q.view(torch.uint8), q_ref.view(torch.uint8))
+    assert float(s[0, 0]) == 0.25 or shape == (5, 7) and float(s[0, 0]) == 0.25
+    assert bool(((q.view(torch.uint8) & 0x7F) <= 0x7E).all())  # never NaN: |x / s| <= 448
+    z, sz = oracle.block_cast_to_fp8(torch.zeros(130, 130, dtype=torch.bfloat16))
+    assert not bool(z.view(torch.uint8).any()) and bool((sz == 2.0 ** -22).all())  # floor 1e-4 / 448 rounds up to 2^-22
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_block_dequant_against_torch(oracle, dtype):
+    g = torch.Generator().manual_seed(31)
+    n, k = 200, 300
+    codes = torch.randint(0, 256, (n, k), generator=g, dtype=torch.uint8)
+    codes = torch.where((codes & 0x7F) == 0x7F, codes & 0xF7, codes)
+    q = codes.view(torch.float8_e4m3fn)
+    s = torch.rand(2, 3, generator=g) * 0.01 + 1e-4
+    out = oracle.block_dequant_fp8(q, s, dtype)
+    ref = (q.to(torch.float32) * s.repeat_interleave(128, 0).repeat_interleave(128, 1)[:n, :k]).to(dtype)
+    assert torch.equal(out.view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       ref.view(torch.int16 if dtype != torch.float32 else torch.int32))
