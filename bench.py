@@ -15,6 +15,7 @@ Infinity Cache.
   fp8_gemm     the headline alone          quant / quant_ue8m0   one quantizer variant alone
   fp8_decode   FP8 gate_up at M=1          int8_gemm             INT8 gate_up (K=4096 -> N=28672) at M=4096
   fp8:M:K:N    any blockwise-FP8 linear    int8:M:K:N            any INT8 linear
+  fp8_ue8m0:M:K:N  the same linear with power-of-two (UE8M0) scales on both operands
   copy         a plain 256 MiB device copy (calibration of the HBM traffic counters)
   silu_quant   silu(gate) * up fused in front of the group quantizer (packed UE8M0 scales)
 
@@ -297,6 +298,57 @@ def bench_fp8_gemm(name, M, K, N, steps, warmup, with_cpu, w8a16_cpu=False):
 
 # ------------------------------------------------------------------------------------------ INT8 GEMM
 
+def bench_fp8_ue8m0_gemm(name, M, K, N, steps, warmup):
+    """Blockwise-FP8 linear with power-of-two (UE8M0) scales on both operands: the weight re-quantized by
+    requant_weight_ue8m0, the activation quantized with packed exponents; N and K multiples of 128."""
+    import torch
+
+    from sglang_amd import _lib, fp8_kernel, fp8_utils, ops
+    from sglang_amd.workloads import fp8_gemm_algorithmic_bytes, gemm_flops, make_activation
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(N * 10007 + K)
+    nbuf = max(2, min(6, int(600e6 // (N * K)) + 1))
+    ws, wss = [], []
+    for _ in range(nbuf):
+        w_q, w_s = device_block_fp8_weight(N, K, gen, dev)
+        w2, sw = fp8_utils.requant_weight_ue8m0(w_q, w_s, [128, 128])
+        ws.append(w2)
+        wss.append(sw)
+    x = make_activation(M, K).to(dev)
+    x_q, x_s = fp8_kernel.sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True,
+                                                           scale_ue8m0=True, enable_v2=True)
+
+    def step(i):
+        return ops.fp8_blockwise_mm_ue8m0(x_q, ws[i], x_s, wss[i], torch.bfloat16)
+
+    if M <= 256 or N * K <= 16e6:
+        L = _lib.lib()
+        wsb = L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(M, N, K)
+        wsbuf = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+        outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+        stream = torch.cuda.current_stream().cuda_stream
+        args = [(x_q.data_ptr(), ws[i].data_ptr(), x_s.data_ptr(), wss[i].data_ptr(), None, outs[i].data_ptr(), _lib.BF16, M, N, K,
+                 x_q.stride(0), ws[i].stride(0), x_s.stride(1), wss[i].stride(0), wss[i].stride(1), outs[i].stride(0),
+                 wsbuf.data_ptr(), wsb, stream) for i in range(nbuf)]
+
+        def step(i):  # noqa: F811
+            _lib.check(L.mi355_fp8_blockwise_mm_ue8m0(*args[i]))
+
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms, b2b)
+    flops, nbytes = gemm_flops(M, N, K), fp8_gemm_algorithmic_bytes(M, N, K)
+    plan = _lib.gemm_plan("fp8", M, N, K)
+    kern = "pingpong (MFMA-applied scales)" if plan["kernel"] == "pingpong" else plan["kernel"] + " after unpack"
+    return {
+        "workload": f"fp8_gemm_ue8m0 {name} M={M} K={K} N={N} (e4m3fn x e4m3fn, packed UE8M0 scales on both sides, bf16 out)",
+        "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "fp8(e4m3fn) MFMA with block scales, f32 accumulate", "kernel": kern,
+        "roofline": _roofline(flops, nbytes, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
+    }
+
+
 def bench_int8_gemm(name, M, K, N, steps, warmup, with_cpu=False):
     import torch
 
@@ -500,6 +552,9 @@ def main():
     elif wl == "int8_gemm":
         K, N = LLAMA3_8B["gate_up"]
         rec = bench_int8_gemm("gate_up", 4096, K, N, S, W, cpu)
+    elif wl.startswith("fp8_ue8m0:"):
+        _, M, K, N = wl.split(":")
+        rec = bench_fp8_ue8m0_gemm("shape", int(M), int(K), int(N), S, W)
     elif wl.startswith("fp8:") or wl.startswith("int8:"):
         kind, M, K, N = wl.split(":")
         fn = bench_fp8_gemm if kind == "fp8" else bench_int8_gemm
@@ -513,6 +568,7 @@ def main():
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 4096, K, N, S, W, cpu)
         if full:
+            also.append(bench_fp8_ue8m0_gemm("gate_up", 4096, K, N, S, W))
             also.append(bench_silu_quant(S, W))
             K, N = DSV3_MLP["down"]
             also.append(bench_fp8_gemm("down", 4096, K, N, S, W, False))

@@ -109,6 +109,28 @@ int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const 
                            void* stream);
 
 /*
+ * Blockwise FP8 GEMM with power-of-two (UE8M0) scales on BOTH operands, the form DeepSeek-V3 checkpoints take after
+ * requant_weight_ue8m0 and activations take from per_token_group_quant_fp8(scale_ue8m0=True):
+ *   out[m,n] = cast( sum_kb 2^(ea[m,kb] - 127) * 2^(eb[n,kb] - 127) * sum_{k in block kb} a[m,k] * b[n,k]  (+ bias[n]) )
+ *   sa_words  int32, four exponent bytes per word (byte kb & 3 of word kb >> 2): word (m, kw) at sa_words[kw * sa_sk + m]
+ *             (token index fastest: the packed column-major layout of create_per_token_group_quant_fp8_output_scale)
+ *   sb_words  int32, same packing per weight ROW: word (n, kw) at sb_words[n * sb_sn + kw * sb_sk]; the rows of one
+ *             128-channel block carry the same bytes (what the 128 x 128 block requantization produces), and the block's
+ *             first row is the one that is read
+ *   bias      NULL or [N] in the output dtype, added in the epilogue
+ * On gfx950 the matrix instruction applies such scales itself (v_mfma_scale_f32_16x16x128_f8f6f4), so for large M the
+ * K loop carries no scale arithmetic at all; other shapes expand the exponents to fp32 scales in the workspace and take
+ * the kernels of mi355_fp8_blockwise_mm.  Replaces w8a8_block_fp8_matmul_deepgemm / deep_gemm gemm_nt_f8f8bf16
+ * (python/sglang/srt/layers/quantization/fp8_kernel.py:1047-1065; caller deepgemm_w8a8_block_fp8_linear_with_fallback,
+ * fp8_utils.py:217-255), whose kernel lives in the DeepGEMM package, not in the reference tree.
+ */
+size_t mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_fp8_blockwise_mm_ue8m0(const void* a, const void* b, const void* sa_words, const void* sb_words, const void* bias,
+                                 void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                 int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
+/*
  * mi355_fp8_blockwise_mm for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose operators allocate
  * their workspaces through the framework.  Same arguments and results as mi355_fp8_blockwise_mm without the workspace:

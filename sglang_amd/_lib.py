@@ -26,6 +26,8 @@ EXPORTS = (
     "mi355_fp8_blockwise_mm_workspace_bytes",
     "mi355_fp8_blockwise_mm",
     "mi355_fp8_blockwise_mm_noalloc",
+    "mi355_fp8_blockwise_mm_ue8m0_workspace_bytes",
+    "mi355_fp8_blockwise_mm_ue8m0",
     "mi355_int8_scaled_mm_workspace_bytes",
     "mi355_int8_scaled_mm",
     "mi355_fp8_blockwise_mm_plan",
@@ -81,6 +83,10 @@ def lib() -> ctypes.CDLL:
     L.mi355_fp8_blockwise_mm_workspace_bytes.restype = sz
     L.mi355_fp8_blockwise_mm.argtypes = [vp, vp, vp, vp, vp, i32] + [i64] * 10 + [vp, sz, vp]
     L.mi355_fp8_blockwise_mm.restype = i32
+    L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes.argtypes = [i64, i64, i64]
+    L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes.restype = sz
+    L.mi355_fp8_blockwise_mm_ue8m0.argtypes = [vp, vp, vp, vp, vp, vp, i32] + [i64] * 9 + [vp, sz, vp]
+    L.mi355_fp8_blockwise_mm_ue8m0.restype = i32
     L.mi355_fp8_blockwise_mm_noalloc.argtypes = [vp, vp, vp, vp, vp, i32] + [i64] * 10 + [vp]
     L.mi355_fp8_blockwise_mm_noalloc.restype = i32
     L.mi355_int8_scaled_mm_workspace_bytes.argtypes = [i64, i64, i64]

@@ -153,6 +153,9 @@ int launch_fp8_pipelined(GemmParams& p, hipStream_t stream, const char* what);
 // Large-M blockwise FP8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases);
 // gemm_fp8_pp.hip.  Same requirements.
 int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what);
+// The same kernel for packed power-of-two (UE8M0) scales on both operands, applied by the MFMA itself: p.sa / p.sb point
+// to 32-bit words of four exponent bytes (see fp8_gemm_pp_kernel).  K % 128 == 0.
+int launch_fp8_pp_ue8m0(GemmParams& p, hipStream_t stream, const char* what);
 // Token scales must be M-major with a pitch that is a multiple of four floats and a 16-byte aligned base.
 
 

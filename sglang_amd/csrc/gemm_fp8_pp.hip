@@ -105,8 +105,12 @@ __device__ __forceinline__ void issue_one(const PpState& s, int i, uint8_t* stag
 
 // The wave's 32 token scales of block b (tokens 32 * wave .. + 31 of the tile) into scale stage b % 4: lanes 0..7 fetch
 // 16 bytes each.  exec is narrowed and restored inside the statement.
+template <bool UE8M0>
 __device__ __forceinline__ void issue_scales(const PpState& s, int b) {
-  const float* base = s.sa_base + (int64_t)min(b, s.kb_last) * s.sa_sk;  // wave-uniform
+  // fp32 scales: one row of floats per K block; packed exponents: one row of 32-bit words per four K blocks (fetched
+  // again for each of the four, which keeps the load count per K block constant)
+  const int srow = UE8M0 ? (min(b, s.kb_last) >> 2) : min(b, s.kb_last);
+  const float* base = s.sa_base + (int64_t)srow * s.sa_sk;  // wave-uniform
   asm volatile("" : "+s"(base));
   const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(g_scale + (b & 3) * G_BM + s.wave * 32);
   uint64_t saved;
@@ -119,9 +123,9 @@ __device__ __forceinline__ void issue_scales(const PpState& s, int b) {
 
 // Set A of block b: scales, channel bands, token rows 0..63 and 128..191 (7 loads).  Set B: token rows 64..127, 192..255.
 constexpr int SET_A = 7, SET_B = 2;
-template <bool KFULL>
+template <bool KFULL, bool UE8M0>
 __device__ __forceinline__ void issue_set_a(const PpState& s, uint8_t* stage, int b) {
-  issue_scales(s, b);
+  issue_scales<UE8M0>(s, b);
 #pragma unroll
   for (int i = 4; i < 8; ++i) issue_one<KFULL>(s, i, stage, b);
   issue_one<KFULL>(s, 0, stage, b);
@@ -153,8 +157,9 @@ __device__ __forceinline__ void memory_end() {
 
 // Memory phase, operand part: token tiles 4 * HALF .. + 3 of `cur` (and, for HALF == 0, the four weight fragments)
 // into registers; their scales times the weight-block scale.
-template <int HALF>
-__device__ __forceinline__ void read_operands(const PpState& s, const uint8_t* cur, const float* sc_cur, float sbv,
+// UE8M0: scb[jj] carries (as bits) the token's packed exponent word shifted so that the byte of this K block is byte 0.
+template <int HALF, bool UE8M0>
+__device__ __forceinline__ void read_operands(const PpState& s, const uint8_t* cur, const float* sc_cur, float sbv, int kb,
                                               Frag (&w)[G_NT], Frag (&tok)[G_HT], float (&scb)[G_HT]) {
   const lds_cptr ch0 = (lds_cptr)cur + s.ch_off[0], ch1 = (lds_cptr)cur + s.ch_off[1];
   const lds_cptr tk0 = (lds_cptr)cur + s.tok_off[0], tk1 = (lds_cptr)cur + s.tok_off[1];
@@ -172,7 +177,12 @@ __device__ __forceinline__ void read_operands(const PpState& s, const uint8_t* c
     tok[jj].hi = lds16(tk1, (HALF * G_HT + jj) * 2048);
   }
 #pragma unroll
-  for (int jj = 0; jj < G_HT; ++jj) scb[jj] = scp[(HALF * G_HT + jj) * 16] * sbv;
+  for (int jj = 0; jj < G_HT; ++jj) {
+    if constexpr (UE8M0)
+      scb[jj] = __uint_as_float(__float_as_uint(scp[(HALF * G_HT + jj) * 16]) >> ((kb & 3) * 8));
+    else
+      scb[jj] = scp[(HALF * G_HT + jj) * 16] * sbv;
+  }
 }
 
 // The promotion of the last MFMA of a compute phase is left to the start of the wave's next memory phase (the other
@@ -216,7 +226,27 @@ __device__ __forceinline__ void compute(const Frag (&w)[G_NT], const Frag (&tok)
   pd.scale = scb[G_HT - 1];
 }
 
-template <bool KFULL>
+// Compute phase with power-of-two scales on both sides: the MFMA applies them itself (scale operands: byte 0 of each
+// lane's register; lane l supplies the scale of operand row l % 16 for K sub-block l / 16 - here one value per row), so
+// the products go straight into the accumulators and no vector arithmetic is left in the phase.
+template <int HALF>
+__device__ __forceinline__ void compute_ue8m0(const Frag (&w)[G_NT], const Frag (&tok)[G_HT], const float (&scb)[G_HT],
+                                              int w_scale, float (&acc)[G_NT][G_MT][4]) {
+#pragma unroll
+  for (int jj = 0; jj < G_HT; ++jj)
+#pragma unroll
+    for (int i = 0; i < G_NT; ++i) {
+      float* a = acc[i][HALF * G_HT + jj];
+      const v4f r = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w[i]), as_v8i(tok[jj]), v4f{a[0], a[1], a[2], a[3]}, 0,
+                                                                     0, 0, w_scale, 0, (int)__float_as_uint(scb[jj]));
+      a[0] = r[0], a[1] = r[1], a[2] = r[2], a[3] = r[3];
+    }
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// UE8M0: p.sa / p.sb point to packed exponent words (int32): token word (m, kw) at sa[kw * sa_sk + m], channel word
+// (n, kw) at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb.
+template <bool KFULL, bool UE8M0>
 __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -259,7 +289,9 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
   s.sa_base = p.sa;
   s.sa_off = (uint32_t)min(m0 + wave * 32 + (lane & 7) * 4, (p.M - 1) & ~3) * 4u;  // quads past M refetch the last one
   s.sa_sk = p.sa_sk;
-  s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * G_WN, p.N - 1) / 128) * p.sb_sn);
+  s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(UE8M0 ? min(n0 + wave_n * G_WN, p.N - 1)
+                                                                                  : min(n0 + wave_n * G_WN, p.N - 1) / 128) *
+                                     p.sb_sn);
   s.sb_sk = p.sb_sk;
 
   float acc[G_NT][G_MT][4];
@@ -277,9 +309,9 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
   pd.scale = 0.f;
 
   // ---- prologue: all of block 0 and set A of block 1
-  issue_set_a<KFULL>(s, g_stage0, 0);
+  issue_set_a<KFULL, UE8M0>(s, g_stage0, 0);
   issue_set_b<KFULL>(s, g_stage0, 0);
-  issue_set_a<KFULL>(s, g_stage1, 1);
+  issue_set_a<KFULL, UE8M0>(s, g_stage1, 1);
   float sb_cur = s.sb_ptr[0];
   asm volatile("s_waitcnt vmcnt(7)\n\ts_barrier" ::: "memory");  // block 0 is in LDS (set A of block 1 may be in flight)
   if (grp == 1) compute_end();  // group 1 runs one phase behind group 0
@@ -287,30 +319,34 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
   // One K block: M0, C0, M1, C1.  `cur` holds block kb; `nxt` takes set B of block kb + 1, `cur` set A of block kb + 2.
   auto k_block = [&](uint8_t* cur, uint8_t* nxt, int kb, float sbv) {
     const float* sc_cur = g_scale + (kb & 3) * G_BM;
-    retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
-    read_operands<0>(s, cur, sc_cur, sbv, w, tok, scb);
+    // the weight block's exponent byte, in byte 0 of a register (sbv then carries the packed word as bits)
+    const int w_scale = UE8M0 ? (int)(__float_as_uint(sbv) >> ((kb & 3) * 8)) : 0;
+    if constexpr (!UE8M0) retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
+    read_operands<0, UE8M0>(s, cur, sc_cur, sbv, kb, w, tok, scb);
     issue_set_b<KFULL>(s, nxt, kb + 1);
     memory_end();
-    compute<0>(w, tok, scb, acc, pd);
+    if constexpr (UE8M0) compute_ue8m0<0>(w, tok, scb, w_scale, acc);
+    else compute<0>(w, tok, scb, acc, pd);
     compute_end();
-    retire<0>(pd, acc);
-    read_operands<1>(s, cur, sc_cur, sbv, w, tok, scb);
-    issue_set_a<KFULL>(s, cur, kb + 2);
+    if constexpr (!UE8M0) retire<0>(pd, acc);
+    read_operands<1, UE8M0>(s, cur, sc_cur, sbv, kb, w, tok, scb);
+    issue_set_a<KFULL, UE8M0>(s, cur, kb + 2);
     memory_end();
-    compute<1>(w, tok, scb, acc, pd);
+    if constexpr (UE8M0) compute_ue8m0<1>(w, tok, scb, w_scale, acc);
+    else compute<1>(w, tok, scb, acc, pd);
     compute_end();
   };
 
   int kb = 0;
   for (; kb + 1 < nkb; kb += 2) {
-    const float sb_1 = s.sb_ptr[(int64_t)(kb + 1) * s.sb_sk];
-    const float sb_2 = s.sb_ptr[(int64_t)min(kb + 2, nkb - 1) * s.sb_sk];
+    const float sb_1 = s.sb_ptr[(int64_t)(UE8M0 ? (kb + 1) >> 2 : kb + 1) * s.sb_sk];
+    const float sb_2 = s.sb_ptr[(int64_t)(UE8M0 ? min(kb + 2, nkb - 1) >> 2 : min(kb + 2, nkb - 1)) * s.sb_sk];
     k_block(g_stage0, g_stage1, kb, sb_cur);
     k_block(g_stage1, g_stage0, kb + 1, sb_1);
     sb_cur = sb_2;
   }
   if (kb < nkb) k_block(g_stage0, g_stage1, kb, sb_cur);
-  retire<1>(pd, acc);
+  if constexpr (!UE8M0) retire<1>(pd, acc);
   if (grp == 0) compute_end();  // as many barriers as group 1
   // the last requests refetch the last block into rows nobody reads any more: they must not outlive the workgroup's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -354,9 +390,19 @@ int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_n = (p.N + G_BN - 1) / G_BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
   if (p.K % KSTEP == 0)
-    hipLaunchKernelGGL(fp8_gemm_pp_kernel<true>, grid, dim3(G_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, false>), grid, dim3(G_THREADS), 0, stream, p);
   else
-    hipLaunchKernelGGL(fp8_gemm_pp_kernel<false>, grid, dim3(G_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_pp_kernel<false, false>), grid, dim3(G_THREADS), 0, stream, p);
+  return check_launch(what);
+}
+
+// The same kernel with packed power-of-two scales on both operands (see fp8_gemm_pp_kernel).  Needs K % 128 == 0, token
+// words M-major with a pitch that is a multiple of four words and a 16-byte aligned base.
+int launch_fp8_pp_ue8m0(GemmParams& p, hipStream_t stream, const char* what) {
+  p.tiles_m = (p.M + G_BM - 1) / G_BM;
+  p.tiles_n = (p.N + G_BN - 1) / G_BN;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, true>), grid, dim3(G_THREADS), 0, stream, p);
   return check_launch(what);
 }
 

@@ -667,6 +667,82 @@ extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float*
   return run_gemm<true>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
 }
 
+namespace {
+
+// out[r * o_row + kb * o_kb] = 2^(byte - 127), byte = byte kb & 3 of word words[(kb >> 2) * w_kw + r * row_step * w_row]:
+// packed exponents as fp32 scales, for the kernels that take those.  Byte 0 is 2^-127 (a subnormal float), byte 255 NaN.
+__global__ __launch_bounds__(256) void unpack_ue8m0_kernel(const uint32_t* words, int64_t w_row, int64_t w_kw, int row_step,
+                                                           float* out, int64_t o_row, int64_t o_kb, int rows, int KB) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)rows * KB) return;
+  // consecutive threads walk rows: token words are contiguous over rows, and so is the M-major output
+  const int kb = (int)(idx / rows), r = (int)(idx - (int64_t)kb * rows);
+  const uint32_t w = words[(int64_t)(kb >> 2) * w_kw + (int64_t)r * row_step * w_row];
+  const uint32_t byte = (w >> ((kb & 3) * 8)) & 0xffu;
+  const uint32_t bits = byte == 0 ? 0x00400000u : (byte == 255 ? 0x7fc00000u : byte << 23);
+  out[(int64_t)r * o_row + (int64_t)kb * o_kb] = __uint_as_float(bits);
+}
+
+size_t ue8m0_unpacked_bytes(int64_t M, int64_t N, int64_t K) {
+  const int64_t kb = (K + KSTEP - 1) / KSTEP;
+  const size_t b = ((size_t)((M + 3) & ~3ll) * (size_t)kb + (size_t)((N + 127) / 128) * (size_t)kb) * 4u;
+  return (b + 255) & ~(size_t)255;
+}
+
+}  // namespace
+
+extern "C" size_t mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  return ue8m0_unpacked_bytes(M, N, K) + workspace_bytes(M, N, K, true);
+}
+
+extern "C" int mi355_fp8_blockwise_mm_ue8m0(const void* a, const void* b, const void* sa_words, const void* sb_words,
+                                            const void* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                            int64_t ldb, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo,
+                                            void* workspace, size_t workspace_bytes_given, void* stream) {
+  const char* what = "mi355_fp8_blockwise_mm_ue8m0";
+  GemmParams p;
+  bool empty;
+  // strides of the packed words stand in for the fp32 scale strides of the shared argument check
+  int rc = fp8_mm_params(what, a, b, static_cast<const float*>(sa_words), static_cast<const float*>(sb_words), out, out_dtype, M,
+                         N, K, lda, ldb, 1, sa_sk, sb_sn, sb_sk, ldo, p, empty);
+  if (rc != MI355_OK || empty) return rc;
+  MI355_REQUIRE(((reinterpret_cast<uintptr_t>(sa_words) | reinterpret_cast<uintptr_t>(sb_words)) & 3) == 0,
+                MI355_ERR_INVALID_ARGUMENT, "%s: scale words must be 4-byte aligned", what);
+  MI355_REQUIRE(bias == nullptr || out_dtype != MI355_F32, MI355_ERR_INVALID_ARGUMENT,
+                "%s: a bias needs a 16-bit output type (it has the output's type)", what);
+  p.bias = bias;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  p.kb_total = (p.K + KSTEP - 1) / KSTEP;
+  const Route r = choose_route(true, p.M, p.N, p.K, p.lda, p.ldb, operands_aligned(p));
+  const bool words_conform = (sa_sk & 3) == 0 && sa_sk >= ((M + 3) & ~3ll) && (reinterpret_cast<uintptr_t>(sa_words) & 15) == 0;
+  if (r.kernel == RK_PINGPONG && K % KSTEP == 0 && words_conform) {
+    // the MFMA applies both exponents itself: no scale arithmetic at all
+    p.splits = 1, p.kb_per_split = p.kb_total;
+    return launch_fp8_pp_ue8m0(p, st, what);
+  }
+  // every other shape: exponents to fp32 scales in the head of the workspace (tokens M-major, weights one row per
+  // 128-channel block, read from the block's first channel), then the fp32-scale kernels
+  const size_t head = ue8m0_unpacked_bytes(M, N, K);
+  MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= head, MI355_ERR_WORKSPACE,
+                "%s: needs a workspace of at least %zu bytes, got %zu", what, head, workspace_bytes_given);
+  MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 15) == 0, MI355_ERR_WORKSPACE, "%s: workspace must be 16-byte aligned", what);
+  const int KB = p.kb_total;
+  const int64_t ldm = (M + 3) & ~3ll;
+  const int NB = (int)((N + 127) / 128);
+  float* sa_f = static_cast<float*>(workspace);
+  float* sb_f = sa_f + ldm * KB;
+  hipLaunchKernelGGL(unpack_ue8m0_kernel, dim3((unsigned)(((int64_t)M * KB + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint32_t*>(sa_words), (int64_t)1, sa_sk, 1, sa_f, (int64_t)1, ldm, (int)M, KB);
+  hipLaunchKernelGGL(unpack_ue8m0_kernel, dim3((unsigned)(((int64_t)NB * KB + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint32_t*>(sb_words), sb_sn, sb_sk, 128, sb_f, (int64_t)KB, (int64_t)1, NB, KB);
+  rc = check_launch(what);
+  if (rc != MI355_OK) return rc;
+  p.sa = sa_f, p.sa_sm = 1, p.sa_sk = ldm;
+  p.sb = sb_f, p.sb_sn = KB, p.sb_sk = 1;
+  return run_gemm<true>(p, static_cast<uint8_t*>(workspace) + head, workspace_bytes_given - head, st, what);
+}
+
 extern "C" int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, const float* sa, const float* sb, void* out,
                                               int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                                               int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo,

@@ -215,6 +215,20 @@ def sglang_per_token_group_quant_fp8(
     return x_q, x_s
 
 
+def w8a8_block_fp8_matmul_deepgemm(A: torch.Tensor, B: torch.Tensor, As: torch.Tensor, Bs: torch.Tensor,
+                                   block_size: List[int], output_dtype: torch.dtype) -> torch.Tensor:
+    """fp8_kernel.py:1047-1065: C = A @ B^T with packed UE8M0 scales on both operands (DeepGEMM's gemm_nt_f8f8bf16 in
+    the reference): ``As`` int32 [..., M, ceil(K/512)] packed along tokens, ``Bs`` int32 [N, ceil(K/512)] packed along
+    weight rows (fp8_utils.transform_scale_ue8m0)."""
+    assert list(block_size) == [128, 128]
+    assert output_dtype == torch.bfloat16, "Deepgemm only supports output tensor type as bfloat16"
+    K = A.shape[-1]
+    a2 = A.reshape(-1, K)
+    as2 = As.reshape(-1, As.shape[-1]) if As.dim() > 2 else As
+    C = ops.fp8_blockwise_mm_ue8m0(a2, B, as2, Bs, output_dtype)
+    return C.view(*A.shape[:-1], B.shape[0])
+
+
 def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
     """fp8_kernel.py:573-589: one scale per row, ``(x_q, x_s [M, 1])``."""
     assert x.is_contiguous(), "`x` is not contiguous"

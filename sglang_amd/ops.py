@@ -356,6 +356,41 @@ def block_fp8_linear(x2d: torch.Tensor, weight: torch.Tensor, weight_scale: torc
     return out
 
 
+def fp8_blockwise_mm_ue8m0(a: torch.Tensor, b: torch.Tensor, a_words: torch.Tensor, b_words: torch.Tensor,
+                           out_dtype: torch.dtype, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Blockwise FP8 GEMM with packed power-of-two scales on both sides: a [M, K] e4m3fn, b [N, K] e4m3fn (the weight as
+    stored), a_words int32 [M, ceil(K/512)] and b_words int32 [N, ceil(K/512)], both with stride 1 along their first
+    dimension (the layouts of create_per_token_group_quant_fp8_output_scale(scale_ue8m0=True) and
+    fp8_utils.transform_scale_ue8m0).  What deep_gemm's gemm_nt_f8f8bf16 computes for the reference
+    (python/sglang/srt/layers/quantization/fp8_kernel.py:1047-1065)."""
+    _require(a.is_cuda and b.is_cuda, "fp8_blockwise_mm_ue8m0: operands must be CUDA tensors")
+    _require(a.dim() == 2 and b.dim() == 2 and a.stride(1) == 1 and b.stride(1) == 1, "fp8_blockwise_mm_ue8m0: row-major operands expected")
+    _require(a.dtype == torch.float8_e4m3fn and b.dtype == torch.float8_e4m3fn, "fp8_blockwise_mm_ue8m0: operands must be Float8_e4m3fn")
+    M, K = a.shape
+    N = b.size(0)
+    _require(b.size(1) == K, "fp8_blockwise_mm_ue8m0: shapes cannot be multiplied")
+    kw = (((K + 127) // 128) + 3) // 4
+    for t, rows, name in ((a_words, M, "a_words"), (b_words, N, "b_words")):
+        _require(t.dtype == torch.int32 and t.dim() == 2 and t.size(0) == rows and t.size(1) >= kw,
+                 f"fp8_blockwise_mm_ue8m0: {name} must be int32 [{rows}, >= {kw}]")
+    _require(M <= 1 or a_words.stride(0) == 1, "fp8_blockwise_mm_ue8m0: a_words must be packed along tokens (stride(0) == 1)")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "fp8_blockwise_mm_ue8m0: out_dtype must be Half or BFloat16")
+    if bias is not None:
+        _require(bias.numel() == N and bias.is_contiguous() and bias.dtype == out_dtype,
+                 "fp8_blockwise_mm_ue8m0: bias must be a contiguous [N] tensor of the output dtype")
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    if M == 0 or N == 0:
+        return out
+    L = lib()
+    ws_bytes = L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(M, N, K)
+    ws = _workspace(ws_bytes, a.device)
+    check(L.mi355_fp8_blockwise_mm_ue8m0(
+        a.data_ptr(), b.data_ptr(), a_words.data_ptr(), b_words.data_ptr(), bias.data_ptr() if bias is not None else None,
+        out.data_ptr(), _DT[out_dtype], M, N, K, a.stride(0), b.stride(0), a_words.stride(1), b_words.stride(0), b_words.stride(1),
+        out.stride(0), ws.data_ptr() if ws is not None else None, ws_bytes, _stream()))
+    return out
+
+
 # ---------------------------------------------------------------- INT8 GEMM
 
 def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[torch.Tensor] = None):

@@ -1,0 +1,122 @@
+"""GPU parity of the blockwise FP8 GEMM with packed power-of-two (UE8M0) scales on both operands
+(mi355_fp8_blockwise_mm_ue8m0; the reference's w8a8_block_fp8_matmul_deepgemm / deepgemm_w8a8_block_fp8_linear_with_fallback,
+python/sglang/srt/layers/quantization/fp8_kernel.py:1047-1065, fp8_utils.py:217-255).
+
+The oracle is the blockwise GEMM oracle fed with the decoded scales 2^(byte - 127).  Floating point:
+|out - ref| <= 1e-2 * |ref| + 1e-4 * mag, as for the fp32-scale GEMM (tests/test_gpu_fp8_gemm.py); with small-integer
+operands every product and partial sum is exact in fp32 and the result must match bit for bit, whichever kernel runs.
+Large shapes take the kernel whose MFMA applies the scales itself, the others the fp32-scale kernels behind an unpack
+step; both are covered, and so are K extents whose last exponent word is only partly used."""
+import pytest
+import torch
+
+from sglang_amd.workloads import make_activation, make_fp8_weight
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+
+# (M, N, K): two-phase kernel with hardware scales (>= 256 tiles of 256 x 256): K of 4, 9 and 5 blocks; ragged M;
+# then decode, mid-M, generic routes through the unpack step
+SHAPES = [(4096, 4352, 512), (4096, 4352, 1152), (4000, 4352, 640), (4, 512, 1024), (16, 2048, 7168), (200, 16384, 2048),
+          (50, 384, 512), (1500, 640, 1024)]
+
+
+def _unpack_bytes(words, groups):
+    dense = torch.empty(tuple(words.shape), dtype=torch.int32)
+    dense.copy_(words.cpu())
+    return dense.view(torch.uint8).reshape(words.shape[0], -1)[:, :groups]
+
+
+def _operands(M, N, K, gpu, seed):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.fp8_utils import requant_weight_ue8m0
+
+    w_q, w_s = make_fp8_weight(N, K, seed=seed)
+    w2, sb_words = requant_weight_ue8m0(w_q.to(gpu), w_s.to(gpu), [128, 128])
+    x = make_activation(M, K, seed=seed + 1).to(gpu)
+    x_q, sa_words = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True,
+                                                     enable_v2=True)
+    return x_q, sa_words, w2, sb_words
+
+
+def _reference(oracle, x_q, sa_words, w2, sb_words, rows=None):
+    K = x_q.shape[1]
+    KB = K // 128
+    sa = torch.exp2(_unpack_bytes(sa_words, KB).float() - 127.0)
+    sb = torch.exp2(_unpack_bytes(sb_words, KB).float() - 127.0)[::128].contiguous()
+    a = x_q.cpu()
+    if rows is not None:
+        a, sa = a[rows].contiguous(), sa[rows].contiguous()
+    return oracle.fp8_blockwise_mm(a, w2.cpu(), sa.contiguous(), sb, torch.float32, want_abs=True)
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_ue8m0_gemm_against_oracle(gpu, oracle, M, N, K):
+    from sglang_amd import _lib
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul_deepgemm
+
+    print(f"case M={M} N={N} K={K} -> {_lib.gemm_plan('fp8', M, N, K)['kernel']}", flush=True)
+    x_q, sa_words, w2, sb_words = _operands(M, N, K, gpu, 3 * M + N + K)
+    out = w8a8_block_fp8_matmul_deepgemm(x_q, w2, sa_words, sb_words, [128, 128], torch.bfloat16)
+    assert tuple(out.shape) == (M, N) and out.dtype == torch.bfloat16
+    g = torch.Generator().manual_seed(M)
+    rows = torch.arange(M) if M <= 256 else torch.cat([torch.tensor([0, 127, 128, 255, 256, M - 1]), torch.randperm(M, generator=g)[:26]])
+    ref, mag = _reference(oracle, x_q, sa_words, w2, sb_words, rows)
+    err = (out[rows.to(gpu)].float().cpu() - ref).abs()
+    tol = 1e-2 * ref.abs() + 1e-4 * mag
+    assert bool((err <= tol).all()), float((err - tol).max())
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 4352, 1152), (16, 2048, 1024), (200, 16384, 640)])
+def test_ue8m0_gemm_exact_integers(gpu, oracle, M, N, K):
+    """Operands in {-2..2}, exponents in a narrow band: every block product and every partial sum is an integer times a
+    power of two well inside fp32, so any summation order gives the same bits."""
+    from sglang_amd import ops
+
+    g = torch.Generator().manual_seed(K + M)
+    a = torch.randint(-2, 3, (M, K), generator=g).float().to(FP8)
+    w = torch.randint(-2, 3, (N, K), generator=g).float().to(FP8)
+    KB, KW = K // 128, (K // 128 + 3) // 4
+    ea = torch.randint(120, 129, (M, KB), generator=g, dtype=torch.uint8)
+    eb = torch.randint(122, 131, ((N + 127) // 128, KB), generator=g, dtype=torch.uint8)
+
+    def pack(e, rows_out, repeat):  # [R, KB] bytes -> int32 [rows_out, KW] with stride(0) == 1
+        full = torch.zeros(e.shape[0], KW * 4, dtype=torch.uint8)
+        full[:, :KB] = e
+        words = full.view(torch.int32).repeat_interleave(repeat, 0)[:rows_out]           # [rows, KW]
+        pad = (rows_out + 3) // 4 * 4
+        buf = torch.zeros(KW, pad, dtype=torch.int32)
+        buf[:, :rows_out] = words.t()
+        return buf
+
+    sa_buf, sb_buf = pack(ea, M, 1).to(gpu), pack(eb, N, 128).to(gpu)
+    sa_words, sb_words = sa_buf.t()[:M], sb_buf.t()[:N]
+    out = ops.fp8_blockwise_mm_ue8m0(a.to(gpu), w.to(gpu), sa_words, sb_words, torch.bfloat16)
+    ref = oracle.fp8_blockwise_mm(a, w, torch.exp2(ea.float() - 127), torch.exp2(eb.float() - 127), torch.bfloat16)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("M", [8, 4096])
+def test_deepgemm_linear_wrapper(gpu, oracle, M):
+    from sglang_amd.fp8_utils import deepgemm_w8a8_block_fp8_linear_with_fallback, requant_weight_ue8m0
+
+    N, K = 4352, 512
+    w_q, w_s = make_fp8_weight(N, K, seed=9)
+    w2, sb_words = requant_weight_ue8m0(w_q.to(gpu), w_s.to(gpu), [128, 128])
+    x = make_activation(M, K, seed=10)
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    out = deepgemm_w8a8_block_fp8_linear_with_fallback(x.to(gpu).view(M // 4, 4, K), w2, [128, 128], sb_words, None, bias.to(gpu))
+    assert tuple(out.shape) == (M // 4, 4, N) and out.dtype == torch.bfloat16
+    v = x.clone()
+    q_o, s_o = oracle.group_quant(v, 128, mode="mul", layout="ue8m0")
+    sa = torch.exp2(oracle.unpack_ue8m0(s_o, K // 128).float() - 127.0)
+    sb = torch.exp2(_unpack_bytes(sb_words, K // 128).float() - 127.0)[::128].contiguous()
+    rows = torch.arange(M) if M <= 64 else torch.tensor([0, 1, 255, 256, 4095])
+    ref, mag = oracle.fp8_blockwise_mm(q_o[rows].contiguous(), w2.cpu(), sa[rows].contiguous(), sb, torch.float32, want_abs=True)
+    ref = ref + bias.float()[None, :]
+    err = (out.reshape(M, N)[rows.to(gpu)].float().cpu() - ref).abs()
+    tol = 1e-2 * ref.abs() + 1e-4 * mag + 2.0 ** -8 * ref.abs()
+    assert bool((err <= tol).all()), float((err - tol).max())
+    # an fp32 block scale tensor (a checkpoint that was not re-quantized) takes the ordinary block-FP8 linear
+    out2 = deepgemm_w8a8_block_fp8_linear_with_fallback(x.to(gpu), w_q.to(gpu), [128, 128], w_s.to(gpu), None, None)
+    assert tuple(out2.shape) == (M, N)
