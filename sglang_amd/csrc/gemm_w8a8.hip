@@ -669,18 +669,29 @@ extern "C" int mi355_fp8_blockwise_mm(const void* a, const void* b, const float*
 
 namespace {
 
-// out[r * o_row + kb * o_kb] = 2^(byte - 127), byte = byte kb & 3 of word words[(kb >> 2) * w_kw + r * row_step * w_row]:
-// packed exponents as fp32 scales, for the kernels that take those.  Byte 0 is 2^-127 (a subnormal float), byte 255 NaN.
-__global__ __launch_bounds__(256) void unpack_ue8m0_kernel(const uint32_t* words, int64_t w_row, int64_t w_kw, int row_step,
-                                                           float* out, int64_t o_row, int64_t o_kb, int rows, int KB) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (int64_t)rows * KB) return;
-  // consecutive threads walk rows: token words are contiguous over rows, and so is the M-major output
-  const int kb = (int)(idx / rows), r = (int)(idx - (int64_t)kb * rows);
-  const uint32_t w = words[(int64_t)(kb >> 2) * w_kw + (int64_t)r * row_step * w_row];
-  const uint32_t byte = (w >> ((kb & 3) * 8)) & 0xffu;
-  const uint32_t bits = byte == 0 ? 0x00400000u : (byte == 255 ? 0x7fc00000u : byte << 23);
-  out[(int64_t)r * o_row + (int64_t)kb * o_kb] = __uint_as_float(bits);
+// Packed exponents as fp32 scales 2^(byte - 127), for the kernels that take those; byte kb & 3 of word kb >> 2 belongs to
+// K block kb.  Byte 0 is 2^-127 (a subnormal float), byte 255 NaN.  One launch for both operands:
+//   tokens   sa_out[kb * ldm + m]  from sa_words[(kb >> 2) * sa_kw + m]                  (threads 0 .. M * KB - 1)
+//   weights  sb_out[nb * KB + kb]  from sb_words[(kb >> 2) * sb_kw + 128 * nb * sb_row]  (the block's first row; the rest)
+__device__ __forceinline__ float ue8m0_to_f32(uint32_t word, int kb) {
+  const uint32_t byte = (word >> ((kb & 3) * 8)) & 0xffu;
+  return __uint_as_float(byte == 0 ? 0x00400000u : (byte == 255 ? 0x7fc00000u : byte << 23));
+}
+__global__ __launch_bounds__(256) void unpack_ue8m0_kernel(const uint32_t* sa_words, int64_t sa_kw, float* sa_out, int64_t ldm,
+                                                           int M, const uint32_t* sb_words, int64_t sb_row, int64_t sb_kw,
+                                                           float* sb_out, int NB, int KB) {
+  int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t n_tok = (int64_t)M * KB;
+  if (idx < n_tok) {
+    // consecutive threads walk tokens: the words are contiguous over tokens, and so is the M-major output
+    const int kb = (int)(idx / M), m = (int)(idx - (int64_t)kb * M);
+    sa_out[(int64_t)kb * ldm + m] = ue8m0_to_f32(sa_words[(int64_t)(kb >> 2) * sa_kw + m], kb);
+    return;
+  }
+  idx -= n_tok;
+  if (idx >= (int64_t)NB * KB) return;
+  const int nb = (int)(idx / KB), kb = (int)(idx - (int64_t)nb * KB);
+  sb_out[idx] = ue8m0_to_f32(sb_words[(int64_t)(kb >> 2) * sb_kw + (int64_t)nb * 128 * sb_row], kb);
 }
 
 size_t ue8m0_unpacked_bytes(int64_t M, int64_t N, int64_t K) {
@@ -732,10 +743,9 @@ extern "C" int mi355_fp8_blockwise_mm_ue8m0(const void* a, const void* b, const 
   const int NB = (int)((N + 127) / 128);
   float* sa_f = static_cast<float*>(workspace);
   float* sb_f = sa_f + ldm * KB;
-  hipLaunchKernelGGL(unpack_ue8m0_kernel, dim3((unsigned)(((int64_t)M * KB + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint32_t*>(sa_words), (int64_t)1, sa_sk, 1, sa_f, (int64_t)1, ldm, (int)M, KB);
-  hipLaunchKernelGGL(unpack_ue8m0_kernel, dim3((unsigned)(((int64_t)NB * KB + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint32_t*>(sb_words), sb_sn, sb_sk, 128, sb_f, (int64_t)KB, (int64_t)1, NB, KB);
+  hipLaunchKernelGGL(unpack_ue8m0_kernel, dim3((unsigned)(((int64_t)(M + NB) * KB + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint32_t*>(sa_words), sa_sk, sa_f, ldm, (int)M, static_cast<const uint32_t*>(sb_words), sb_sn,
+                     sb_sk, sb_f, NB, KB);
   rc = check_launch(what);
   if (rc != MI355_OK) return rc;
   p.sa = sa_f, p.sa_sm = 1, p.sa_sk = ldm;
