@@ -24,6 +24,7 @@ struct GemmParams {
   const float* sb;
   const void* bias;        // optional [N] in the output dtype (INT8 GEMM; per-channel FP8 epilogue)
   const float* col_scale;  // FP8 only, optional [N]: per-channel scale applied in the epilogue (fp8_scaled_mm)
+  const float* row_scale;  // FP8 two-phase kernel in its epilogue-scaled mode only: per-token scale [M]
   void* out;
   void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
   int M, N, K;
@@ -156,6 +157,9 @@ int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what);
 // The same kernel for packed power-of-two (UE8M0) scales on both operands, applied by the MFMA itself: p.sa / p.sb point
 // to 32-bit words of four exponent bytes (see fp8_gemm_pp_kernel).  K % 128 == 0.
 int launch_fp8_pp_ue8m0(GemmParams& p, hipStream_t stream, const char* what);
+// The same kernel with one scale per token (p.row_scale) and per channel (p.col_scale) applied after the K loop, which
+// then carries no scale arithmetic; p.sa must point to >= 4 * M readable, 16-byte aligned bytes.  K % 128 == 0.
+int launch_fp8_pp_rowcol(GemmParams& p, hipStream_t stream, const char* what);
 // Token scales must be M-major with a pitch that is a multiple of four floats and a 16-byte aligned base.
 
 

@@ -38,6 +38,7 @@
 namespace mi355 {
 namespace {
 
+constexpr int SM_BLOCK_F32 = 0, SM_UE8M0 = 1, SM_EPILOGUE = 2;
 constexpr int G_THREADS = 512;
 constexpr int G_BM = 256, G_BN = 256, G_WM = 128, G_WN = 64;
 constexpr int G_MT = G_WM / 16, G_NT = G_WN / 16;  // 8 token tiles x 4 channel tiles per wave
@@ -157,8 +158,9 @@ __device__ __forceinline__ void memory_end() {
 
 // Memory phase, operand part: token tiles 4 * HALF .. + 3 of `cur` (and, for HALF == 0, the four weight fragments)
 // into registers; their scales times the weight-block scale.
-// UE8M0: scb[jj] carries (as bits) the token's packed exponent word shifted so that the byte of this K block is byte 0.
-template <int HALF, bool UE8M0>
+// SM_UE8M0: scb[jj] carries (as bits) the token's packed exponent word shifted so that the byte of this K block is byte 0;
+// SM_EPILOGUE: the exponent byte of 1.0.
+template <int HALF, int SM>
 __device__ __forceinline__ void read_operands(const PpState& s, const uint8_t* cur, const float* sc_cur, float sbv, int kb,
                                               Frag (&w)[G_NT], Frag (&tok)[G_HT], float (&scb)[G_HT]) {
   const lds_cptr ch0 = (lds_cptr)cur + s.ch_off[0], ch1 = (lds_cptr)cur + s.ch_off[1];
@@ -178,8 +180,10 @@ __device__ __forceinline__ void read_operands(const PpState& s, const uint8_t* c
   }
 #pragma unroll
   for (int jj = 0; jj < G_HT; ++jj) {
-    if constexpr (UE8M0)
+    if constexpr (SM == SM_UE8M0)
       scb[jj] = __uint_as_float(__float_as_uint(scp[(HALF * G_HT + jj) * 16]) >> ((kb & 3) * 8));
+    else if constexpr (SM == SM_EPILOGUE)
+      scb[jj] = __uint_as_float(127u);
     else
       scb[jj] = scp[(HALF * G_HT + jj) * 16] * sbv;
   }
@@ -244,10 +248,48 @@ __device__ __forceinline__ void compute_ue8m0(const Frag (&w)[G_NT], const Frag 
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// UE8M0: p.sa / p.sb point to packed exponent words (int32): token word (m, kw) at sa[kw * sa_sk + m], channel word
-// (n, kw) at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb.
-template <bool KFULL, bool UE8M0>
+// r[v] = row_scale[m] * (col_scale[n + v] * r[v]) + bias[n + v], each step rounded (the order of fp8_scaled_mm's epilogue,
+// sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:529-547); channels at or past N repeat the last one and are never stored.
+__device__ __forceinline__ void row_col_epilogue(const GemmParams& p, int m, int n, float* r) {
+  const float rs = p.row_scale[min(m, p.M - 1)];
+  const uint16_t* b = reinterpret_cast<const uint16_t*>(p.bias);
+  float cs[4], bv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (n + 4 <= p.N && (reinterpret_cast<uintptr_t>(p.col_scale + n) & 15) == 0 &&
+      (p.bias == nullptr || (reinterpret_cast<uintptr_t>(b + n) & 7) == 0)) {
+    // one 16-byte and one 8-byte load instead of eight scattered ones
+    const v4f c = *reinterpret_cast<const v4f*>(p.col_scale + n);
+    cs[0] = c[0], cs[1] = c[1], cs[2] = c[2], cs[3] = c[3];
+    if (p.bias) {
+      const u32x2 hb = *reinterpret_cast<const u32x2*>(b + n);
+      const uint32_t h[4] = {hb.x & 0xffffu, hb.x >> 16, hb.y & 0xffffu, hb.y >> 16};
+#pragma unroll
+      for (int v = 0; v < 4; ++v) bv[v] = (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(h[v]) : f16_bits_to_f32(h[v]);
+    }
+  } else {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int nn = min(n + v, p.N - 1);
+      cs[v] = p.col_scale[nn];
+      if (p.bias) bv[v] = (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(b[nn]) : f16_bits_to_f32(b[nn]);
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const float t = mul_rn(rs, mul_rn(cs[v], r[v]));
+    r[v] = p.bias ? add_rn(t, bv[v]) : t;
+  }
+}
+
+// SM, where the scales are applied:
+//   SM_BLOCK_F32  fp32 scales per K block, by promotion FMAs (the blockwise GEMM of the reference);
+//   SM_UE8M0      p.sa / p.sb point to packed exponent words (int32): token word (m, kw) at sa[kw * sa_sk + m], channel word
+//                 (n, kw) at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb; the MFMA applies them;
+//   SM_EPILOGUE   one scale per token (p.row_scale) and per channel (p.col_scale), applied once, after the K loop, as
+//                 row_scale * (col_scale * acc) + bias; the K loop accumulates in the MFMA with unit scales.
+template <bool KFULL, int SM>
 __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams p) {
+  constexpr bool UE8M0 = SM == SM_UE8M0;
+  constexpr bool HW_SCALE = SM != SM_BLOCK_F32;  // scale operands of the MFMA instead of promotion FMAs
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -319,20 +361,20 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
   // One K block: M0, C0, M1, C1.  `cur` holds block kb; `nxt` takes set B of block kb + 1, `cur` set A of block kb + 2.
   auto k_block = [&](uint8_t* cur, uint8_t* nxt, int kb, float sbv) {
     const float* sc_cur = g_scale + (kb & 3) * G_BM;
-    // the weight block's exponent byte, in byte 0 of a register (sbv then carries the packed word as bits)
-    const int w_scale = UE8M0 ? (int)(__float_as_uint(sbv) >> ((kb & 3) * 8)) : 0;
-    if constexpr (!UE8M0) retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
-    read_operands<0, UE8M0>(s, cur, sc_cur, sbv, kb, w, tok, scb);
+    // the weight block's exponent byte, in byte 0 of a register (for SM_UE8M0 sbv carries the packed word as bits)
+    const int w_scale = UE8M0 ? (int)(__float_as_uint(sbv) >> ((kb & 3) * 8)) : 127;
+    if constexpr (!HW_SCALE) retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
+    read_operands<0, SM>(s, cur, sc_cur, sbv, kb, w, tok, scb);
     issue_set_b<KFULL>(s, nxt, kb + 1);
     memory_end();
-    if constexpr (UE8M0) compute_ue8m0<0>(w, tok, scb, w_scale, acc);
+    if constexpr (HW_SCALE) compute_ue8m0<0>(w, tok, scb, w_scale, acc);
     else compute<0>(w, tok, scb, acc, pd);
     compute_end();
-    if constexpr (!UE8M0) retire<0>(pd, acc);
-    read_operands<1, UE8M0>(s, cur, sc_cur, sbv, kb, w, tok, scb);
+    if constexpr (!HW_SCALE) retire<0>(pd, acc);
+    read_operands<1, SM>(s, cur, sc_cur, sbv, kb, w, tok, scb);
     issue_set_a<KFULL, UE8M0>(s, cur, kb + 2);
     memory_end();
-    if constexpr (UE8M0) compute_ue8m0<1>(w, tok, scb, w_scale, acc);
+    if constexpr (HW_SCALE) compute_ue8m0<1>(w, tok, scb, w_scale, acc);
     else compute<1>(w, tok, scb, acc, pd);
     compute_end();
   };
@@ -346,7 +388,7 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
     sb_cur = sb_2;
   }
   if (kb < nkb) k_block(g_stage0, g_stage1, kb, sb_cur);
-  if constexpr (!UE8M0) retire<1>(pd, acc);
+  if constexpr (!HW_SCALE) retire<1>(pd, acc);
   if (grp == 0) compute_end();  // as many barriers as group 1
   // the last requests refetch the last block into rows nobody reads any more: they must not outlive the workgroup's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -358,7 +400,8 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
     for (int j = 0; j < G_MT; ++j)
 #pragma unroll
       for (int i = 0; i < G_NT; ++i) {
-        fp8_channel_epilogue(p, n0 + wave_n * G_WN + i * 16 + 4 * q, acc[i][j]);
+        if constexpr (SM == SM_EPILOGUE) row_col_epilogue(p, m0 + grp * G_WM + j * 16 + l16, n0 + wave_n * G_WN + i * 16 + 4 * q, acc[i][j]);
+        else fp8_channel_epilogue(p, n0 + wave_n * G_WN + i * 16 + 4 * q, acc[i][j]);
         out_tile_put4(g_stages, grp * G_WM + j * 16 + l16, wave_n * G_WN + i * 16 + 4 * q, p.out_dtype, acc[i][j]);
       }
     __syncthreads();
@@ -374,7 +417,8 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
     for (int i = 0; i < G_NT; ++i) {
       const int n = n0 + wave_n * G_WN + i * 16 + 4 * q;
       if (n >= p.N) continue;
-      fp8_channel_epilogue(p, n, acc[i][j]);
+      if constexpr (SM == SM_EPILOGUE) row_col_epilogue(p, m, n, acc[i][j]);
+      else fp8_channel_epilogue(p, n, acc[i][j]);
       store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], min(4, p.N - n), vec_ok);
     }
   }
@@ -390,9 +434,9 @@ int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_n = (p.N + G_BN - 1) / G_BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
   if (p.K % KSTEP == 0)
-    hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, false>), grid, dim3(G_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, SM_BLOCK_F32>), grid, dim3(G_THREADS), 0, stream, p);
   else
-    hipLaunchKernelGGL((fp8_gemm_pp_kernel<false, false>), grid, dim3(G_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_pp_kernel<false, SM_BLOCK_F32>), grid, dim3(G_THREADS), 0, stream, p);
   return check_launch(what);
 }
 
@@ -402,7 +446,19 @@ int launch_fp8_pp_ue8m0(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + G_BM - 1) / G_BM;
   p.tiles_n = (p.N + G_BN - 1) / G_BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
-  hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, true>), grid, dim3(G_THREADS), 0, stream, p);
+  hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, SM_UE8M0>), grid, dim3(G_THREADS), 0, stream, p);
+  return check_launch(what);
+}
+
+
+// Per-token x per-channel scales applied in the epilogue (p.row_scale [M], p.col_scale [N], optional p.bias); the K loop
+// runs without any scale arithmetic.  p.sa must point to at least 4 * M readable, 16-byte aligned bytes (the scale-load
+// slots of the schedule still fetch, nobody reads what they bring) and p.sb to one readable float.  K % 128 == 0.
+int launch_fp8_pp_rowcol(GemmParams& p, hipStream_t stream, const char* what) {
+  p.tiles_m = (p.M + G_BM - 1) / G_BM;
+  p.tiles_n = (p.N + G_BN - 1) / G_BN;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, SM_EPILOGUE>), grid, dim3(G_THREADS), 0, stream, p);
   return check_launch(what);
 }
 

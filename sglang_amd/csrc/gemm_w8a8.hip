@@ -832,6 +832,16 @@ extern "C" int mi355_fp8_scaled_mm(const void* a, const void* b, const float* sa
   MI355_REQUIRE(sb != nullptr, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
   p.col_scale = sb;
   p.bias = bias;
+  p.kb_total = (p.K + KSTEP - 1) / KSTEP;
+  const Route r = choose_route(true, p.M, p.N, p.K, p.lda, p.ldb, operands_aligned(p));
+  if (r.kernel == RK_PINGPONG && K % KSTEP == 0) {
+    // large M: accumulate in the MFMA with unit scales, apply both scales once in the epilogue (the reference's order)
+    p.row_scale = sa;
+    p.sa = reinterpret_cast<const float*>(p.a);  // readable filler for the schedule's scale-load slots
+    p.sa_sk = 0;
+    p.splits = 1, p.kb_per_split = p.kb_total;
+    return launch_fp8_pp_rowcol(p, static_cast<hipStream_t>(stream), what);
+  }
   return run_gemm<true>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
 }
 
