@@ -55,6 +55,36 @@ def test_argument_validation_happens_before_any_device_work():
     assert L.mi355_last_error() == b""
 
 
+def test_newer_entry_points_validate_before_any_device_work():
+    """Every check below fails (or succeeds as an empty problem) on the host: no kernel is launched without a GPU."""
+    from sglang_amd import _lib
+
+    L = _lib.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    # per-tensor quantizer: dtype, per-row scale copy only in static mode, empty tensor
+    assert L.mi355_per_tensor_quant_fp8(p, _lib.I8, p, p, 16, 0, None, 0, None) == 1
+    assert L.mi355_per_tensor_quant_fp8(p, _lib.BF16, p, p, 16, 0, p, 4, None) == 1 and b"static" in L.mi355_last_error()
+    assert L.mi355_per_tensor_quant_fp8(p, _lib.BF16, p, None, 16, 0, None, 0, None) == 1
+    assert L.mi355_per_tensor_quant_fp8(None, _lib.BF16, None, p, 0, 0, None, 0, None) == 0
+    # fused activation + quantizer: fp32 input is not a 16-bit type, hidden size must be whole groups, empty problem
+    assert L.mi355_silu_mul_group_quant_fp8(p, _lib.F32, p, p, 1, 4, 128, None, 0, 4, None) == 1
+    assert L.mi355_silu_mul_group_quant_fp8(p, _lib.BF16, p, p, 1, 4, 100, None, 0, 4, None) == 2
+    assert L.mi355_silu_mul_group_quant_fp8(None, _lib.BF16, None, None, 0, 4, 128, None, 0, 4, None) == 0
+    # weight-side block cast / dequant
+    assert L.mi355_block_cast_to_fp8(p, _lib.I8, p, p, 128, 128, None) == 1
+    assert L.mi355_block_cast_to_fp8(None, _lib.BF16, None, None, 0, 128, None) == 0
+    assert L.mi355_block_dequant_fp8(p, p, p, _lib.I8, 128, 128, None) == 1
+    assert L.mi355_block_dequant_fp8(None, None, None, _lib.BF16, 128, 0, None) == 0
+    # UE8M0 GEMM: bias needs a 16-bit output, strides at least the row length, empty problem; workspace query is pure
+    assert L.mi355_fp8_blockwise_mm_ue8m0(p, p, p, p, p, p, _lib.F32, 4, 128, 128, 128, 128, 4, 1, 128, 128, None, 0, None) == 1
+    assert L.mi355_fp8_blockwise_mm_ue8m0(p, p, p, p, None, p, _lib.BF16, 4, 128, 128, 64, 128, 4, 1, 128, 128, None, 0, None) == 1
+    assert L.mi355_fp8_blockwise_mm_ue8m0(p, p, p, p, None, p, _lib.BF16, 0, 128, 128, 128, 128, 4, 1, 128, 128, None, 0, None) == 0
+    assert L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(0, 128, 128) == 0
+    need = L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(4, 512, 1024)
+    assert need > 0 and need % 256 == 0
+
+
 def test_operator_schemas_are_the_reference_ones():
     from sglang_amd import ops
 
