@@ -109,6 +109,37 @@ int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const 
                            void* stream);
 
 /*
+ * Grouped blockwise FP8 GEMM: the expert GEMMs of a mixture-of-experts layer in one call.  Token rows of all experts are
+ * stacked; expert e owns rows expert_offsets[e] .. expert_offsets[e] + problem_sizes[3 * e] - 1 and
+ *   out[r, n] = cast( sum_kb scales_a[r, kb] * scales_b[e, n / 128, kb] * sum_{k in block kb} a[r, k] * b[e, n, k] )
+ *   a             e4m3fn [total_m, K], row stride lda;  scales_a fp32, element (r, kb) at scales_a[r * sa_sm + kb * sa_sk]
+ *   b             e4m3fn, expert e's [N, K] matrix at b + e * b_expert_stride, row stride ldb (bytes = elements)
+ *   scales_b      fp32, block (e, nb, kb) at scales_b[e * sb_expert_stride + nb * sb_sn + kb * sb_sk]
+ *   problem_sizes int32 [num_experts, 3] ON THE DEVICE: (rows, N, K) per expert; only the row counts are read, N and K
+ *                 are the arguments (the reference's callers build every row with the same N and K)
+ *   expert_offsets int32 [num_experts] ON THE DEVICE: first stacked row of each expert
+ *   out           bfloat16 or float16 [total_m, N], row stride ldo; rows owned by no expert are left untouched
+ * Row counts and offsets are clamped into [0, total_m] on the device, so inconsistent routing data gives wrong rows, not
+ * out-of-bounds accesses.  K % 128 == 0 and 16-byte aligned operand rows are required (MI355_ERR_UNSUPPORTED otherwise).
+ * The tile schedule and the re-laid-out token scales live in `workspace` (256-byte aligned,
+ * >= ..._workspace_bytes(num_experts, total_m, N, K)); nothing is allocated, three launches on `stream`.
+ * Replaces fp8_blockwise_scaled_grouped_mm (sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:650-810, set-up kernel
+ * sgl-kernel/csrc/moe/cutlass_moe_helper.cu:17-80, Python sgl-kernel/python/sgl_kernel/moe.py:96-135; caller
+ * cutlass_fused_experts_fp8, python/sglang/srt/layers/moe/cutlass_moe.py:146-201).  The reference's pointer, stride and
+ * scale-layout arrays are scratch its own set-up kernel fills; here that scratch is the workspace.
+ * ..._plan writes "kernel=grouped_dma3 tile=<64|128>x256 max_tiles_m=<n> tiles_n=<n>" (host only).
+ */
+size_t mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes(int64_t num_experts, int64_t total_m, int64_t N, int64_t K);
+int mi355_fp8_blockwise_scaled_grouped_mm_plan(int64_t num_experts, int64_t total_m, int64_t N, int64_t K, char* buf,
+                                               size_t buf_len);
+int mi355_fp8_blockwise_scaled_grouped_mm(const void* a, const void* b, const float* scales_a, const float* scales_b, void* out,
+                                          int out_dtype, const int32_t* problem_sizes, const int32_t* expert_offsets,
+                                          int64_t num_experts, int64_t total_m, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                          int64_t b_expert_stride, int64_t sa_sm, int64_t sa_sk, int64_t sb_expert_stride,
+                                          int64_t sb_sn, int64_t sb_sk, int64_t ldo, void* workspace, size_t workspace_bytes,
+                                          void* stream);
+
+/*
  * Blockwise FP8 GEMM with power-of-two (UE8M0) scales on BOTH operands, the form DeepSeek-V3 checkpoints take after
  * requant_weight_ue8m0 and activations take from per_token_group_quant_fp8(scale_ue8m0=True):
  *   out[m,n] = cast( sum_kb 2^(ea[m,kb] - 127) * 2^(eb[n,kb] - 127) * sum_{k in block kb} a[m,k] * b[n,k]  (+ bias[n]) )

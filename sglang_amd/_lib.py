@@ -28,6 +28,9 @@ EXPORTS = (
     "mi355_fp8_blockwise_mm_noalloc",
     "mi355_fp8_blockwise_mm_ue8m0_workspace_bytes",
     "mi355_fp8_blockwise_mm_ue8m0",
+    "mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes",
+    "mi355_fp8_blockwise_scaled_grouped_mm_plan",
+    "mi355_fp8_blockwise_scaled_grouped_mm",
     "mi355_int8_scaled_mm_workspace_bytes",
     "mi355_int8_scaled_mm",
     "mi355_fp8_blockwise_mm_plan",
@@ -89,6 +92,12 @@ def lib() -> ctypes.CDLL:
     L.mi355_fp8_blockwise_mm_ue8m0.restype = i32
     L.mi355_fp8_blockwise_mm_noalloc.argtypes = [vp, vp, vp, vp, vp, i32] + [i64] * 10 + [vp]
     L.mi355_fp8_blockwise_mm_noalloc.restype = i32
+    L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes.argtypes = [i64, i64, i64, i64]
+    L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes.restype = sz
+    L.mi355_fp8_blockwise_scaled_grouped_mm_plan.argtypes = [i64, i64, i64, i64, ctypes.c_char_p, sz]
+    L.mi355_fp8_blockwise_scaled_grouped_mm_plan.restype = i32
+    L.mi355_fp8_blockwise_scaled_grouped_mm.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp] + [i64] * 13 + [vp, sz, vp]
+    L.mi355_fp8_blockwise_scaled_grouped_mm.restype = i32
     L.mi355_int8_scaled_mm_workspace_bytes.argtypes = [i64, i64, i64]
     L.mi355_int8_scaled_mm_workspace_bytes.restype = sz
     L.mi355_int8_scaled_mm.argtypes = [vp, vp, vp, vp, vp, vp, i32] + [i64] * 6 + [vp, sz, vp]
@@ -133,6 +142,18 @@ def gemm_plan(kind: str, M: int, N: int, K: int, aligned: bool = True) -> dict:
     for item in buf.value.decode().split():
         k, v = item.split("=")
         out[k] = v if k == "kernel" else int(v)
+    return out
+
+
+def grouped_gemm_plan(num_experts: int, total_m: int, N: int, K: int) -> dict:
+    """Tiling of the grouped FP8 GEMM for this many experts and stacked rows: {"kernel": str, "tile": "64x256" | "128x256",
+    "max_tiles_m": int, "tiles_n": int}."""
+    buf = ctypes.create_string_buffer(256)
+    check(lib().mi355_fp8_blockwise_scaled_grouped_mm_plan(num_experts, total_m, N, K, buf, len(buf)))
+    out = {}
+    for item in buf.value.decode().split():
+        k, v = item.split("=")
+        out[k] = v if k in ("kernel", "tile") else int(v)
     return out
 
 

@@ -172,6 +172,21 @@ struct Dma3Plan {
 };
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K);
 int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);   // bm: 64 or 128, from dma3_plan()
+
+// Grouped problems on the same tile body: token rows of all experts stacked in one matrix, one weight matrix per expert.
+// `g` describes expert 0 (a, out, b, sb, and sa = the re-laid-out token scales: M-major, every expert's first row moved
+// to column ((row0 + 3) & ~3) + 4 * expert so that each expert starts on a whole quad); N, K, strides and kb_total are
+// common to all experts; splits = 1.  `tiles` has one record per token tile, written on the device from the problem
+// sizes: {expert (-1: unused), first stacked row of the expert, rows of the expert, first row of the tile in the expert}.
+struct GroupedParams {
+  GemmParams g;
+  const v4i* tiles;
+  int64_t b_expert_stride;   // bytes between consecutive experts' weight matrices
+  int64_t sb_expert_stride;  // floats between consecutive experts' weight-block scales
+  int max_tiles_m;           // records in `tiles`; the grid is max_tiles_m * tiles_n
+  int out_elem;              // bytes per output element
+};
+int launch_fp8_grouped_dma3(GroupedParams& gp, int bm, hipStream_t stream, const char* what);  // bm: 64 or 128
 int launch_int8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
 
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases, direct-to-LDS loads,

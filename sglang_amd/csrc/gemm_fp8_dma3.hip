@@ -148,8 +148,9 @@ __device__ __forceinline__ void wait_and_barrier() {
   else asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
 }
 
+// One BM x 256 output tile at (m0, n0), K blocks of split `split`, by the whole workgroup.
 template <int BM, bool SPLIT>
-__global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmParams p) {
+__device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, int split) {
   constexpr int WM = BM / 2, MT = WM / 16, LOADS = Dma3State<BM>::LOADS;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -157,9 +158,7 @@ __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmPara
   const int wave_m = wave >> 2, wave_n = wave & 3;
   const int l16 = lane & 15, q = lane >> 4;
 
-  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
-  const int m0 = tc.tile_m * BM, n0 = tc.tile_n * T_BN;
-  const int kb_begin = tc.split * p.kb_per_split;
+  const int kb_begin = split * p.kb_per_split;
   const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
   const int nkb = kb_end - kb_begin;
 
@@ -242,7 +241,7 @@ __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmPara
       if (n >= p.N) continue;
       const int nvalid = min(4, p.N - n);
       if constexpr (SPLIT) {
-        float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)tc.split * p.M + m) * p.N + n;
+        float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)split * p.M + m) * p.N + n;
 #pragma unroll
         for (int v = 0; v < 4; ++v)
           if (v < nvalid) wsp[v] = acc[i][j][v];
@@ -252,6 +251,42 @@ __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmPara
       }
     }
   }
+}
+
+template <int BM, bool SPLIT>
+__global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmParams p) {
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
+  dma3_tile<BM, SPLIT>(p, tc.tile_m * BM, tc.tile_n * T_BN, tc.split);
+}
+
+// Grouped problems: the workgroup looks its token tile up in the table the plan kernel wrote, moves the operand bases to
+// that expert and runs the ordinary tile.  Workgroup ids are renumbered so that each XCD gets a contiguous range (as in
+// tile_of_block); inside a range GROUPED_GM token tiles at a time are walked over all channel tiles, token tile fastest,
+// so that the token tiles of one expert that use the same weight rows run together on one XCD's L2.
+constexpr int GROUPED_GM = 4;
+
+template <int BM>
+__global__ __launch_bounds__(T_THREADS) void fp8_grouped_dma3_kernel(const GroupedParams gp) {
+  int bid = blockIdx.x;
+  const int per = gridDim.x >> 3;
+  if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
+  const int span = GROUPED_GM * gp.g.tiles_n;
+  const int grp = bid / span, r = bid - grp * span;
+  const int gm = min(GROUPED_GM, gp.max_tiles_m - grp * GROUPED_GM);
+  const int tile_n = r / gm, t = grp * GROUPED_GM + r % gm;
+  const v4i rec = gp.tiles[t];
+  const int e = __builtin_amdgcn_readfirstlane(rec.x);
+  if (e < 0) return;  // the whole workgroup leaves before any barrier
+  const int row0 = __builtin_amdgcn_readfirstlane(rec.y), rows = __builtin_amdgcn_readfirstlane(rec.z);
+  const int m0 = __builtin_amdgcn_readfirstlane(rec.w);
+  GemmParams p = gp.g;
+  p.a += (int64_t)row0 * p.lda;
+  p.b += (int64_t)e * gp.b_expert_stride;
+  p.sb += (int64_t)e * gp.sb_expert_stride;
+  p.sa += ((row0 + 3) & ~3) + 4 * e;
+  p.out = reinterpret_cast<uint8_t*>(p.out) + (int64_t)row0 * p.ldo * gp.out_elem;
+  p.M = rows;
+  dma3_tile<BM, false>(p, m0, tile_n * T_BN, 0);
 }
 
 template <int BM>
@@ -304,6 +339,17 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
   pl.kb_per_split = (int)((kb_total + pl.splits - 1) / pl.splits);
   pl.efficiency = best_score;
   return pl;
+}
+
+int launch_fp8_grouped_dma3(GroupedParams& gp, int bm, hipStream_t stream, const char* what) {
+  gp.g.tiles_n = (gp.g.N + T_BN - 1) / T_BN;
+  gp.g.splits = 1, gp.g.kb_per_split = gp.g.kb_total;
+  const dim3 grid((unsigned)(gp.max_tiles_m * gp.g.tiles_n));
+  if (bm == 64)
+    hipLaunchKernelGGL(fp8_grouped_dma3_kernel<64>, grid, dim3(T_THREADS), 0, stream, gp);
+  else
+    hipLaunchKernelGGL(fp8_grouped_dma3_kernel<128>, grid, dim3(T_THREADS), 0, stream, gp);
+  return check_launch(what);
 }
 
 int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what) {
