@@ -16,6 +16,7 @@ Infinity Cache.
   fp8_decode   FP8 gate_up at M=1          int8_gemm             INT8 gate_up (K=4096 -> N=28672) at M=4096
   fp8:M:K:N    any blockwise-FP8 linear    int8:M:K:N            any INT8 linear
   fp8_ue8m0:M:K:N  the same linear with power-of-two (UE8M0) scales on both operands
+  fp8_grouped:E:ROWS:K:N  grouped FP8 GEMM of E experts with ROWS token rows each (mixture-of-experts)
   copy         a plain 256 MiB device copy (calibration of the HBM traffic counters)
   silu_quant   silu(gate) * up fused in front of the group quantizer (packed UE8M0 scales)
 
@@ -349,6 +350,55 @@ def bench_fp8_ue8m0_gemm(name, M, K, N, steps, warmup):
     }
 
 
+def bench_fp8_grouped_gemm(E, m_per, K, N, steps, warmup):
+    """Grouped blockwise-FP8 GEMM (the expert GEMMs of a mixture-of-experts layer): E experts with m_per stacked token
+    rows each, one [N, K] weight per expert; the shapes of sgl-kernel/benchmark/bench_fp8_blockwise_group_gemm.py.  One
+    step is the whole call: schedule kernel, scale re-layout and the GEMM."""
+    import torch
+
+    from sglang_amd import _lib, fp8_kernel
+    from sglang_amd.workloads import make_activation
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(N * 10007 + K + E)
+    T = E * m_per
+    nbuf = max(2, min(6, int(600e6 // (E * N * K)) + 1))
+    ws, wss = [], []
+    for _ in range(nbuf):
+        w_q, w_s = device_block_fp8_weight(E * N, K, gen, dev)
+        ws.append(w_q.view(E, N, K))
+        wss.append(w_s.view(E, N // 128, K // 128))
+    x = make_activation(T, K).to(dev)
+    x_q, x_s = fp8_kernel.sglang_per_token_group_quant_fp8(x, 128)
+    sizes = torch.tensor([[m_per, N, K]] * E, dtype=torch.int32, device=dev)
+    offsets = torch.arange(E, dtype=torch.int32, device=dev) * m_per
+    L = _lib.lib()
+    wsb = L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes(E, T, N, K)
+    wsbuf = torch.empty(wsb, dtype=torch.uint8, device=dev)
+    outs = [torch.empty(T, N, dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+    stream = torch.cuda.current_stream().cuda_stream
+    args = [(x_q.data_ptr(), ws[i].data_ptr(), x_s.data_ptr(), wss[i].data_ptr(), outs[i].data_ptr(), _lib.BF16, sizes.data_ptr(),
+             offsets.data_ptr(), E, T, N, K, x_q.stride(0), K, N * K, x_s.stride(0), x_s.stride(1), wss[i].stride(0),
+             wss[i].stride(1), wss[i].stride(2), N, wsbuf.data_ptr(), wsb, stream) for i in range(nbuf)]
+
+    def step(i):
+        _lib.check(L.mi355_fp8_blockwise_scaled_grouped_mm(*args[i]))
+
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms, b2b)
+    kb = K // 128
+    flops = 2.0 * T * N * K
+    nbytes = float(E * N * K + T * K + 4 * T * kb + 4 * E * (N // 128) * kb + 2 * T * N)
+    plan = _lib.grouped_gemm_plan(E, T, N, K)
+    return {
+        "workload": f"fp8_grouped_gemm E={E} rows/expert={m_per} K={K} N={N} (e4m3fn x e4m3fn, 1x128 / 128x128 fp32 scales, bf16 out)",
+        "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "fp8(e4m3fn) MFMA, f32 accumulate", "kernel": f"{plan['kernel']} {plan['small_tile']} (+ schedule, scale re-layout)",
+        "roofline": _roofline(flops, nbytes, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
+    }
+
+
 def bench_int8_gemm(name, M, K, N, steps, warmup, with_cpu=False):
     import torch
 
@@ -555,6 +605,9 @@ def main():
     elif wl.startswith("fp8_ue8m0:"):
         _, M, K, N = wl.split(":")
         rec = bench_fp8_ue8m0_gemm("shape", int(M), int(K), int(N), S, W)
+    elif wl.startswith("fp8_grouped:"):
+        _, E, m_per, K, N = wl.split(":")
+        rec = bench_fp8_grouped_gemm(int(E), int(m_per), int(K), int(N), S, W)
     elif wl.startswith("fp8:") or wl.startswith("int8:"):
         kind, M, K, N = wl.split(":")
         fn = bench_fp8_gemm if kind == "fp8" else bench_int8_gemm

@@ -122,12 +122,13 @@ int mi355_fp8_blockwise_mm(const void* a, const void* b, const float* sa, const 
  * Row counts and offsets are clamped into [0, total_m] on the device, so inconsistent routing data gives wrong rows, not
  * out-of-bounds accesses.  K % 128 == 0 and 16-byte aligned operand rows are required (MI355_ERR_UNSUPPORTED otherwise).
  * The tile schedule and the re-laid-out token scales live in `workspace` (256-byte aligned,
- * >= ..._workspace_bytes(num_experts, total_m, N, K)); nothing is allocated, three launches on `stream`.
+ * >= ..._workspace_bytes(num_experts, total_m, N, K)); nothing is allocated, three or four launches on `stream`.
  * Replaces fp8_blockwise_scaled_grouped_mm (sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:650-810, set-up kernel
  * sgl-kernel/csrc/moe/cutlass_moe_helper.cu:17-80, Python sgl-kernel/python/sgl_kernel/moe.py:96-135; caller
  * cutlass_fused_experts_fp8, python/sglang/srt/layers/moe/cutlass_moe.py:146-201).  The reference's pointer, stride and
  * scale-layout arrays are scratch its own set-up kernel fills; here that scratch is the workspace.
- * ..._plan writes "kernel=grouped_dma3 tile=<64|128>x256 max_tiles_m=<n> tiles_n=<n>" (host only).
+ * ..._plan writes "kernel=grouped_pingpong+grouped_dma3 small_tile=<64|128>x256 max_big_tiles=<n> max_small_tiles=<n>
+ * tiles_n=<n>" (host only): experts are cut into 256-row tiles plus, for a rest of at most 128 rows, small tiles.
  */
 size_t mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes(int64_t num_experts, int64_t total_m, int64_t N, int64_t K);
 int mi355_fp8_blockwise_scaled_grouped_mm_plan(int64_t num_experts, int64_t total_m, int64_t N, int64_t K, char* buf,

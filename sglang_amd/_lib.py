@@ -146,14 +146,14 @@ def gemm_plan(kind: str, M: int, N: int, K: int, aligned: bool = True) -> dict:
 
 
 def grouped_gemm_plan(num_experts: int, total_m: int, N: int, K: int) -> dict:
-    """Tiling of the grouped FP8 GEMM for this many experts and stacked rows: {"kernel": str, "tile": "64x256" | "128x256",
-    "max_tiles_m": int, "tiles_n": int}."""
+    """Tiling of the grouped FP8 GEMM for this many experts and stacked rows: {"kernel": str, "small_tile": "64x256" |
+    "128x256", "max_big_tiles": int, "max_small_tiles": int, "tiles_n": int}."""
     buf = ctypes.create_string_buffer(256)
     check(lib().mi355_fp8_blockwise_scaled_grouped_mm_plan(num_experts, total_m, N, K, buf, len(buf)))
     out = {}
     for item in buf.value.decode().split():
         k, v = item.split("=")
-        out[k] = v if k in ("kernel", "tile") else int(v)
+        out[k] = v if k in ("kernel", "small_tile") else int(v)
     return out
 
 

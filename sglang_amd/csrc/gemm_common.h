@@ -173,20 +173,53 @@ struct Dma3Plan {
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K);
 int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);   // bm: 64 or 128, from dma3_plan()
 
-// Grouped problems on the same tile body: token rows of all experts stacked in one matrix, one weight matrix per expert.
-// `g` describes expert 0 (a, out, b, sb, and sa = the re-laid-out token scales: M-major, every expert's first row moved
-// to column ((row0 + 3) & ~3) + 4 * expert so that each expert starts on a whole quad); N, K, strides and kb_total are
-// common to all experts; splits = 1.  `tiles` has one record per token tile, written on the device from the problem
-// sizes: {expert (-1: unused), first stacked row of the expert, rows of the expert, first row of the tile in the expert}.
+// Grouped problems on the tile bodies of the dense kernels: token rows of all experts stacked in one matrix, one weight
+// matrix per expert.  `g` describes expert 0 (a, out, b, sb, and sa = the re-laid-out token scales: M-major, every
+// expert's first row moved to column ((row0 + 3) & ~3) + 4 * expert so that each expert starts on a whole quad); N, K,
+// strides and kb_total are common to all experts; splits = 1.  `tiles` is written on the device from the problem sizes:
+// tiles[0].x = number of token tiles of this launch, then one record per token tile: {expert, first stacked row of the
+// expert, rows of the expert, first row of the tile in the expert}.
 struct GroupedParams {
   GemmParams g;
   const v4i* tiles;
   int64_t b_expert_stride;   // bytes between consecutive experts' weight matrices
   int64_t sb_expert_stride;  // floats between consecutive experts' weight-block scales
-  int max_tiles_m;           // records in `tiles`; the grid is max_tiles_m * tiles_n
+  int max_tiles_m;           // upper bound on the number of records; the grid is max_tiles_m * tiles_n
   int out_elem;              // bytes per output element
 };
-int launch_fp8_grouped_dma3(GroupedParams& gp, int bm, hipStream_t stream, const char* what);  // bm: 64 or 128
+// Workgroup -> (token tile record, channel tile) and the parameter block of that tile's expert.  The grid is sized for the
+// largest possible number of token tiles; workgroups past the real number (known only on the device) leave at once.  The
+// ids below it are renumbered so that each XCD gets a contiguous range (as in tile_of_block; it has to be the real
+// number, or the XCDs that are handed the high ids would get nothing but empty workgroups); inside a range GROUPED_GM
+// token tiles at a time are walked over all channel tiles, token tile fastest, so that the token tiles of one expert
+// that use the same weight rows run together on one XCD's L2.  Returns false for a workgroup without a tile.
+constexpr int GROUPED_GM = 4;
+__device__ __forceinline__ bool grouped_tile_of_block(const GroupedParams& gp, GemmParams& p, int& m0, int& tile_n) {
+  const int count = min(__builtin_amdgcn_readfirstlane(gp.tiles[0].x), gp.max_tiles_m);
+  const int total = count * gp.g.tiles_n;
+  int bid = blockIdx.x;
+  if (bid >= total) return false;
+  const int per = total >> 3;
+  if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
+  const int span = GROUPED_GM * gp.g.tiles_n;
+  const int grp = bid / span, r = bid - grp * span;
+  const int gm = min(GROUPED_GM, count - grp * GROUPED_GM);
+  tile_n = r / gm;
+  const v4i rec = gp.tiles[1 + grp * GROUPED_GM + r % gm];
+  const int e = __builtin_amdgcn_readfirstlane(rec.x);
+  const int row0 = __builtin_amdgcn_readfirstlane(rec.y);
+  m0 = __builtin_amdgcn_readfirstlane(rec.w);
+  p = gp.g;
+  p.a += (int64_t)row0 * p.lda;
+  p.b += (int64_t)e * gp.b_expert_stride;
+  p.sb += (int64_t)e * gp.sb_expert_stride;
+  p.sa += ((row0 + 3) & ~3) + 4 * e;
+  p.out = reinterpret_cast<uint8_t*>(p.out) + (int64_t)row0 * p.ldo * gp.out_elem;
+  p.M = __builtin_amdgcn_readfirstlane(rec.z);
+  return true;
+}
+int launch_fp8_grouped_dma3(GroupedParams& gp, int bm, hipStream_t stream, const char* what);  // gemm_fp8_dma3.hip; bm: 64 or 128
+int launch_fp8_grouped_pp(GroupedParams& gp, hipStream_t stream, const char* what);            // gemm_fp8_pp.hip: 256-row tiles
 int launch_int8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
 
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases, direct-to-LDS loads,

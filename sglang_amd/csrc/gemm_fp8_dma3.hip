@@ -259,33 +259,13 @@ __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmPara
   dma3_tile<BM, SPLIT>(p, tc.tile_m * BM, tc.tile_n * T_BN, tc.split);
 }
 
-// Grouped problems: the workgroup looks its token tile up in the table the plan kernel wrote, moves the operand bases to
-// that expert and runs the ordinary tile.  Workgroup ids are renumbered so that each XCD gets a contiguous range (as in
-// tile_of_block); inside a range GROUPED_GM token tiles at a time are walked over all channel tiles, token tile fastest,
-// so that the token tiles of one expert that use the same weight rows run together on one XCD's L2.
-constexpr int GROUPED_GM = 4;
-
+// Grouped problems (see GroupedParams): the workgroup's token tile comes from the table the plan kernel wrote, the
+// operand bases move to that tile's expert, and the ordinary tile runs.
 template <int BM>
 __global__ __launch_bounds__(T_THREADS) void fp8_grouped_dma3_kernel(const GroupedParams gp) {
-  int bid = blockIdx.x;
-  const int per = gridDim.x >> 3;
-  if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
-  const int span = GROUPED_GM * gp.g.tiles_n;
-  const int grp = bid / span, r = bid - grp * span;
-  const int gm = min(GROUPED_GM, gp.max_tiles_m - grp * GROUPED_GM);
-  const int tile_n = r / gm, t = grp * GROUPED_GM + r % gm;
-  const v4i rec = gp.tiles[t];
-  const int e = __builtin_amdgcn_readfirstlane(rec.x);
-  if (e < 0) return;  // the whole workgroup leaves before any barrier
-  const int row0 = __builtin_amdgcn_readfirstlane(rec.y), rows = __builtin_amdgcn_readfirstlane(rec.z);
-  const int m0 = __builtin_amdgcn_readfirstlane(rec.w);
-  GemmParams p = gp.g;
-  p.a += (int64_t)row0 * p.lda;
-  p.b += (int64_t)e * gp.b_expert_stride;
-  p.sb += (int64_t)e * gp.sb_expert_stride;
-  p.sa += ((row0 + 3) & ~3) + 4 * e;
-  p.out = reinterpret_cast<uint8_t*>(p.out) + (int64_t)row0 * p.ldo * gp.out_elem;
-  p.M = rows;
+  GemmParams p;
+  int m0, tile_n;
+  if (!grouped_tile_of_block(gp, p, m0, tile_n)) return;  // the whole workgroup leaves before any barrier
   dma3_tile<BM, false>(p, m0, tile_n * T_BN, 0);
 }
 

@@ -286,8 +286,9 @@ __device__ __forceinline__ void row_col_epilogue(const GemmParams& p, int m, int
 //                 (n, kw) at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb; the MFMA applies them;
 //   SM_EPILOGUE   one scale per token (p.row_scale) and per channel (p.col_scale), applied once, after the K loop, as
 //                 row_scale * (col_scale * acc) + bias; the K loop accumulates in the MFMA with unit scales.
+// One 256 x 256 output tile at (m0, n0) by the whole workgroup.
 template <bool KFULL, int SM>
-__global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams p) {
+__device__ __forceinline__ void pp_tile(const GemmParams& p, const int m0, const int n0) {
   constexpr bool UE8M0 = SM == SM_UE8M0;
   constexpr bool HW_SCALE = SM != SM_BLOCK_F32;  // scale operands of the MFMA instead of promotion FMAs
   const int tid = threadIdx.x;
@@ -297,8 +298,6 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
   const int wave_n = wave & 3;
   const int l16 = lane & 15, q = lane >> 4;
 
-  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
-  const int m0 = tc.tile_m * G_BM, n0 = tc.tile_n * G_BN;
   const int nkb = p.kb_total;
 
   PpState s;
@@ -424,9 +423,30 @@ __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams
   }
 }
 
+template <bool KFULL, int SM>
+__global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams p) {
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
+  pp_tile<KFULL, SM>(p, tc.tile_m * G_BM, tc.tile_n * G_BN);
+}
 
+// Grouped problems (see GroupedParams): the workgroup's token tile comes from the table the plan kernel wrote, the
+// operand bases move to that tile's expert.  Workgroup order as in fp8_grouped_dma3_kernel.
+__global__ __launch_bounds__(G_THREADS) void fp8_grouped_pp_kernel(const GroupedParams gp) {
+  GemmParams p;
+  int m0, tile_n;
+  if (!grouped_tile_of_block(gp, p, m0, tile_n)) return;  // the whole workgroup leaves before any barrier
+  pp_tile<true, SM_BLOCK_F32>(p, m0, tile_n * G_BN);
+}
 
 }  // namespace
+
+int launch_fp8_grouped_pp(GroupedParams& gp, hipStream_t stream, const char* what) {
+  gp.g.tiles_n = (gp.g.N + G_BN - 1) / G_BN;
+  gp.g.splits = 1, gp.g.kb_per_split = gp.g.kb_total;
+  const dim3 grid((unsigned)(gp.max_tiles_m * gp.g.tiles_n));
+  hipLaunchKernelGGL(fp8_grouped_pp_kernel, grid, dim3(G_THREADS), 0, stream, gp);
+  return check_launch(what);
+}
 
 // Needs 16-byte aligned rows, row offsets below 4 GiB and conforming token scales (fp8_scales_conform).
 int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what) {

@@ -99,6 +99,7 @@ def test_random_expert_sizes(gpu, oracle, num_experts, out_dtype):
     ("prefill_like", [130, 257, 128, 64, 511, 129, 300, 200], 768, 1024, "128x256"),
     ("tile_edges", [64, 65, 63, 128, 127, 129, 1, 256], 256, 256, "128x256"),
     ("many_small", [3] * 300, 128, 256, "64x256"),
+    ("large_experts", [1000, 513, 384, 2], 512, 512, "128x256"),
     ("ragged_channels", [40, 90, 17], 200, 384, "64x256"),
 ])
 def test_shapes_and_tile_heights(gpu, oracle, name, sizes, N, K, tile):
@@ -106,7 +107,7 @@ def test_shapes_and_tile_heights(gpu, oracle, name, sizes, N, K, tile):
 
     print(f"case {name}", flush=True)
     a, w, sa, sw, offsets, T = _problem(sizes, N, K, len(sizes) + N)
-    assert _lib.grouped_gemm_plan(len(sizes), T, N, K)["tile"] == tile
+    assert _lib.grouped_gemm_plan(len(sizes), T, N, K)["small_tile"] == tile
     out = _call(gpu, a, w, sa, sw, sizes, offsets, torch.bfloat16)  # no usable workspace given: the wrapper allocates one
     _verify(oracle, out, a, w, sa, sw, sizes, offsets, name)
 
