@@ -44,6 +44,9 @@ SCHEMAS = {
     "Tensor out_ptrs, Tensor a_scales_ptrs, Tensor b_scales_ptrs, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, "
     "Tensor stride_a, Tensor stride_b, Tensor stride_c, Tensor layout_sfa, Tensor layout_sfb, Tensor problem_sizes, "
     "Tensor expert_offsets, Tensor workspace) -> ()",
+    "es_fp8_blockwise_scaled_grouped_mm": "es_fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a, Tensor b, Tensor scales_a, "
+    "Tensor scales_b, Tensor stride_a, Tensor stride_b, Tensor stride_d, Tensor problem_sizes, Tensor expert_offsets, "
+    "Tensor workspace) -> ()",
 }
 
 
@@ -397,16 +400,9 @@ def fp8_blockwise_mm_ue8m0(a: torch.Tensor, b: torch.Tensor, a_words: torch.Tens
 
 # ---------------------------------------------------------------- grouped FP8 GEMM (mixture-of-experts)
 
-def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a, scales_b,
-                                    stride_a, stride_b, stride_c, layout_sfa, layout_sfb, problem_sizes, expert_offsets,
-                                    workspace):
-    """sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:650-810 (checks :668-706).  ``a`` [total_m, K] e4m3fn row-major,
-    ``b`` [E, K, N] e4m3fn column-major per expert (storage [E, N, K]), ``scales_a`` fp32 [total_m, K/128], ``scales_b``
-    fp32 [E, K/128, N/128] (storage [E, N/128, K/128]), ``problem_sizes`` int32 [E, 3] and ``expert_offsets`` int32 [E] on
-    the device, ``output`` [total_m, N] written in place.  The pointer, stride and scale-layout tensors are scratch of the
-    reference's kernels: they are type-checked like there and not used.  ``workspace`` is used when it is large enough
-    (the reference's callers pass hundreds of megabytes), otherwise a temporary one is allocated."""
-    op = "fp8_blockwise_scaled_grouped_mm"
+def _grouped_mm(op, output, a, b, scales_a, scales_b, problem_sizes, expert_offsets, workspace):
+    """Checks common to both grouped entry points (fp8_blockwise_moe_kernel.cu:668-677, es_fp8_blockwise.cu:46-55), the
+    layout checks the kernels need, and the call."""
     _require(problem_sizes.dim() == 2, "problem_sizes must be 2D tensor")
     _require(problem_sizes.size(1) == 3, "problem_sizes must have shape (num_experts, 3)")
     _require(problem_sizes.size(0) == expert_offsets.size(0), "Number of experts in problem_sizes must match expert_offsets")
@@ -416,19 +412,13 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
     _require(output.dtype in (torch.bfloat16, torch.float16), "output must be bfloat16 or half")
     _require(scales_a.dtype == torch.float32, "scales_a must be float32")
     _require(scales_b.dtype == torch.float32, "scales_b must be float32")
-    for t, name in ((stride_a, "stride_a"), (stride_b, "stride_b"), (stride_c, "stride_c")):
-        _require(t.dtype == torch.int64 and t.dim() == 1, f"{name} must be a 1D int64 tensor")
-    for t, name in ((layout_sfa, "layout_sfa"), (layout_sfb, "layout_sfb")):
-        _require(t.dtype == torch.int32 and t.dim() == 2, f"{name} must be a 2D int32 tensor")
     _require(expert_offsets.dtype == torch.int32 and expert_offsets.dim() == 1, "expert_offsets must be a 1D int32 tensor")
     _require(output.dim() == 2, "output must be 2D tensor")
     _require(a.dim() == 2, "a must be 2D tensor")
     _require(b.dim() == 3, "b must be 3D tensor")
     _require(scales_a.dim() == 2, "scales_a must be 2D tensor")
     _require(scales_b.dim() == 3, "scales_b must be 3D tensor")
-    for t, name in ((a_ptrs, "a_ptrs"), (b_ptrs, "b_ptrs"), (out_ptrs, "out_ptrs"), (a_scales_ptrs, "a_scales_ptrs"),
-                    (b_scales_ptrs, "b_scales_ptrs"), (workspace, "workspace")):
-        _require(t.dim() == 1, f"{name} must be 1D tensor")
+    _require(workspace.dim() == 1, "workspace must be 1D tensor")
     _require(a.is_cuda and b.is_cuda and output.is_cuda and problem_sizes.is_cuda and expert_offsets.is_cuda,
              f"{op}: tensors must be CUDA tensors")
     total_m, K = a.shape
@@ -453,6 +443,33 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
         problem_sizes.data_ptr(), expert_offsets.data_ptr(), E, total_m, N, K, a.stride(0), b.stride(2), b.stride(0),
         scales_a.stride(0), scales_a.stride(1), scales_b.stride(0), scales_b.stride(2), scales_b.stride(1), output.stride(0),
         ws.data_ptr(), ws.numel() * ws.element_size(), _stream()))
+
+
+def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a, scales_b,
+                                    stride_a, stride_b, stride_c, layout_sfa, layout_sfb, problem_sizes, expert_offsets,
+                                    workspace):
+    """sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:650-810 (checks :668-706).  ``a`` [total_m, K] e4m3fn row-major,
+    ``b`` [E, K, N] e4m3fn column-major per expert (storage [E, N, K]), ``scales_a`` fp32 [total_m, K/128], ``scales_b``
+    fp32 [E, K/128, N/128] (storage [E, N/128, K/128]), ``problem_sizes`` int32 [E, 3] and ``expert_offsets`` int32 [E] on
+    the device, ``output`` [total_m, N] written in place.  The pointer, stride and scale-layout tensors are scratch of the
+    reference's kernels: they are type-checked like there and not used.  ``workspace`` is used when it is large enough
+    (the reference's callers pass hundreds of megabytes), otherwise a temporary one is allocated."""
+    for t, name in ((stride_a, "stride_a"), (stride_b, "stride_b"), (stride_c, "stride_c")):
+        _require(t.dtype == torch.int64 and t.dim() == 1, f"{name} must be a 1D int64 tensor")
+    for t, name in ((layout_sfa, "layout_sfa"), (layout_sfb, "layout_sfb")):
+        _require(t.dtype == torch.int32 and t.dim() == 2, f"{name} must be a 2D int32 tensor")
+    for t, name in ((a_ptrs, "a_ptrs"), (b_ptrs, "b_ptrs"), (out_ptrs, "out_ptrs"), (a_scales_ptrs, "a_scales_ptrs"),
+                    (b_scales_ptrs, "b_scales_ptrs")):
+        _require(t.dim() == 1, f"{name} must be 1D tensor")
+    _grouped_mm("fp8_blockwise_scaled_grouped_mm", output, a, b, scales_a, scales_b, problem_sizes, expert_offsets, workspace)
+
+
+def es_fp8_blockwise_scaled_grouped_mm(output, a, b, scales_a, scales_b, stride_a, stride_b, stride_d, problem_sizes,
+                                       expert_offsets, workspace):
+    """sgl-kernel/csrc/expert_specialization/es_fp8_blockwise.cu:33-170: the same computation on the same layouts without
+    the caller-provided scratch tensors.  The reference sorts experts into low / middle / high row counts and runs one
+    tile configuration on each; here the device-built schedule does that per tile (256-row tiles and a small-tile rest)."""
+    _grouped_mm("es_fp8_blockwise_scaled_grouped_mm", output, a, b, scales_a, scales_b, problem_sizes, expert_offsets, workspace)
 
 
 # ---------------------------------------------------------------- INT8 GEMM
@@ -546,6 +563,7 @@ def register() -> None:
         "sgl_per_token_quant_fp8": sgl_per_token_quant_fp8,
         "sgl_per_tensor_quant_fp8": sgl_per_tensor_quant_fp8,
         "fp8_blockwise_scaled_grouped_mm": fp8_blockwise_scaled_grouped_mm,
+        "es_fp8_blockwise_scaled_grouped_mm": es_fp8_blockwise_scaled_grouped_mm,
     }
     for name, fn in impls.items():
         if not hasattr(torch.ops.sgl_kernel, name):
@@ -561,6 +579,7 @@ def register() -> None:
     torch.library.register_fake("sgl_kernel::sgl_per_token_quant_fp8", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_tensor_quant_fp8", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::fp8_blockwise_scaled_grouped_mm", lambda *a: None, lib=_torch_lib)
+    torch.library.register_fake("sgl_kernel::es_fp8_blockwise_scaled_grouped_mm", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit", lambda *a: None, lib=_torch_lib)
     torch.library.register_fake("sgl_kernel::sgl_per_token_group_quant_8bit_v2", lambda *a: None, lib=_torch_lib)
     _registered = True

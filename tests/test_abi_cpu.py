@@ -83,6 +83,21 @@ def test_newer_entry_points_validate_before_any_device_work():
     assert L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(0, 128, 128) == 0
     need = L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(4, 512, 1024)
     assert need > 0 and need % 256 == 0
+    # grouped GEMM: output dtype, K whole blocks, workspace present and large enough, empty problem; queries are pure
+    G = L.mi355_fp8_blockwise_scaled_grouped_mm
+    tail = (128, 128, 128 * 128, 1, 1, 1, 1, 1, 128)  # lda, ldb, expert stride, scale strides, ldo
+    assert G(p, p, p, p, p, _lib.F32, p, p, 2, 8, 128, 128, *tail, p, 1 << 20, None) == 1
+    assert G(p, p, p, p, p, _lib.BF16, p, p, 2, 8, 128, 100, 100, 100, 12800, 1, 1, 1, 1, 1, 128, p, 1 << 20, None) == 2
+    assert G(p, p, p, p, p, _lib.BF16, None, p, 2, 8, 128, 128, *tail, p, 1 << 20, None) == 1
+    assert G(p, p, p, p, p, _lib.BF16, p, p, 2, 8, 128, 128, *tail, None, 0, None) == 4 and b"workspace" in L.mi355_last_error()
+    assert G(p, p, p, p, p, _lib.BF16, p, p, 2, 8, 128, 128, *tail, p, 16, None) == 4
+    assert G(None, None, None, None, None, _lib.BF16, None, None, 0, 0, 128, 128, *tail, None, 0, None) == 0
+    W = L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes
+    assert W(0, 8, 128, 128) == 0 and W(2, 8, 128, 128) % 256 == 0 and W(256, 32768, 512, 7168) > W(256, 256, 512, 7168) > 0
+    plan = _lib.grouped_gemm_plan(256, 32768, 512, 7168)
+    assert plan["small_tile"] == "128x256" and plan["max_big_tiles"] == 32768 // 129 and plan["max_small_tiles"] == 256
+    assert _lib.grouped_gemm_plan(256, 256, 512, 7168) == {
+        "kernel": "grouped_pingpong+grouped_dma3", "small_tile": "64x256", "max_big_tiles": 1, "max_small_tiles": 256, "tiles_n": 2}
 
 
 def test_operator_schemas_are_the_reference_ones():

@@ -143,6 +143,25 @@ def test_token_scales_in_either_layout(gpu, oracle):
     assert torch.equal(out_row, out_col)
 
 
+def test_expert_specialised_entry_point(gpu, oracle):
+    """es_fp8_blockwise_scaled_grouped_mm (sgl-kernel/tests/test_es_fp8_blockwise_moe.py:103-196): same layouts, no
+    scratch tensors in the argument list; same result as the other entry point, bit for bit."""
+    from sglang_amd.sgl_kernel import es_fp8_blockwise_scaled_grouped_mm
+
+    sizes = [200, 1, 77, 300, 0, 129]
+    E, N, K = len(sizes), 384, 768
+    a, w, sa, sw, offsets, T = _problem(sizes, N, K, 21)
+    out = torch.full((T, N), 7.0, dtype=torch.bfloat16, device=gpu)
+    strides = torch.full((E,), K, dtype=torch.int64, device=gpu)
+    es_fp8_blockwise_scaled_grouped_mm(
+        out, a.to(gpu), w.to(gpu).transpose(1, 2), sa.to(gpu), sw.to(gpu).transpose(1, 2), strides, strides,
+        torch.full((E,), N, dtype=torch.int64, device=gpu),
+        torch.tensor([[m, N, K] for m in sizes], dtype=torch.int32, device=gpu),
+        torch.tensor(offsets, dtype=torch.int32, device=gpu), torch.empty(16 << 20, dtype=torch.uint8, device=gpu))
+    _verify(oracle, out, a, w, sa, sw, sizes, offsets, "es")
+    assert torch.equal(out, _call(gpu, a, w, sa, sw, sizes, offsets, torch.bfloat16))
+
+
 def test_reference_acceptance_criterion(gpu):
     """sgl-kernel/tests/test_fp8_blockwise_moe.py:24-29, :205-216: quantize bf16 operands (1 x 128 groups, 128 x 128
     blocks), run the grouped GEMM, compare with the unquantized product: 1 - 2<x,y> / (<x,x> + <y,y>) < 1e-3."""

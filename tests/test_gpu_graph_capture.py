@@ -72,3 +72,61 @@ def test_capture_and_replay_matches_eager(gpu, oracle, M):
             ref, mag = oracle.fp8_blockwise_mm(q_o, w_q.cpu(), s_o, w_s.cpu(), torch.float32, want_abs=True)
             err = (got[2].float().cpu() - ref).abs()
             assert bool((err <= 1e-2 * ref.abs() + 1e-4 * mag).all())
+
+
+def test_grouped_gemm_replays_with_new_routing(gpu, oracle):
+    """The grouped FP8 GEMM inside a graph: problem sizes and expert offsets are device data, so a replay with a different
+    routing (other rows per expert, experts gaining and losing 256-row tiles) rebuilds its tile schedule on the device.
+    Each replay is compared with the eager call on the same data and the first one with the oracle."""
+    from sglang_amd.sgl_kernel import es_fp8_blockwise_scaled_grouped_mm
+
+    E, N, K, T = 6, 512, 1024, 900
+    g = torch.Generator().manual_seed(3)
+    a = ((torch.rand(T, K, generator=g) - 0.5) * 896).clamp(-448, 448).to(torch.float8_e4m3fn)
+    w = ((torch.rand(E, N, K, generator=g) - 0.5) * 896).clamp(-448, 448).to(torch.float8_e4m3fn)
+    sa = torch.rand(T, K // 128, generator=g) * 1e-2 + 1e-4
+    sw = torch.rand(E, N // 128, K // 128, generator=g) * 1e-2 + 1e-4
+    routings = [[150, 150, 150, 150, 150, 150], [700, 0, 1, 60, 139, 0], [0, 0, 0, 0, 0, 900], [3, 290, 7, 300, 44, 256]]
+    a_d, w_d, sa_d, sw_d = a.to(gpu), w.to(gpu).transpose(1, 2), sa.to(gpu), sw.to(gpu).transpose(1, 2)
+    strides = torch.full((E,), K, dtype=torch.int64, device=gpu)
+    ws = torch.empty(8 << 20, dtype=torch.uint8, device=gpu)
+
+    def tensors(sizes):
+        offs = [sum(sizes[:e]) for e in range(E)]
+        return (torch.tensor([[m, N, K] for m in sizes], dtype=torch.int32, device=gpu),
+                torch.tensor(offs, dtype=torch.int32, device=gpu), offs)
+
+    static_ps, static_eo, _ = tensors(routings[0])
+    static_out = torch.zeros(T, N, dtype=torch.bfloat16, device=gpu)
+
+    def run(out, ps, eo):
+        es_fp8_blockwise_scaled_grouped_mm(out, a_d, w_d, sa_d, sw_d, strides, strides, strides, ps, eo, ws)
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        run(static_out, static_ps, static_eo)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            run(static_out, static_ps, static_eo)
+    torch.cuda.synchronize()
+
+    for i, sizes in enumerate(routings[1:] + routings[:1]):
+        ps, eo, offs = tensors(sizes)
+        static_ps.copy_(ps)
+        static_eo.copy_(eo)
+        static_out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = static_out.clone()
+        want = torch.zeros_like(got)
+        run(want, ps, eo)  # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), (i, sizes)
+        if i == 0:
+            for e, (m, r0) in enumerate(zip(sizes, offs)):
+                if m:
+                    ref, mag = oracle.fp8_blockwise_mm(a[r0:r0 + m], w[e], sa[r0:r0 + m], sw[e], torch.float32, want_abs=True)
+                    err = (got[r0:r0 + m].float().cpu() - ref).abs()
+                    assert bool((err <= 1e-2 * ref.abs() + 1e-4 * mag + 2.0 ** -8 * ref.abs()).all()), e
