@@ -623,6 +623,9 @@ def main():
         if full:
             also.append(bench_fp8_ue8m0_gemm("gate_up", 4096, K, N, S, W))
             also.append(bench_silu_quant(S, W))
+            # expert GEMMs of DeepSeek-R1 (shapes of the reference's grouped-GEMM benchmark): prefill TP=8, prefill EP=16, decode EP=8
+            for E, rows, Kg, Ng in ((256, 128, 7168, 512), (16, 512, 7168, 4096), (32, 4, 7168, 4096)):
+                also.append(bench_fp8_grouped_gemm(E, rows, Kg, Ng, S, W))
             K, N = DSV3_MLP["down"]
             also.append(bench_fp8_gemm("down", 4096, K, N, S, W, False))
             for nm, (K, N) in DSV3_MLA.items():
