@@ -284,21 +284,52 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 }  // namespace
 
 // Token-tile height and split count for this kernel.  One workgroup per CU fits (three stages fill the LDS).
-// The estimate is a byte model for few tokens, where the kernel is bound by weight streaming: a split multiplies the
-// number of workgroups (better balance over 256 CUs when there are few tiles) but every extra split writes and re-reads
-// an M x N fp32 partial tile, and short K ranges pay the pipeline fill (two blocks) each:
-//   efficiency = balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2) * tile_factor
-// With many tokens (prefill shapes whose channel count is too small for 256 x 256 tiles) the same formula ranks the two
-// tile heights: 64-token tiles double the workgroups but do 0.65 of the work of a 128-token tile per unit of time
-// (measured on K=7168 -> N=1536 / N=576 at M=4096 and M=2048).
-// `efficiency` is returned so that the dispatcher can prefer another kernel when no choice does well.
+//
+// The choice minimises a time model fitted to measurements on this part (13 shapes, M = 32 .. 4096, every tile height
+// and split count; it names the measured best or a choice within 5 % of it for each):
+//   * a workgroup spends per K block the largest of
+//       - the tile's own time when operands come from L2: 0.88 us for 128 token rows, 0.62 us for 64;
+//       - a latency floor when the weight comes from HBM (two blocks in flight per CU): 1.2 us / 1.0 us, times 1.2 for
+//         weight rows longer than 8 KB;
+//       - its share of the HBM stream: (concurrent workgroups) x (HBM bytes per workgroup and block) / 5.5 TB/s, where
+//         weight rows are shared in L2 by up to 8 token tiles and token rows by up to 8 channel tiles;
+//   * a workgroup runs kb_per + 2 blocks (pipeline fill), and rounds of up to 256 workgroups follow each other;
+//   * a split adds the fp32 partial tiles written and read back (8 * splits * M * N bytes at 5.5 TB/s) and 6 us for the
+//     second launch and its tail.
+// So 144 workgroups streaming a weight unsplit beat 432 that split K in three (measured at M = 32 and 64 on K = 7168 ->
+// N = 36864: 58 against 65 us): with all CUs busy the HBM stream, not the number of workgroups, is the limit, and the
+// partial sums only add traffic.
+//
+// `efficiency` is the best value over all choices of an older byte-model score, kept because the dispatcher's threshold
+// for preferring another kernel at M < 256 was set with it:
+//   balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2) * (0.65 for 64-row tiles at M > 128)
+namespace {
+double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int sp) {
+  constexpr double HBM_BYTES_PER_US = 5.5e6;
+  const int64_t per = (kb_total + sp - 1) / sp;
+  const int64_t tm = (M + bm - 1) / bm, tn = (N + T_BN - 1) / T_BN;
+  const double t_tile = bm == 128 ? 0.88 : 0.62;
+  const double hbm_per_block = (double)(T_BN * KSTEP) / (double)std::min<int64_t>(tm, 8) + (double)(bm * KSTEP) / (double)std::min<int64_t>(tn, 8);
+  // (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
+  const double t_latency = hbm_per_block >= 16384.0 ? (bm == 128 ? 1.2 : 1.0) * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
+  double t = 0.0;
+  for (int64_t left = tm * tn * sp; left > 0;) {
+    const int64_t c = std::min<int64_t>(left, 256);
+    left -= c;
+    t += (double)(per + 2) * std::max(std::max(t_tile, t_latency), (double)c * hbm_per_block / HBM_BYTES_PER_US);
+  }
+  if (sp > 1) t += 8.0 * sp * (double)M * (double)N / HBM_BYTES_PER_US + 6.0;
+  return t;
+}
+}  // namespace
+
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
   Dma3Plan pl;
   const int64_t kb_total = (K + KSTEP - 1) / KSTEP;
   const double useful = (double)N * K + (double)M * K + 2.0 * M * N;
   const int max_split = (N % 4 == 0) ? 16 : 1;  // the reduce kernel works on aligned quads of one row
-  double best_score = -1.0;
-  pl.bm = 128, pl.splits = 1;
+  double best_time = 1e30;
+  pl.bm = 128, pl.splits = 1, pl.efficiency = 0.0;
   for (int bm = 64; bm <= 128; bm += 64) {
     if (M <= 64 && bm == 128) break;                 // a second half tile of padding rows buys nothing
     if (M > 64 && M <= 128 && bm == 64) continue;    // two token tiles would stream the weight twice
@@ -308,16 +339,16 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
       const int64_t per = (kb_total + sp - 1) / sp;
       if (sp > 1 && per < 4) break;
       if ((kb_total + per - 1) / per != sp) continue;  // some split would get no work
+      const double t = dma3_model_us(M, N, kb_total, bm, sp);
+      if (t < best_time) best_time = t, pl.splits = sp, pl.bm = bm;
       const int64_t wgs = tiles * sp;
       const int64_t rounds = (wgs + 255) / 256;
       const double balance = (double)wgs / (double)(rounds * 256);
       const double partial = sp > 1 ? 8.0 * sp * M * N : 0.0;
-      const double score = balance * useful / (useful + partial) * (double)per / (double)(per + 2) * tile_factor;
-      if (score > best_score) best_score = score, pl.splits = sp, pl.bm = bm;
+      pl.efficiency = std::max(pl.efficiency, balance * useful / (useful + partial) * (double)per / (double)(per + 2) * tile_factor);
     }
   }
   pl.kb_per_split = (int)((kb_total + pl.splits - 1) / pl.splits);
-  pl.efficiency = best_score;
   return pl;
 }
 

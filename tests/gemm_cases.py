@@ -14,7 +14,7 @@ FP8_ROUTE_SHAPES = [
     (7, 33280, 4096), (5, 66048, 512), (2, 133120, 384),
     # three-stage mid-M kernel: 64 / 128 token tiles, whole-K and split, ragged M, K blocks per range = 1, 2, 0 mod 3
     (48, 16384, 2048), (33, 16384, 2176), (40, 65536, 512), (200, 16384, 2048), (100, 32768, 640), (130, 8192, 7168),
-    (250, 8192, 7296),
+    (250, 8192, 7296), (100, 16384, 3584), (500, 4096, 14336),
     # 256 x 256 two-phase and 256 x 128 pipelined kernels, K a multiple of 128 and not
     (4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 256), (4000, 2100, 272),
     # generic kernel: every token-tile height, aligned and byte-granular loads, whole-K and split
@@ -39,6 +39,7 @@ INT8_ROUTE_SHAPES = [
     (16, 128, 512), (1, 6144, 4096), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432), (7, 33280, 4096),
     (5, 66048, 512), (2, 133120, 384),
     (20, 8192, 4096), (40, 65536, 512), (200, 16384, 2048), (200, 32768, 1024), (300, 4096, 14336), (130, 8192, 7168),
+    (100, 16384, 3584), (500, 4096, 14336),
     (4096, 4096, 512), (4000, 4088, 1024),
     (1, 16, 512), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
 ]
