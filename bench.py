@@ -566,7 +566,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU; it contains no collective, and a run with --gpus N>1 "
-              "is not provided (DESIGN.md, 'How the path would shard').", file=sys.stderr)
+              "is not provided (tokens shard by rows, weights by N or K, outside these kernels).", file=sys.stderr)
         sys.exit(2)
 
     import torch
