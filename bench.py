@@ -19,6 +19,7 @@ Infinity Cache.
   fp8_grouped:E:ROWS:K:N  grouped FP8 GEMM of E experts with ROWS token rows each (mixture-of-experts)
   copy         a plain 256 MiB device copy (calibration of the HBM traffic counters)
   silu_quant   silu(gate) * up fused in front of the group quantizer (packed UE8M0 scales)
+  per_token_fp8 / per_token_int8 / per_tensor_fp8 / block_cast   the other quantizers of the path
 
 Per-launch durations are HIP events on the launch stream (torch's current stream, which is the stream
 handed to the C ABI).  `roofline.achieved` = algorithmic FLOPs (2*M*N*K) or bytes per launch / MEDIAN
@@ -504,6 +505,56 @@ def bench_silu_quant(steps, warmup):
     }
 
 
+def bench_row_quant(kind, steps, warmup):
+    """The other activation / weight quantizers of the path on bf16 data, as HBM-bound kernels: per-token FP8 and INT8
+    (one scale per row), per-tensor FP8 (dynamic: absmax pass + quantize pass, the scale word cleared by a fill kernel in
+    between) and the 128 x 128 block cast of a weight to power-of-two scales.  Algorithmic bytes: every input element read
+    once (twice for the two-pass per-tensor quantizer), every code written once, plus the scales."""
+    import torch
+
+    from sglang_amd import _lib
+
+    dev = torch.device("cuda:0")
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(9)
+    nbuf = 3
+    if kind == "block_cast":
+        R, C = 36864, 7168
+        xs = [(torch.randn(R, C, generator=gen, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16) for _ in range(nbuf)]
+        qs = [torch.empty(R, C, dtype=torch.float8_e4m3fn, device=dev) for _ in range(nbuf)]
+        ss = [torch.empty(R // 128, C // 128, dtype=torch.float32, device=dev) for _ in range(nbuf)]
+        step = lambda i: _lib.check(L.mi355_block_cast_to_fp8(xs[i].data_ptr(), _lib.BF16, qs[i].data_ptr(), ss[i].data_ptr(), R, C, stream))
+        alg, name, kern = R * C * 3 + 4 * ss[0].numel(), f"block_cast_to_fp8 weight [{R}, {C}] bf16 -> e4m3fn, 128x128 power-of-two scales", "block_cast"
+    else:
+        from sglang_amd.workloads import make_activation
+
+        M, K = (16384, 4096) if kind == "per_token_int8" else (16384, 7168)
+        base = make_activation(M, K).to(dev)
+        xs = [base.clone() for _ in range(nbuf)]
+        qs = [torch.empty(M, K, dtype=torch.int8 if kind == "per_token_int8" else torch.float8_e4m3fn, device=dev) for _ in range(nbuf)]
+        if kind == "per_tensor_fp8":
+            ss = [torch.zeros(1, dtype=torch.float32, device=dev) for _ in range(nbuf)]
+
+            def step(i):
+                ss[i].zero_()  # the dynamic quantizer merges block maxima into the scale word: it starts from zero
+                _lib.check(L.mi355_per_tensor_quant_fp8(xs[i].data_ptr(), _lib.BF16, qs[i].data_ptr(), ss[i].data_ptr(), M * K, 0, None, 0, stream))
+            alg, kern = M * K * (2 + 2 + 1) + 4, "per_tensor_absmax + per_tensor_quant"
+        else:
+            ss = [torch.empty(M, 1, dtype=torch.float32, device=dev) for _ in range(nbuf)]
+            fn = L.mi355_per_token_quant_int8 if kind == "per_token_int8" else L.mi355_per_token_quant_fp8
+            step = lambda i: _lib.check(fn(xs[i].data_ptr(), _lib.BF16, qs[i].data_ptr(), ss[i].data_ptr(), M, K, stream))
+            alg, kern = M * K * 3 + 4 * M, "per_token_quant"
+        name = f"{kind}_quant M={M} K={K} bf16"
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms, b2b)
+    return {
+        "workload": name, "value": alg / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "f32 arithmetic, 8-bit out", "kernel": kern, "roofline": _roofline(0, alg, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
+    }
+
+
 def bench_copy(steps, warmup):
     """Plain device-to-device copy of a known size (256 MiB read + 256 MiB written per launch): the calibration
     workload for the FETCH_SIZE / WRITE_SIZE counters behind `roofline.traffic`."""
@@ -596,6 +647,8 @@ def main():
         rec = bench_copy(S, W)
     elif wl == "silu_quant":
         rec = bench_silu_quant(S, W)
+    elif wl in ("per_token_fp8", "per_token_int8", "per_tensor_fp8", "block_cast"):
+        rec = bench_row_quant(wl, S, W)
     elif wl == "fp8_decode":
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 1, K, N, S, W, cpu)
@@ -618,6 +671,7 @@ def main():
             # the bandwidth-bound quantizer is measured first: right after the MFMA-heavy GEMMs the chip's power state
             # makes a 60 us streaming kernel read ~15 % slow
             quant = [bench_quant(S, W, False, cpu), bench_quant(S, W, True, False)]
+            also += [bench_row_quant(k, S, W) for k in ("per_token_fp8", "per_token_int8", "per_tensor_fp8", "block_cast")]
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 4096, K, N, S, W, cpu)
         if full:
