@@ -8,6 +8,9 @@
 //         gives scale 0 and zeros, as in sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85.
 // Rows of up to 8192 two-byte elements stay in registers between the two phases; longer rows are
 // re-read (from L2).
+// Two-byte inputs with rows of at most 8192 elements (every hidden size of the benchmark models) take a second kernel: one
+// WAVE per row, four rows per workgroup, the row in registers (up to 16 x 16 bytes per lane), no LDS and no barrier -
+// 16384 workgroups of one short row each spend a visible share of their life starting up and at the barrier.
 #include "common.h"
 
 namespace mi355 {
@@ -50,6 +53,84 @@ __device__ __forceinline__ float wave_allreduce_max(float v) {
   return r;
 }
 
+// Scale of a row from its |x| maximum (written by the caller) and the factor the elements are multiplied with.
+template <bool FP8_OUT>
+__device__ __forceinline__ float row_scale(float amax, float& mul) {
+  if constexpr (FP8_OUT) {
+    const float scale = amax / 448.0f;
+    mul = (scale == 0.f) ? 0.f : 1.0f / scale;
+    return scale;
+  } else {
+    mul = 127.0f / amax;
+    return amax / 127.0f;
+  }
+}
+
+// One 16-byte vector of input -> 4 or 8 codes at d.
+template <int DT, bool FP8_OUT, bool STREAM>
+__device__ __forceinline__ void emit_vector(const u32x4& raw, float mul, int8_t* d) {
+  constexpr int VEC = (DT == MI355_F32) ? 4 : 8;
+  float f[VEC];
+  unpack16<DT>(raw, f);
+  uint32_t w[VEC / 4];
+#pragma unroll
+  for (int j = 0; j < VEC / 4; ++j) {
+    uint32_t pk = 0;
+    if constexpr (FP8_OUT) {
+      float t[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) t[b] = fmaxf(fminf(f[4 * j + b] * mul, 448.0f), -448.0f);
+      int c = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
+      c = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c, true);
+      pk = (uint32_t)c;
+    } else {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) pk |= ((uint32_t)(int)roundf(f[4 * j + b] * mul) & 0xffu) << (8 * b);
+    }
+    w[j] = pk;
+  }
+  if constexpr (VEC == 8) {
+    if constexpr (STREAM) __builtin_nontemporal_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(d));
+    else *reinterpret_cast<u32x2*>(d) = u32x2{w[0], w[1]};
+  } else {
+    *reinterpret_cast<uint32_t*>(d) = w[0];
+  }
+}
+
+// One wave per row, the row in registers: NV vectors of eight two-byte elements per lane (K <= 512 * NV).
+template <int DT, bool FP8_OUT, int NV>
+__global__ __launch_bounds__(256) void per_token_quant_wave_kernel(const void* x, int8_t* q, float* s, int64_t M, int64_t K) {
+  static_assert(DT != MI355_F32, "two-byte inputs");
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int nvec = (int)(K / 8);
+  const u32x4* src = reinterpret_cast<const u32x4*>(x) + row * nvec;
+  u32x4 keep[NV];
+  float amax = FP8_OUT ? 0.f : 1e-10f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + 64 * i;
+    keep[i] = (v < nvec) ? __builtin_nontemporal_load(src + v) : u32x4{0, 0, 0, 0};
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    float f[8];
+    unpack16<DT>(keep[i], f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
+  }
+  amax = wave_allreduce_max(amax);
+  float mul;
+  const float scale = row_scale<FP8_OUT>(amax, mul);
+  if (lane == 0) s[row] = scale;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + 64 * i;
+    if (v < nvec) emit_vector<DT, FP8_OUT, true>(keep[i], mul, q + row * K + (int64_t)v * 8);
+  }
+}
+
 template <int DT, bool FP8_OUT>
 __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int8_t* q, float* s, int64_t K) {
   constexpr int VEC = (DT == MI355_F32) ? 4 : 8;
@@ -80,41 +161,10 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int
   __syncthreads();
   amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
   float mul;
-  if constexpr (FP8_OUT) {
-    const float scale = amax / 448.0f;
-    if (threadIdx.x == 0) s[row] = scale;
-    mul = (scale == 0.f) ? 0.f : 1.0f / scale;
-  } else {
-    if (threadIdx.x == 0) s[row] = amax / 127.0f;
-    mul = 127.0f / amax;
-  }
+  const float scale = row_scale<FP8_OUT>(amax, mul);
+  if (threadIdx.x == 0) s[row] = scale;
 
-  auto emit = [&](const u32x4& raw, int64_t v) {
-    float f[VEC];
-    unpack16<DT>(raw, f);
-    uint32_t w[VEC / 4];
-#pragma unroll
-    for (int j = 0; j < VEC / 4; ++j) {
-      uint32_t pk = 0;
-      if constexpr (FP8_OUT) {
-        float t[4];
-#pragma unroll
-        for (int b = 0; b < 4; ++b) t[b] = fmaxf(fminf(f[4 * j + b] * mul, 448.0f), -448.0f);
-        int c = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
-        c = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c, true);
-        pk = (uint32_t)c;
-      } else {
-#pragma unroll
-        for (int b = 0; b < 4; ++b) pk |= ((uint32_t)(int)roundf(f[4 * j + b] * mul) & 0xffu) << (8 * b);
-      }
-      w[j] = pk;
-    }
-    int8_t* d = q + row * K + v * VEC;
-    if constexpr (VEC == 8)
-      *reinterpret_cast<u32x2*>(d) = u32x2{w[0], w[1]};
-    else
-      *reinterpret_cast<uint32_t*>(d) = w[0];
-  };
+  auto emit = [&](const u32x4& raw, int64_t v) { emit_vector<DT, FP8_OUT, false>(raw, mul, q + row * K + v * VEC); };
 #pragma unroll
   for (int i = 0; i < KEEP; ++i) {
     const int64_t v = threadIdx.x + 256 * i;
@@ -144,6 +194,23 @@ int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float
   MI355_REQUIRE(M < (1ll << 31), MI355_ERR_INVALID_ARGUMENT, "%s: too many rows", what);
   hipStream_t st = static_cast<hipStream_t>(stream);
   int8_t* qq = static_cast<int8_t*>(q);
+  if (x_dtype != MI355_F32 && K <= 8192) {  // one wave per row
+    const dim3 grid((unsigned)((M + 3) / 4));
+    const int nv = (int)((K / 8 + 63) / 64);
+#define MI355_WAVE_ROWS(DT, NV) \
+  hipLaunchKernelGGL((per_token_quant_wave_kernel<DT, FP8_OUT, NV>), grid, dim3(256), 0, st, x, qq, s, M, K)
+    if (x_dtype == MI355_BF16) {
+      if (nv <= 4) MI355_WAVE_ROWS(MI355_BF16, 4);
+      else if (nv <= 8) MI355_WAVE_ROWS(MI355_BF16, 8);
+      else MI355_WAVE_ROWS(MI355_BF16, 16);
+    } else {
+      if (nv <= 4) MI355_WAVE_ROWS(MI355_F16, 4);
+      else if (nv <= 8) MI355_WAVE_ROWS(MI355_F16, 8);
+      else MI355_WAVE_ROWS(MI355_F16, 16);
+    }
+#undef MI355_WAVE_ROWS
+    return check_launch(what);
+  }
   switch (x_dtype) {
     case MI355_F32:
       hipLaunchKernelGGL((per_token_quant_kernel<MI355_F32, FP8_OUT>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);

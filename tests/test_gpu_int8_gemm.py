@@ -117,7 +117,7 @@ def test_reference_test_distribution(gpu, oracle):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("M,K", [(1, 512), (7, 4096), (64, 14336), (33, 16384 + 512)])
+@pytest.mark.parametrize("M,K", [(1, 512), (7, 4096), (64, 14336), (33, 16384 + 512), (5, 8192), (6, 2056), (9, 8200)])
 def test_per_token_quant_int8(gpu, oracle, dtype, M, K):
     from sglang_amd.int8_kernel import per_token_quant_int8
     from sglang_amd.workloads import make_activation

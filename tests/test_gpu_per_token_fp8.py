@@ -12,7 +12,7 @@ FP8 = torch.float8_e4m3fn
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("M,K", [(1, 512), (7, 4096), (64, 7168), (33, 16384 + 512), (3, 8)])
+@pytest.mark.parametrize("M,K", [(1, 512), (7, 4096), (64, 7168), (33, 16384 + 512), (3, 8), (5, 8192), (6, 2056), (9, 8200)])
 def test_per_token_quant_fp8_bits(gpu, oracle, dtype, M, K):
     from sglang_amd.fp8_kernel import sglang_per_token_quant_fp8
 
