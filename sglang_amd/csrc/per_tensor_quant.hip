@@ -54,7 +54,20 @@ __global__ __launch_bounds__(256) void per_tensor_absmax_kernel(const void* x, f
   const int64_t nvec = n / VEC;
   const u32x4* src = reinterpret_cast<const u32x4*>(x);
   float m = 0.f;
-  for (int64_t v = gid; v < nvec; v += stride) {
+  int64_t v = gid;
+  for (; v + 3 * stride < nvec; v += 4 * stride) {  // four loads in flight per thread
+    u32x4 r[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) r[u] = src[v + u * stride];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float f[VEC];
+      unpack_vec<DT>(r[u], f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) m = fmaxf(m, fabsf(f[j]));
+    }
+  }
+  for (; v < nvec; v += stride) {
     float f[VEC];
     unpack_vec<DT>(src[v], f);
 #pragma unroll
@@ -84,9 +97,9 @@ __global__ __launch_bounds__(256) void per_tensor_quant_kernel(const void* x, ui
     for (int64_t r = gid; r < rows; r += stride) scale_rows[r] = s;
   const int64_t nvec = n / VEC;
   const u32x4* src = reinterpret_cast<const u32x4*>(x);
-  for (int64_t v = gid; v < nvec; v += stride) {
+  auto emit = [&](const u32x4& raw, int64_t v) {
     float f[VEC];
-    unpack_vec<DT>(src[v], f);
+    unpack_vec<DT>(raw, f);
     uint32_t w[VEC / 4];
 #pragma unroll
     for (int j = 0; j < VEC / 4; ++j) {
@@ -95,10 +108,19 @@ __global__ __launch_bounds__(256) void per_tensor_quant_kernel(const void* x, ui
       w[j] = (uint32_t)c;
     }
     if constexpr (VEC == 8)
-      *reinterpret_cast<u32x2*>(q + v * VEC) = u32x2{w[0], w[1]};
+      __builtin_nontemporal_store(u32x2{w[0], w[1]}, reinterpret_cast<u32x2*>(q + v * VEC));
     else
       *reinterpret_cast<uint32_t*>(q + v * VEC) = w[0];
+  };
+  int64_t v = gid;
+  for (; v + 3 * stride < nvec; v += 4 * stride) {  // four loads in flight per thread
+    u32x4 r[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) r[u] = __builtin_nontemporal_load(src + v + u * stride);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) emit(r[u], v + u * stride);
   }
+  for (; v < nvec; v += stride) emit(src[v], v);
   for (int64_t i = nvec * VEC + gid; i < n; i += stride) {
     const float t = clamp448(elem_f32<DT>(x, i) * inv);
     q[i] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(t, t, 0, false) & 0xff);
