@@ -16,6 +16,7 @@ Infinity Cache.
   fp8_decode   FP8 gate_up at M=1          int8_gemm             INT8 gate_up (K=4096 -> N=28672) at M=4096
   fp8:M:K:N    any blockwise-FP8 linear    int8:M:K:N            any INT8 linear
   fp8_ue8m0:M:K:N  the same linear with power-of-two (UE8M0) scales on both operands
+  fp8_linear:M:K:N  a whole block-FP8 linear, bf16 in -> bf16 out, one call (fp8_linear2: quantizer call + GEMM call)
   fp8_grouped:E:ROWS:K:N  grouped FP8 GEMM of E experts with ROWS token rows each (mixture-of-experts)
   copy         a plain 256 MiB device copy (calibration of the HBM traffic counters)
   silu_quant   silu(gate) * up fused in front of the group quantizer (packed UE8M0 scales)
@@ -400,6 +401,58 @@ def bench_fp8_grouped_gemm(E, m_per, K, N, steps, warmup):
     }
 
 
+def bench_fp8_linear(M, K, N, steps, warmup, two_step):
+    """A whole block-FP8 linear from bf16 activations to bf16 output: the one-call entry point (at decode sizes the GEMM
+    kernel quantizes in its prologue), or, with two_step, quantizer call + GEMM call as the reference's wrappers do."""
+    import torch
+
+    from sglang_amd import _lib
+    from sglang_amd.workloads import fp8_gemm_algorithmic_bytes, gemm_flops, make_activation
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(N * 10007 + K)
+    nbuf = max(2, min(6, int(600e6 // (N * K)) + 1))
+    ws = [device_block_fp8_weight(N, K, gen, dev) for _ in range(nbuf)]
+    x = make_activation(M, K).to(dev)
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+    kb = K // 128
+    if two_step:
+        q = torch.empty(M, K, dtype=torch.float8_e4m3fn, device=dev)
+        pitch = (M + 3) // 4 * 4
+        sa = torch.empty(kb, pitch, dtype=torch.float32, device=dev)
+        wsb = L.mi355_fp8_blockwise_mm_workspace_bytes(M, N, K)
+        wsbuf = torch.empty(max(wsb, 256), dtype=torch.uint8, device=dev)
+
+        def step(i):
+            _lib.check(L.mi355_group_quant_8bit(x.data_ptr(), _lib.BF16, q.data_ptr(), _lib.FP8_E4M3FN, sa.data_ptr(), M, K, 128, 1e-10,
+                                                -448.0, 448.0, _lib.QUANT_DIV, _lib.SCALE_F32, 0.0, 1, pitch, stream))
+            _lib.check(L.mi355_fp8_blockwise_mm(q.data_ptr(), ws[i][0].data_ptr(), sa.data_ptr(), ws[i][1].data_ptr(), outs[i].data_ptr(),
+                                                _lib.BF16, M, N, K, K, K, 1, pitch, ws[i][1].stride(0), ws[i][1].stride(1), N,
+                                                wsbuf.data_ptr(), wsb, stream))
+    else:
+        wsb = L.mi355_fp8_block_linear_workspace_bytes(M, N, K)
+        wsbuf = torch.empty(max(wsb, 256), dtype=torch.uint8, device=dev)
+
+        def step(i):
+            _lib.check(L.mi355_fp8_block_linear(x.data_ptr(), _lib.BF16, ws[i][0].data_ptr(), ws[i][1].data_ptr(), ws[i][1].stride(0),
+                                                ws[i][1].stride(1), None, outs[i].data_ptr(), _lib.BF16, M, N, K, K, N,
+                                                wsbuf.data_ptr(), wsb, stream))
+
+    wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
+    st = _stats(ms, b2b)
+    flops, nbytes = gemm_flops(M, N, K), fp8_gemm_algorithmic_bytes(M, N, K) + M * K
+    plan = _lib.gemm_plan("fp8", M, N, K)
+    return {
+        "workload": f"fp8_linear{'_two_step' if two_step else ''} M={M} K={K} N={N} (bf16 in, 1x128 quantization, blockwise GEMM, bf16 out)",
+        "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "fp8(e4m3fn) MFMA, f32 accumulate", "kernel": ("quantizer + " if two_step or plan["kernel"] != "decode" else "") + plan["kernel"],
+        "roofline": _roofline(flops, nbytes, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
+    }
+
+
 def bench_int8_gemm(name, M, K, N, steps, warmup, with_cpu=False):
     import torch
 
@@ -658,6 +711,9 @@ def main():
     elif wl.startswith("fp8_ue8m0:"):
         _, M, K, N = wl.split(":")
         rec = bench_fp8_ue8m0_gemm("shape", int(M), int(K), int(N), S, W)
+    elif wl.startswith("fp8_linear:") or wl.startswith("fp8_linear2:"):
+        kind, M, K, N = wl.split(":")
+        rec = bench_fp8_linear(int(M), int(K), int(N), S, W, kind == "fp8_linear2")
     elif wl.startswith("fp8_grouped:"):
         _, E, m_per, K, N = wl.split(":")
         rec = bench_fp8_grouped_gemm(int(E), int(m_per), int(K), int(N), S, W)

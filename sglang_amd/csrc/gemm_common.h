@@ -25,6 +25,9 @@ struct GemmParams {
   const void* bias;        // optional [N] in the output dtype (INT8 GEMM; per-channel FP8 epilogue)
   const float* col_scale;  // FP8 only, optional [N]: per-channel scale applied in the epilogue (fp8_scaled_mm)
   const float* row_scale;  // FP8 two-phase kernel in its epilogue-scaled mode only: per-token scale [M]
+  const void* x16;         // FP8 decode kernel only, optional: unquantized tokens [M, K] (x_dtype, row stride ldx elements);
+  int64_t ldx;             // when set, the kernel quantizes them per 1 x 128 group itself and ignores a / sa
+  int x_dtype;
   void* out;
   void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
   int M, N, K;

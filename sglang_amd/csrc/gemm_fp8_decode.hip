@@ -41,6 +41,7 @@ __shared__ __attribute__((aligned(1024))) uint8_t r_stage1[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_stage2[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_stage3[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_tok[KB_PER * TOK_BLOCK];
+__shared__ float r_sa[KB_PER * 16];  // token scales of the range when the kernel quantizes the tokens itself
 
 // 16 zero bytes in global memory: the source of token chunks that lie past the end of K (short last range), so that
 // whatever weight block is refetched there multiplies zeros.  Not const: it must share the operands' address space.
@@ -132,9 +133,75 @@ __device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* sta
   }
 }
 
+// max over the 16 lanes of a DPP row
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
+  return v;
+}
+
+// QUANT (FP8 only): the tokens come unquantized (p.x16, bf16 or fp16) and the workgroup quantizes the 16 x KB_PER groups of
+// its K range itself, straight into the token stage, with the arithmetic of the group quantizer's reference path
+// (amax floored at 1e-10, s = amax / 448, q = e4m3fn(clamp(x / s)), group_quant.hip) - so a linear layer at decode sizes
+// is this kernel plus the reduce, without a quantizer launch in front.  16 lanes per group (8 elements each), one token
+// per 16 lanes, one K block per step; codes go where the direct-to-LDS copy would have put them.
+template <int KBP>
+__device__ __forceinline__ void load_raw_tokens(const GemmParams& p, int kb_begin, u32x4 (&raw)[KBP]) {
+  const int gl = threadIdx.x & 15, m = threadIdx.x >> 4;
+  if (m >= p.M) return;  // token rows past M are never stored: whatever the stage holds there will do
+  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(p.x16) + (int64_t)m * p.ldx + gl * 8;
+#pragma unroll
+  for (int d = 0; d < KBP; ++d)
+    raw[d] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)min(kb_begin + d, p.kb_total - 1) * KSTEP);
+}
+// x / s, correctly rounded, given r = RN(1 / s): two Markstein steps, as in the group quantizer (group_quant.hip), where
+// the conditions under which this equals the `/` operator are stated and checked.
+__device__ __forceinline__ float div_by_shared(float x, float s, float r) {
+  float q = x * r;
+  q = fmaf(fmaf(-q, s, x), r, q);
+  q = fmaf(fmaf(-q, s, x), r, q);
+  return q;
+}
+template <int KBP>
+__device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begin, const u32x4 (&raw)[KBP], uint8_t* tok,
+                                                float* sa_lds) {
+  const int gl = threadIdx.x & 15, m = threadIdx.x >> 4;
+  if (m >= p.M) return;
+#pragma unroll
+  for (int d = 0; d < KBP; ++d) {
+    const uint32_t w[4] = {raw[d].x, raw[d].y, raw[d].z, raw[d].w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = p.x_dtype == MI355_BF16 ? __uint_as_float(w[i] << 16) : f16_bits_to_f32(w[i] & 0xffffu);
+      v[2 * i + 1] = p.x_dtype == MI355_BF16 ? __uint_as_float(w[i] & 0xffff0000u) : f16_bits_to_f32(w[i] >> 16);
+    }
+    float amax = 1e-10f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    amax = row16_max(amax);
+    const float sc = amax / 448.0f;
+    const float rcp = 1.0f / sc;
+    float t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = fminf(fmaxf(div_by_shared(v[j], sc, rcp), -448.0f), 448.0f);
+    int c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
+    c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c0, true);
+    int c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], 0, false);
+    c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], c1, true);
+    const bool valid = kb_begin + d < p.kb_total;  // blocks past the end of K: zero tokens, zero scale
+    *reinterpret_cast<u32x2*>(tok + d * TOK_BLOCK + m * KSTEP + (((gl >> 1) ^ (m & 7)) << 4) + (gl & 1) * 8) =
+        valid ? u32x2{(uint32_t)c0, (uint32_t)c1} : u32x2{0u, 0u};
+    if (gl == 0) sa_lds[d * 16 + m] = valid ? sc : 0.f;
+  }
+}
+
 // SPLIT: raw partial sums to the workspace (more than one K range).
-template <bool IS_FP8, bool SPLIT>
+template <bool IS_FP8, bool SPLIT, bool QUANT = false>
 __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, int groups_per_wg, int wg_per_split) {
+  static_assert(IS_FP8 || !QUANT, "the fused quantizer belongs to the FP8 path");
   using AccT = typename std::conditional<IS_FP8, float, int>::type;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -170,21 +237,31 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
   for (int h = 0; h < 2; ++h) s.tk_off[h] = l16 * KSTEP + (((q + 4 * h) ^ (l16 & 7)) << 4);
 
   // ---- start the weight ring, then stage the tokens of this K range (all waves share them)
+  u32x4 raw_tok[QUANT ? KB_PER : 1];
+  if constexpr (QUANT) load_raw_tokens<KB_PER>(p, kb_begin, raw_tok);  // requested first: they are needed first
   issue_weights<false>(s, r_stage0, 0);
   issue_weights<false>(s, r_stage1, 1);
   issue_weights<false>(s, r_stage2, 2);
+  if constexpr (QUANT) {
+    quantize_tokens<KB_PER>(p, kb_begin, raw_tok, r_tok, r_sa);
+  } else {
 #pragma unroll
-  for (int e = 0; e < 2 * KB_PER / WAVES; ++e) {  // 16 instructions of 8 rows x 128 B, 4 per wave
-    const int inst = wave * (2 * KB_PER / WAVES) + e;
-    const int d = inst >> 1, half = inst & 1;
-    const int m = min(half * 8 + lrow, p.M - 1);           // rows past M repeat the last token, never stored
-    const uint8_t* src = p.a + (int64_t)m * p.lda + (int64_t)(kb_begin + d) * KSTEP + logical * 16;
-    if (kb_begin + d >= p.kb_total) src = reinterpret_cast<const uint8_t*>(r_zero16);  // blocks past K: zeros
-    __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(r_tok + d * TOK_BLOCK + half * 1024), 16, 0, 0);
+    for (int e = 0; e < 2 * KB_PER / WAVES; ++e) {  // 16 instructions of 8 rows x 128 B, 4 per wave
+      const int inst = wave * (2 * KB_PER / WAVES) + e;
+      const int d = inst >> 1, half = inst & 1;
+      const int m = min(half * 8 + lrow, p.M - 1);           // rows past M repeat the last token, never stored
+      const uint8_t* src = p.a + (int64_t)m * p.lda + (int64_t)(kb_begin + d) * KSTEP + logical * 16;
+      if (kb_begin + d >= p.kb_total) src = reinterpret_cast<const uint8_t*>(r_zero16);  // blocks past K: zeros
+      __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(r_tok + d * TOK_BLOCK + half * 1024), 16, 0, 0);
+    }
   }
   // FP8: token scales of the range (blocks past the end of K multiply zero tokens; their scale is set to zero too)
   float sa_r[KB_PER];
-  if constexpr (IS_FP8) {
+  if constexpr (QUANT) {
+    __syncthreads();  // codes and scales of the range are in LDS
+#pragma unroll
+    for (int d = 0; d < KB_PER; ++d) sa_r[d] = r_sa[d * 16 + l16];
+  } else if constexpr (IS_FP8) {
     const float* sa_row = p.sa + (int64_t)min(l16, p.M - 1) * p.sa_sm;
 #pragma unroll
     for (int d = 0; d < KB_PER; ++d) {
@@ -195,7 +272,7 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
 #pragma unroll
     for (int d = 0; d < KB_PER; ++d) sa_r[d] = 0.f;
   }
-  __syncthreads();  // the only barrier: tokens are in LDS
+  if constexpr (!QUANT) __syncthreads();  // the only barrier: tokens are in LDS
 
   const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
   // FP8 weight-block scales: one per K block and 128-channel group; fetched one group ahead so that using them never
@@ -315,6 +392,15 @@ static int launch_decode(GemmParams& p, int gpw, hipStream_t stream, const char*
   p.tiles_m = 1;
   p.tiles_n = groups_n;
   const dim3 grid((unsigned)(wg_per_split * p.splits));
+  if constexpr (IS_FP8) {
+    if (p.x16 != nullptr) {  // tokens arrive unquantized
+      if (p.splits > 1)
+        hipLaunchKernelGGL((decode_kernel<true, true, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+      else
+        hipLaunchKernelGGL((decode_kernel<true, false, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+      return check_launch(what);
+    }
+  }
   if (p.splits > 1)
     hipLaunchKernelGGL((decode_kernel<IS_FP8, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
   else

@@ -879,6 +879,18 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
   float* sa = reinterpret_cast<float*>(q + q_bytes);
   const int64_t pitch = (M + 3) & ~3ll;
   const size_t sa_bytes = align256((size_t)pitch * (size_t)(K / KSTEP) * 4u);
+  // Decode sizes: the GEMM kernel quantizes the tokens of each K range itself (same arithmetic), no quantizer launch.
+  if (x_dtype != MI355_F32 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && ldw % 16 == 0 &&
+      choose_route(true, M, N, K, K, ldw, true).kernel == RK_DECODE) {
+    GemmParams p;
+    bool empty;
+    // a / sa are not read by the kernel in this mode; they only have to satisfy the checks
+    int rc = fp8_mm_params(what, x, w, w_scale, w_scale, out, out_dtype, M, N, K, K, ldw, 1, (M + 3) & ~3ll, ws_sn, ws_sk, ldo, p, empty);
+    if (rc != MI355_OK || empty) return rc;
+    p.bias = bias;
+    p.x16 = x, p.ldx = K, p.x_dtype = x_dtype;
+    return run_gemm<true>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
+  }
   // quantize with q = x / s, the arithmetic of the reference's column-major path (fp8_kernel.py:164-212 via fp8_utils.py:201-203)
   int rc = mi355_group_quant_8bit(x, x_dtype, q, MI355_FP8_E4M3FN, sa, M, K, KSTEP, 1e-10f, -448.0f, 448.0f, MI355_QUANT_DIV,
                                   MI355_SCALE_F32, 0.0f, 1, pitch, stream);

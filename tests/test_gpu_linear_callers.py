@@ -35,6 +35,32 @@ def test_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
         assert bool(torch.isfinite(out).all())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (3, 16640, 4480), (8, 7168, 18432), (16, 512, 512), (5, 66048, 512), (9, 256, 128)])
+def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype):
+    """At decode sizes the one-call linear has no quantizer launch: the GEMM kernel quantizes the tokens of each K range
+    in its prologue.  Same arithmetic on the same codes and scales as quantizer + GEMM in two steps, so the outputs must
+    be identical bit for bit (split and unsplit plans, several channel groups per workgroup, a short last K range, rows
+    past M); the two-step path is held to the oracle elsewhere, and once more here."""
+    from sglang_amd import _lib
+    from sglang_amd.fp8_kernel import per_token_group_quant_fp8
+    from sglang_amd.fp8_utils import w8a8_block_fp8_linear
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    assert _lib.gemm_plan("fp8", M, N, K)["kernel"] == "decode"
+    x = make_activation(M, K, seed=M + N, dtype=dtype)
+    x[0, :128] = 0  # a group of zeros: scale 1e-10 / 448, codes 0
+    w_q, w_s = make_fp8_weight(N, K, seed=K)
+    xg, wg, sg = x.to(gpu), w_q.to(gpu), w_s.to(gpu)
+    fused = w8a8_block_fp8_linear(xg, wg, [128, 128], sg)
+    q, s = per_token_group_quant_fp8(xg, 128, column_major_scales=True)
+    two_step = fp8_blockwise_scaled_mm(q, wg.t(), s, sg.t(), dtype)
+    assert fused.dtype == dtype and torch.equal(fused.view(torch.int16), two_step.view(torch.int16))
+    xq, xs = oracle.group_quant(x, 128, mode="div")
+    ref, mag = oracle.fp8_blockwise_mm(xq, w_q, xs, w_s, torch.float32, want_abs=True)
+    assert bool(((fused.float().cpu() - ref).abs() <= 1e-2 * ref.abs() + 1e-4 * mag).all())
+
+
 def test_block_fp8_linear_ragged_k_falls_back(gpu, oracle):
     """K not a multiple of 128 cannot be group-quantized; N ragged is fine."""
     from sglang_amd.fp8_utils import w8a8_block_fp8_linear
