@@ -288,7 +288,9 @@ int mi355_fp8_scaled_mm(const void* a, const void* b, const float* sa, const flo
  *          (python/sglang/srt/layers/quantization/fp8_utils.py:184-214, :281-301): per_token_group_quant_fp8, the blockwise
  *          GEMM and `output += bias`.  The activation is quantized with q = x / s (s = max(amax, 1e-10) / 448) into the
  *          workspace, with M-major scales, and the bias is added in fp32 in the GEMM epilogue (the reference adds it
- *          after rounding the GEMM result to the output type).
+ *          after rounding the GEMM result to the output type).  At decode sizes (M <= 16, 16-bit x, N % 128 == 0) there
+ *          is no quantizer launch: the GEMM kernel quantizes the tokens of its K range in its prologue, with the same
+ *          arithmetic, and the result is bit-identical to the two-step sequence.
  *   x [M, K] contiguous F32/F16/BF16, K % 128 == 0; w [N, K] e4m3fn row stride ldw; w_scale element (nb, kb) at
  *   w_scale[nb * ws_sn + kb * ws_sk]; bias NULL or [N] in the output dtype; out [M, N] BF16/F16 row stride ldo.
  *   workspace: mi355_fp8_block_linear_workspace_bytes(M, N, K) bytes, 256-byte aligned.
