@@ -121,7 +121,9 @@ GroupedPlan grouped_plan(int64_t E, int64_t total_m, int64_t K) {
   pl.max_big = (int)(total_m / 129);    // every 256-row tile covers more than 128 rows
   // an expert leaves at most 128 rows to small tiles, and every small tile covers at least one row
   pl.max_small = (int)std::min<int64_t>(total_m, E * (128 / pl.bm));
-  pl.pitch = ((total_m + 3) & ~3ll) + 4 * E;
+  // the last expert's column is at most align4(total_m) - rows + 4 (E - 1) + 3, and the GEMM reads whole quads up to
+  // align4(rows) past it: one more quad of slack keeps that inside the row (and inside the workspace for the last row)
+  pl.pitch = ((total_m + 3) & ~3ll) + 4 * E + 4;
   pl.big_bytes = align256((size_t)(pl.max_big + 1) * sizeof(v4i));  // record 0 holds the count
   pl.small_bytes = align256((size_t)(pl.max_small + 1) * sizeof(v4i));
   pl.scale_bytes = align256((size_t)pl.pitch * (size_t)((K + KSTEP - 1) / KSTEP) * 4u);
