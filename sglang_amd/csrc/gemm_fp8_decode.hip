@@ -145,16 +145,20 @@ __device__ __forceinline__ float row16_max(float v) {
 // QUANT (FP8 only): the tokens come unquantized (p.x16, bf16 or fp16) and the workgroup quantizes the 16 x KB_PER groups of
 // its K range itself, straight into the token stage, with the arithmetic of the group quantizer's reference path
 // (amax floored at 1e-10, s = amax / 448, q = e4m3fn(clamp(x / s)), group_quant.hip) - so a linear layer at decode sizes
-// is this kernel plus the reduce, without a quantizer launch in front.  16 lanes per group (8 elements each), one token
-// per 16 lanes, one K block per step; codes go where the direct-to-LDS copy would have put them.
+// is this kernel plus the reduce, without a quantizer launch in front.  16 lanes per group (8 elements each); codes go
+// where the direct-to-LDS copy would have put them.
 template <int KBP>
 __device__ __forceinline__ void load_raw_tokens(const GemmParams& p, int kb_begin, u32x4 (&raw)[KBP]) {
-  const int gl = threadIdx.x & 15, m = threadIdx.x >> 4;
-  if (m >= p.M) return;  // token rows past M are never stored: whatever the stage holds there will do
-  const uint16_t* xrow = reinterpret_cast<const uint16_t*>(p.x16) + (int64_t)m * p.ldx + gl * 8;
+  // (token, K block) pairs are dealt to the sixteen 16-lane rows of the workgroup, pair r + 16 j to row r: with one token
+  // the eight groups are quantized by eight rows at once instead of one row doing them one after the other
+  const int gl = threadIdx.x & 15, r = threadIdx.x >> 4;
 #pragma unroll
-  for (int d = 0; d < KBP; ++d)
-    raw[d] = *reinterpret_cast<const u32x4*>(xrow + (int64_t)min(kb_begin + d, p.kb_total - 1) * KSTEP);
+  for (int j = 0; j < KBP; ++j) {
+    const int pair = r + 16 * j, m = pair / KBP, d = pair % KBP;
+    if (m < p.M)  // token rows past M are never stored: whatever the stage holds there will do
+      raw[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.x16) + (int64_t)m * p.ldx +
+                                               (int64_t)min(kb_begin + d, p.kb_total - 1) * KSTEP + gl * 8);
+  }
 }
 // x / s, correctly rounded, given r = RN(1 / s): two Markstein steps, as in the group quantizer (group_quant.hip), where
 // the conditions under which this equals the `/` operator are stated and checked.
@@ -167,11 +171,12 @@ __device__ __forceinline__ float div_by_shared(float x, float s, float r) {
 template <int KBP>
 __device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begin, const u32x4 (&raw)[KBP], uint8_t* tok,
                                                 float* sa_lds) {
-  const int gl = threadIdx.x & 15, m = threadIdx.x >> 4;
-  if (m >= p.M) return;
+  const int gl = threadIdx.x & 15, r = threadIdx.x >> 4;
 #pragma unroll
-  for (int d = 0; d < KBP; ++d) {
-    const uint32_t w[4] = {raw[d].x, raw[d].y, raw[d].z, raw[d].w};
+  for (int j = 0; j < KBP; ++j) {
+    const int pair = r + 16 * j, m = pair / KBP, d = pair % KBP;
+    if (m >= p.M) break;  // uniform over the 16-lane row, which is all the DPP reduction below involves
+    const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
     float v[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -180,13 +185,13 @@ __device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begi
     }
     float amax = 1e-10f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(v[j]));
+    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
     amax = row16_max(amax);
     const float sc = amax / 448.0f;
     const float rcp = 1.0f / sc;
     float t[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) t[j] = fminf(fmaxf(div_by_shared(v[j], sc, rcp), -448.0f), 448.0f);
+    for (int e = 0; e < 8; ++e) t[e] = fminf(fmaxf(div_by_shared(v[e], sc, rcp), -448.0f), 448.0f);
     int c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
     c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c0, true);
     int c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], 0, false);
