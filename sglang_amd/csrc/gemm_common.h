@@ -172,8 +172,9 @@ int launch_fp8_pp_rowcol(GemmParams& p, hipStream_t stream, const char* what);
 struct Dma3Plan {
   int bm, splits, kb_per_split;
   double efficiency;  // modelled fraction of the streaming time that is useful (balance, partial sums, pipeline fill)
+  double time_us;     // modelled duration of the chosen plan
 };
-Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K);
+Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8 = false);
 int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);   // bm: 64 or 128, from dma3_plan()
 
 // Grouped problems on the tile bodies of the dense kernels: token rows of all experts stacked in one matrix, one weight

@@ -285,16 +285,17 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 
 // Token-tile height and split count for this kernel.  One workgroup per CU fits (three stages fill the LDS).
 //
-// The choice minimises a time model fitted to measurements on this part (13 shapes, M = 32 .. 4096, every tile height
-// and split count; it names the measured best or a choice within 5 % of it for each):
+// The choice minimises a time model fitted to measurements on this part (24 shapes, M = 32 .. 4096, every tile height
+// and split count; it names the measured best or a choice within 5 % of it for 22 of them, within 12 % for the others):
 //   * a workgroup spends per K block the largest of
-//       - the tile's own time when operands come from L2: 0.88 us for 128 token rows, 0.62 us for 64;
+//       - the tile's own time when operands come from L2: 0.88 us for 128 token rows, 0.58 us for 64 (x 1.2 in a round
+//         that keeps more than 200 CUs busy, x 1.3 for the INT8 kernel);
 //       - a latency floor when the weight comes from HBM (two blocks in flight per CU): 1.2 us / 1.0 us, times 1.2 for
 //         weight rows longer than 8 KB;
 //       - its share of the HBM stream: (concurrent workgroups) x (HBM bytes per workgroup and block) / 5.5 TB/s, where
 //         weight rows are shared in L2 by up to 8 token tiles and token rows by up to 8 channel tiles;
 //   * a workgroup runs kb_per + 2 blocks (pipeline fill), and rounds of up to 256 workgroups follow each other;
-//   * a split adds the fp32 partial tiles written and read back (8 * splits * M * N bytes at 5.5 TB/s) and 6 us for the
+//   * a split adds the fp32 partial tiles written and read back (8 * splits * M * N bytes at 5.5 TB/s) and 10 us for the
 //     second launch and its tail.
 // So 144 workgroups streaming a weight unsplit beat 432 that split K in three (measured at M = 32 and 64 on K = 7168 ->
 // N = 36864: 58 against 65 us): with all CUs busy the HBM stream, not the number of workgroups, is the limit, and the
@@ -304,11 +305,12 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 // for preferring another kernel at M < 256 was set with it:
 //   balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2) * (0.65 for 64-row tiles at M > 128)
 namespace {
-double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int sp) {
+double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int sp, bool is_int8) {
   constexpr double HBM_BYTES_PER_US = 5.5e6;
   const int64_t per = (kb_total + sp - 1) / sp;
   const int64_t tm = (M + bm - 1) / bm, tn = (N + T_BN - 1) / T_BN;
-  const double t_tile = bm == 128 ? 0.88 : 0.62;
+  // (the INT8 kernel of the same structure is 1.3x slower per block: measured on K=4096 -> N=28672 at M = 512 .. 1024)
+  const double t_tile = (bm == 128 ? 0.88 : 0.58) * (is_int8 ? 1.3 : 1.0);
   const double hbm_per_block = (double)(T_BN * KSTEP) / (double)std::min<int64_t>(tm, 8) + (double)(bm * KSTEP) / (double)std::min<int64_t>(tn, 8);
   // (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
   const double t_latency = hbm_per_block >= 16384.0 ? (bm == 128 ? 1.2 : 1.0) * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
@@ -316,14 +318,16 @@ double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int sp) {
   for (int64_t left = tm * tn * sp; left > 0;) {
     const int64_t c = std::min<int64_t>(left, 256);
     left -= c;
-    t += (double)(per + 2) * std::max(std::max(t_tile, t_latency), (double)c * hbm_per_block / HBM_BYTES_PER_US);
+    // with (nearly) every CU multiplying, the clock drops: 1.2x on the tile's own time (measured on multi-round shapes)
+    const double t_own = t_tile * (c > 200 ? 1.2 : 1.0);
+    t += (double)(per + 2) * std::max(std::max(t_own, t_latency), (double)c * hbm_per_block / HBM_BYTES_PER_US);
   }
-  if (sp > 1) t += 8.0 * sp * (double)M * (double)N / HBM_BYTES_PER_US + 6.0;
+  if (sp > 1) t += 8.0 * sp * (double)M * (double)N / HBM_BYTES_PER_US + 10.0;
   return t;
 }
 }  // namespace
 
-Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
+Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8) {
   Dma3Plan pl;
   const int64_t kb_total = (K + KSTEP - 1) / KSTEP;
   const double useful = (double)N * K + (double)M * K + 2.0 * M * N;
@@ -339,7 +343,7 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
       const int64_t per = (kb_total + sp - 1) / sp;
       if (sp > 1 && per < 4) break;
       if ((kb_total + per - 1) / per != sp) continue;  // some split would get no work
-      const double t = dma3_model_us(M, N, kb_total, bm, sp);
+      const double t = dma3_model_us(M, N, kb_total, bm, sp, is_int8);
       if (t < best_time) best_time = t, pl.splits = sp, pl.bm = bm;
       const int64_t wgs = tiles * sp;
       const int64_t rounds = (wgs + 255) / 256;
@@ -349,6 +353,7 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K) {
     }
   }
   pl.kb_per_split = (int)((kb_total + pl.splits - 1) / pl.splits);
+  pl.time_us = best_time;
   return pl;
 }
 

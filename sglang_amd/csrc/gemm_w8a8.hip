@@ -359,7 +359,7 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
   const Plan pl = make_plan(M, N, K);
   size_t need = pl.splits > 1 ? (size_t)pl.splits * (size_t)M * (size_t)N * 4u : 0;
   if (M > 16 && K % KSTEP == 0) {
-    const Dma3Plan dp = dma3_plan(M, N, K);  // (an upper bound: the dispatcher may still pick another kernel)
+    const Dma3Plan dp = dma3_plan(M, N, K, !is_fp8);  // (an upper bound: the dispatcher may still pick another kernel)
     const size_t dneed = dp.splits > 1 ? (size_t)dp.splits * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
   }
@@ -437,7 +437,18 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
     // tiles, when its tiling fills the chip well enough
     // Between 256 and 1024 tokens it beats the generic kernel even where its tiling fills the chip badly (measured on K=4096..7168 ->
     // N=1536..6144: 25 us against 35..63 us); below that the generic kernel's small tiles win for few channels.
-    const Dma3Plan dp = dma3_plan(M, N, K);
+    const Dma3Plan dp = dma3_plan(M, N, K, !is_fp8);
+    // Between 129 and 1024 tokens the two-phase 256 x 256 kernel competes: a round of its tiles takes (K blocks) x 1.39 us
+    // + 11 us (INT8: 1.46 us per block), whatever part of the tile is filled and however many CUs the round uses, so it
+    // wins where the channels alone give it a round's worth of tiles (measured: K=7168 -> N=36864 at M=256: 89 against
+    // 141 us, M=1024: 260 against 308 us; INT8 K=4096 -> N=28672 at M=512: 59 against 94 us) and loses for few channels.
+    if (M > 128 && M <= 1024 && (is_fp8 || K % KSTEP == 0)) {
+      const double pp_us = (double)((tiles_256 + NUM_CUS - 1) / NUM_CUS) * ((double)(K / KSTEP) * (is_fp8 ? 1.39 : 1.46) + 11.0);
+      if (pp_us < dp.time_us) {
+        r.kernel = RK_PINGPONG, r.bm = 256, r.bn = 256, r.splits = 1, r.kb_per_split = (int)(K / KSTEP);
+        return r;
+      }
+    }
     if ((M >= 256 && M <= 1024) || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
       r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = 256, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
       return r;
