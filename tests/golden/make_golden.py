@@ -66,6 +66,59 @@ def main():
     path = os.path.join(HERE, "qlinear_golden.npz")
     np.savez_compressed(path, **out)
     print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
+    write_more()
+
+
+def write_more():
+    """qlinear_golden_more.npz: the quantizers and GEMMs around the first three (per-token and per-tensor FP8, silu * up
+    in front of the group quantizer, weight block cast, per-token x per-channel FP8 GEMM, grouped GEMM)."""
+    out = {}
+    g = torch.Generator().manual_seed(31)
+    x = make_activation(9, 384, seed=77, outlier_frac=0.01)
+    x[3] = 0
+    out["x_bf16"] = bits(x)
+    q, s = oracle.per_token_quant_fp8(x)
+    out["ptq_fp8_q"], out["ptq_fp8_s_f32"] = bits(q), bits(s)
+    q, s = oracle.per_tensor_quant_fp8(x)
+    out["pt_dyn_q"], out["pt_dyn_s_f32"] = bits(q), bits(s)
+    given = torch.tensor([0.0371], dtype=torch.float32)
+    q, _ = oracle.per_tensor_quant_fp8(x, given)
+    out["pt_static_scale_f32"], out["pt_static_q"] = bits(given), bits(q)
+    # silu(gate) * up, then the v2 group quantizer with packed power-of-two scales: [7, 2 x 256]
+    gu = make_activation(7, 512, seed=78, outlier_frac=0.02)
+    v = oracle.silu_mul(gu)
+    q, s = oracle.group_quant(v, 128, mode="mul", layout="ue8m0")
+    out["silu_in_bf16"], out["silu_v_bf16"], out["silu_q"] = bits(gu), bits(v), bits(q)
+    out["silu_bytes"] = oracle.unpack_ue8m0(s, 2).numpy()
+    # 128 x 128 block cast of a weight [130, 200] and its inverse
+    w = (torch.randn(130, 200, generator=g) * 0.02).to(torch.bfloat16)
+    wq, ws = oracle.block_cast_to_fp8(w)
+    out["cast_w_bf16"], out["cast_q"], out["cast_s_f32"] = bits(w), bits(wq), bits(ws)
+    out["cast_back_bf16"] = bits(oracle.block_dequant_fp8(wq, ws, torch.bfloat16))
+    # per-token x per-channel FP8 GEMM with bias: M=9, N=72, K=384
+    aq, asc = oracle.per_token_quant_fp8(x)
+    bq = ((torch.rand(72, 384, generator=g) - 0.5) * 200).to(torch.float8_e4m3fn)
+    sb = torch.rand(72, generator=g) * 1e-2 + 1e-3
+    bias = torch.randn(72, generator=g).to(torch.bfloat16)
+    out["smm_w_q"], out["smm_sb_f32"], out["smm_bias_bf16"] = bits(bq), bits(sb), bits(bias)
+    out["smm_out_f32"] = bits(oracle.fp8_scaled_mm(aq, bq, asc.reshape(-1), sb, torch.float32, None))
+    # grouped GEMM: 3 experts with 5, 0 and 4 of 9 rows, N=128, K=256
+    xg = make_activation(9, 256, seed=79)
+    gq, gs = oracle.group_quant(xg, 128, mode="div")
+    ew = ((torch.rand(3, 128, 256, generator=g) - 0.5) * 200).to(torch.float8_e4m3fn)
+    es = torch.rand(3, 1, 2, generator=g) * 1e-2 + 1e-3
+    rows = [(0, 5), (5, 0), (5, 4)]
+    ref = torch.zeros(9, 128)
+    for e, (r0, m) in enumerate(rows):
+        if m:
+            ref[r0:r0 + m] = oracle.fp8_blockwise_mm(gq[r0:r0 + m], ew[e], gs[r0:r0 + m], es[e], torch.float32)
+    out["grp_a_q"], out["grp_a_s_f32"], out["grp_w_q"], out["grp_w_s_f32"] = bits(gq), bits(gs), bits(ew), bits(es)
+    out["grp_sizes"] = np.array([[m, 128, 256] for _, m in rows], dtype=np.int32)
+    out["grp_offsets"] = np.array([r0 for r0, _ in rows], dtype=np.int32)
+    out["grp_out_f32"] = bits(ref)
+    path = os.path.join(HERE, "qlinear_golden_more.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes,", len(out), "arrays")
 
 
 if __name__ == "__main__":

@@ -95,3 +95,82 @@ def test_gpu_reproduces_gemm_fixtures(gpu, gold):
     out = int8_scaled_mm(a, w.t(), _f32(gold["int8_sa_f32"]).to(gpu), _f32(gold["int8_sb_f32"]).to(gpu), torch.bfloat16,
                          _bf16(gold["int8_bias_bf16"]).to(gpu))
     assert torch.equal(out.cpu().view(torch.int16), gold["int8_out_bf16"])
+
+
+# ---- the quantizers and GEMMs around the first three (tests/golden/qlinear_golden_more.npz)
+
+MORE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "qlinear_golden_more.npz")
+
+
+@pytest.fixture(scope="module")
+def more():
+    z = np.load(MORE, allow_pickle=False)
+    return {k: torch.from_numpy(z[k].copy()) for k in z.files}
+
+
+def test_oracle_reproduces_the_other_fixtures(oracle, more):
+    x = _bf16(more["x_bf16"])
+    q, s = oracle.per_token_quant_fp8(x)
+    assert torch.equal(q.view(torch.uint8), more["ptq_fp8_q"]) and torch.equal(s.view(torch.int32), more["ptq_fp8_s_f32"])
+    q, s = oracle.per_tensor_quant_fp8(x)
+    assert torch.equal(q.view(torch.uint8), more["pt_dyn_q"]) and torch.equal(s.view(torch.int32), more["pt_dyn_s_f32"])
+    q, _ = oracle.per_tensor_quant_fp8(x, _f32(more["pt_static_scale_f32"]))
+    assert torch.equal(q.view(torch.uint8), more["pt_static_q"])
+    v = oracle.silu_mul(_bf16(more["silu_in_bf16"]))
+    assert torch.equal(v.view(torch.int16), more["silu_v_bf16"])
+    q, s = oracle.group_quant(v, 128, mode="mul", layout="ue8m0")
+    assert torch.equal(q.view(torch.uint8), more["silu_q"]) and torch.equal(oracle.unpack_ue8m0(s, 2), more["silu_bytes"])
+    wq, ws = oracle.block_cast_to_fp8(_bf16(more["cast_w_bf16"]))
+    assert torch.equal(wq.view(torch.uint8), more["cast_q"]) and torch.equal(ws.view(torch.int32), more["cast_s_f32"])
+    assert torch.equal(oracle.block_dequant_fp8(wq, ws, torch.bfloat16).view(torch.int16), more["cast_back_bf16"])
+    out = oracle.fp8_scaled_mm(more["ptq_fp8_q"].view(FP8), more["smm_w_q"].view(FP8), _f32(more["ptq_fp8_s_f32"]).reshape(-1),
+                               _f32(more["smm_sb_f32"]), torch.float32, None)
+    assert torch.equal(out.view(torch.int32), more["smm_out_f32"])
+    gq, gs = more["grp_a_q"].view(FP8), _f32(more["grp_a_s_f32"])
+    for e, (r0, m) in enumerate(zip(more["grp_offsets"].tolist(), more["grp_sizes"][:, 0].tolist())):
+        if m:
+            ref = oracle.fp8_blockwise_mm(gq[r0:r0 + m], more["grp_w_q"].view(FP8)[e], gs[r0:r0 + m], _f32(more["grp_w_s_f32"])[e],
+                                          torch.float32)
+            assert torch.equal(ref.view(torch.int32), more["grp_out_f32"][r0:r0 + m])
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_the_other_fixtures(gpu, more):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, sglang_per_token_quant_fp8
+    from sglang_amd.fp8_utils import block_quant_dequant, per_block_cast_to_fp8
+    from sglang_amd.sgl_kernel import es_fp8_blockwise_scaled_grouped_mm, fp8_scaled_mm, sgl_per_tensor_quant_fp8
+
+    x = _bf16(more["x_bf16"]).to(gpu)
+    q, s = sglang_per_token_quant_fp8(x)
+    assert torch.equal(q.cpu().view(torch.uint8), more["ptq_fp8_q"]) and torch.equal(s.cpu().view(torch.int32), more["ptq_fp8_s_f32"])
+    q = torch.empty_like(x, dtype=FP8)
+    s = torch.zeros(1, dtype=torch.float32, device=gpu)
+    sgl_per_tensor_quant_fp8(x, q, s, False)
+    assert torch.equal(q.cpu().view(torch.uint8), more["pt_dyn_q"]) and torch.equal(s.cpu().view(torch.int32), more["pt_dyn_s_f32"])
+    sgl_per_tensor_quant_fp8(x, q, _f32(more["pt_static_scale_f32"]).to(gpu), True)
+    assert torch.equal(q.cpu().view(torch.uint8), more["pt_static_q"])
+    q, s = sglang_per_token_group_quant_fp8(_bf16(more["silu_in_bf16"]).to(gpu), 128, column_major_scales=True, scale_tma_aligned=True,
+                                            scale_ue8m0=True, fuse_silu_and_mul=True, enable_v2=True)
+    assert torch.equal(q.cpu().view(torch.uint8), more["silu_q"])
+    dense = torch.empty(tuple(s.shape), dtype=torch.int32)
+    dense.copy_(s.cpu())
+    assert torch.equal(dense.view(torch.uint8).reshape(s.shape[0], -1)[:, :2], more["silu_bytes"])
+    wq, ws = per_block_cast_to_fp8(_bf16(more["cast_w_bf16"]).to(gpu))
+    assert torch.equal(wq.cpu().view(torch.uint8), more["cast_q"]) and torch.equal(ws.cpu().view(torch.int32), more["cast_s_f32"])
+    back = block_quant_dequant(wq, ws, [128, 128], torch.bfloat16)
+    assert torch.equal(back.cpu().view(torch.int16), more["cast_back_bf16"])
+    # floating point: |err| <= 1e-2 |ref| + 1e-4 * (sum of |terms|), bounded here by the largest |ref| of the matrix
+    ref = _f32(more["smm_out_f32"])
+    out = fp8_scaled_mm(more["ptq_fp8_q"].view(FP8).to(gpu), more["smm_w_q"].view(FP8).to(gpu).t(), _f32(more["ptq_fp8_s_f32"]).to(gpu),
+                        _f32(more["smm_sb_f32"]).to(gpu), torch.bfloat16, None).float().cpu()
+    assert bool(((out - ref).abs() <= 1e-2 * ref.abs() + 2.0 ** -8 * ref.abs() + 1e-4 * ref.abs().max()).all())
+    E, T, N, K = 3, 9, 128, 256
+    outg = torch.full((T, N), 7.0, dtype=torch.bfloat16, device=gpu)
+    strides = torch.full((E,), K, dtype=torch.int64, device=gpu)
+    es_fp8_blockwise_scaled_grouped_mm(
+        outg, more["grp_a_q"].view(FP8).to(gpu), more["grp_w_q"].view(FP8).to(gpu).transpose(1, 2), _f32(more["grp_a_s_f32"]).to(gpu),
+        _f32(more["grp_w_s_f32"]).to(gpu).transpose(1, 2), strides, strides, strides, more["grp_sizes"].to(gpu),
+        more["grp_offsets"].to(gpu), torch.empty(1 << 20, dtype=torch.uint8, device=gpu))
+    ref = _f32(more["grp_out_f32"])
+    got = outg.float().cpu()
+    assert bool(((got - ref).abs() <= 1e-2 * ref.abs() + 2.0 ** -8 * ref.abs() + 1e-4 * ref.abs().max()).all())
