@@ -60,3 +60,65 @@ def test_workspace_covers_the_plan(kind, M, N, K):
     p = plan_for(kind, M, N, K)
     ws = (L.mi355_fp8_blockwise_mm_workspace_bytes if kind == "fp8" else L.mi355_int8_scaled_mm_workspace_bytes)(M, N, K)
     assert ws >= (p["splits"] * M * N * 4 if p["splits"] > 1 else 0)
+
+
+def test_grouped_plan_bounds_hold_for_any_routing():
+    """The grouped GEMM sizes its tile tables and grids on the host from (experts, stacked rows) alone, while the real
+    tile counts come from row counts that only exist on the device.  Replay the device rule here (256-row tiles; a rest of
+    129..255 rows is one more; a rest of 1..128 rows becomes small tiles of the height the plan names) for random and
+    adversarial routings: the host bounds must never be exceeded."""
+    import random
+
+    from sglang_amd import _lib
+
+    rnd = random.Random(7)
+    cases = []
+    for _ in range(300):
+        E = rnd.choice([1, 2, 3, 8, 16, 64, 256, 300])
+        kind = rnd.choice(["uniform", "skewed", "tiny", "edges"])
+        if kind == "uniform":
+            sizes = [rnd.randint(0, 600) for _ in range(E)]
+        elif kind == "skewed":
+            sizes = [rnd.choice([0, 0, 1, 2, 5000]) for _ in range(E)]
+        elif kind == "tiny":
+            sizes = [rnd.randint(0, 3) for _ in range(E)]
+        else:
+            sizes = [rnd.choice([1, 63, 64, 65, 127, 128, 129, 255, 256, 257, 384, 385]) for _ in range(E)]
+        cases.append(sizes)
+    cases += [[128] * 256, [129] * 256, [1] * 256, [64] * 300, [65] * 300, [385] * 16, [0] * 8 + [1]]
+    for sizes in cases:
+        E, total = len(sizes), sum(sizes)
+        if total == 0:
+            continue
+        plan = _lib.grouped_gemm_plan(E, total, 512, 1024)
+        bm = int(plan["small_tile"].split("x")[0])
+        big = small = 0
+        for rows in sizes:
+            b, rest = divmod(rows, 256)
+            if rest > 128:
+                b += 1
+            else:
+                small += -(-rest // bm)
+            big += b
+        assert big <= plan["max_big_tiles"], (sizes[:8], big, plan)
+        assert small <= plan["max_small_tiles"], (sizes[:8], small, plan)
+        # the re-laid-out scale columns: expert e starts at align4(row0) + 4 e and is read in whole quads
+        pitch = (total + 3) // 4 * 4 + 4 * E + 4
+        row0 = 0
+        for e, rows in enumerate(sizes):
+            if rows:
+                assert (row0 + 3) // 4 * 4 + 4 * e + (rows + 3) // 4 * 4 <= pitch
+            row0 += rows
+
+
+def test_mid_m_plans_are_consistent():
+    """Whatever the time model picks, a split must give every K range some work and the ranges must cover K."""
+    from sglang_amd import _lib
+
+    for kind in ("fp8", "int8"):
+        for M in (17, 32, 64, 65, 128, 129, 200, 256, 300, 512, 1000, 1024, 1025, 4096):
+            for N, K in ((576, 7168), (1536, 7168), (7168, 18432), (36864, 7168), (6144, 4096), (4096, 14336), (256, 128), (512, 16384)):
+                p = _lib.gemm_plan(kind, M, N, K)
+                kb = -(-K // 128)
+                assert p["splits"] >= 1 and p["kb_per_split"] >= 1
+                assert p["kb_per_split"] * p["splits"] >= kb and p["kb_per_split"] * (p["splits"] - 1) < kb, (kind, M, N, K, p)
