@@ -23,7 +23,7 @@ namespace mi355 {
 namespace {
 
 constexpr int T_THREADS = 512;
-constexpr int T_BN = 256, T_WN = 64, T_NT = T_WN / 16;
+constexpr int T_BN = 256;  // widest channel tile (sizes the LDS stages); the kernels take BN = 128 or 256
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
@@ -48,9 +48,9 @@ __device__ __forceinline__ u32x4 lds16(lds_cptr p, int imm) {
   return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(p + imm);
 }
 
-template <int BM>
+template <int BM, int BN>
 struct Dma3State {
-  static constexpr int LOADS = (BM + T_BN) / 64;  // tile loads per wave and stage (a wave fills 8 rows per load)
+  static constexpr int LOADS = (BM + BN) / 64;  // tile loads per wave and stage (a wave fills 8 rows per load)
   const uint8_t* a_base;
   const uint8_t* b_base;
   uint32_t goff[LOADS];   // lane's byte offset from the matrix base (rows clamped); first BM/64 loads are token rows
@@ -65,9 +65,9 @@ struct Dma3State {
 // Load number i (< LOADS: tile rows; == LOADS: token scales) of K block kb, written as instructions.
 // The statements write m0; it cannot be listed as a clobber (the compiler reserves the register and rejects the entry), and
 // no compiler-managed use of m0 lies between them and the next statement that sets it.
-template <int BM>
-__device__ __forceinline__ void issue_one(const Dma3State<BM>& s, int i, uint8_t* stage, float* scale, int kb) {
-  constexpr int LOADS = Dma3State<BM>::LOADS;
+template <int BM, int BN>
+__device__ __forceinline__ void issue_one(const Dma3State<BM, BN>& s, int i, uint8_t* stage, float* scale, int kb) {
+  constexpr int LOADS = Dma3State<BM, BN>::LOADS;
   kb = min(kb, s.kb_last);
   if (i < LOADS) {
     const uint8_t* base = (i < BM / 64 ? s.a_base : s.b_base) + (uint64_t)kb * KSTEP;  // wave-uniform
@@ -91,10 +91,10 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM>& s, int i, uint8_t
 }
 
 // One K block out of `cur`; the loads of block kb_next go out over the first LOADS + 1 steps into `nxt`.
-template <int BM>
-__device__ __forceinline__ void k_block(const Dma3State<BM>& s, const uint8_t* cur, const float* sc_cur, float sbv,
-                                        float (&acc)[T_NT][BM / 32][4], uint8_t* nxt, float* sc_nxt, int kb_next) {
-  constexpr int MT = BM / 32, LOADS = Dma3State<BM>::LOADS;
+template <int BM, int BN>
+__device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_t* cur, const float* sc_cur, float sbv,
+                                        float (&acc)[BN / 64][BM / 32][4], uint8_t* nxt, float* sc_nxt, int kb_next) {
+  constexpr int MT = BM / 32, T_NT = BN / 64, LOADS = Dma3State<BM, BN>::LOADS;  // a wave owns BN / 4 channels = T_NT tiles of 16
   static_assert(LOADS + 1 <= MT * T_NT, "one load per step");
   Frag w[T_NT], tokb[2];
   float scb[2];
@@ -111,12 +111,12 @@ __device__ __forceinline__ void k_block(const Dma3State<BM>& s, const uint8_t* c
   v4f part[2];
 #pragma unroll
   for (int t = 0; t < MT * T_NT; ++t) {
-    const int j = t >> 2, i = t & 3;
+    const int j = t / T_NT, i = t % T_NT;
     part[t & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w[i]), as_v8i(tokb[j & 1]),
                                                                    v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first; the rest of the step runs in its shadow
     if (t > 0) {
-      const int pj = (t - 1) >> 2, pi = (t - 1) & 3;
+      const int pj = (t - 1) / T_NT, pi = (t - 1) % T_NT;
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[(t - 1) & 1][v], scb[pj & 1], acc[pi][pj][v]);
     }
@@ -129,12 +129,12 @@ __device__ __forceinline__ void k_block(const Dma3State<BM>& s, const uint8_t* c
       tokb[(j + 1) & 1].hi = lds16(tk1, (j + 1) * 2048);
     }
     if (i == 1 && j + 1 < MT) scb[(j + 1) & 1] = scp[(j + 1) * 16] * sbv;
-    if (t <= LOADS) issue_one<BM>(s, t, nxt, sc_nxt, kb_next);
+    if (t <= LOADS) issue_one<BM, BN>(s, t, nxt, sc_nxt, kb_next);
     __builtin_amdgcn_sched_barrier(0);
   }
   {
     constexpr int t = MT * T_NT - 1;
-    constexpr int pj = t >> 2, pi = t & 3;
+    constexpr int pj = t / T_NT, pi = t % T_NT;
 #pragma unroll
     for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[t & 1][v], scb[pj & 1], acc[pi][pj][v]);
   }
@@ -143,15 +143,18 @@ __device__ __forceinline__ void k_block(const Dma3State<BM>& s, const uint8_t* c
 // Everything but the youngest block's loads has landed; then the workgroup barrier.  Instructions, see the file comment.
 template <int YOUNGER>
 __device__ __forceinline__ void wait_and_barrier() {
-  static_assert(YOUNGER == 6 || YOUNGER == 7, "LOADS + 1 for BM = 64 / 128");
+  static_assert(YOUNGER >= 4 && YOUNGER <= 7, "LOADS + 1 = (BM + BN) / 64 + 1");
   if constexpr (YOUNGER == 7) asm volatile("s_waitcnt vmcnt(7)\n\ts_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
+  else if constexpr (YOUNGER == 6) asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
+  else if constexpr (YOUNGER == 5) asm volatile("s_waitcnt vmcnt(5)\n\ts_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
 }
 
 // One BM x 256 output tile at (m0, n0), K blocks of split `split`, by the whole workgroup.
-template <int BM, bool SPLIT>
+template <int BM, bool SPLIT, int BN = T_BN>
 __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, int split) {
-  constexpr int WM = BM / 2, MT = WM / 16, LOADS = Dma3State<BM>::LOADS;
+  static_assert(BN == 128 || BN == 256, "channel tile");
+  constexpr int WM = BM / 2, MT = WM / 16, T_WN = BN / 4, T_NT = T_WN / 16, LOADS = Dma3State<BM, BN>::LOADS;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -162,7 +165,7 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
   const int nkb = kb_end - kb_begin;
 
-  Dma3State<BM> s;
+  Dma3State<BM, BN> s;
   s.wave = wave;
   s.kb_last = kb_end - 1;
   s.a_base = p.a;
@@ -203,9 +206,9 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
 
   // ---- prologue: blocks 0 and 1 (clamped) into stages 0 and 1
 #pragma unroll
-  for (int i = 0; i <= LOADS; ++i) issue_one<BM>(s, i, t_stage0, t_scale0, kb_begin);
+  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN>(s, i, t_stage0, t_scale0, kb_begin);
 #pragma unroll
-  for (int i = 0; i <= LOADS; ++i) issue_one<BM>(s, i, t_stage1, t_scale1, kb_begin + 1);
+  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN>(s, i, t_stage1, t_scale1, kb_begin + 1);
   wait_and_barrier<LOADS + 1>();  // block 0 has landed everywhere
 
   // ---- three blocks per trip over the three stages; iteration k multiplies block k, requests block k + 2
@@ -214,18 +217,18 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
     const float sb0 = s.sb_ptr[(int64_t)(kb_begin + k) * s.sb_sk];
     const float sb1 = s.sb_ptr[(int64_t)(kb_begin + k + 1) * s.sb_sk];
     const float sb2 = s.sb_ptr[(int64_t)(kb_begin + k + 2) * s.sb_sk];
-    k_block<BM>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2);
+    k_block<BM, BN>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2);
     wait_and_barrier<LOADS + 1>();
-    k_block<BM>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3);
+    k_block<BM, BN>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3);
     wait_and_barrier<LOADS + 1>();
-    k_block<BM>(s, t_stage2, t_scale2, sb2, acc, t_stage1, t_scale1, kb_begin + k + 4);
+    k_block<BM, BN>(s, t_stage2, t_scale2, sb2, acc, t_stage1, t_scale1, kb_begin + k + 4);
     wait_and_barrier<LOADS + 1>();
   }
   if (k < nkb) {  // one or two blocks left, in stages 0 and 1
-    k_block<BM>(s, t_stage0, t_scale0, s.sb_ptr[(int64_t)(kb_begin + k) * s.sb_sk], acc, t_stage2, t_scale2, kb_begin + k + 2);
+    k_block<BM, BN>(s, t_stage0, t_scale0, s.sb_ptr[(int64_t)(kb_begin + k) * s.sb_sk], acc, t_stage2, t_scale2, kb_begin + k + 2);
     wait_and_barrier<LOADS + 1>();
     if (k + 1 < nkb)
-      k_block<BM>(s, t_stage1, t_scale1, s.sb_ptr[(int64_t)(kb_begin + k + 1) * s.sb_sk], acc, t_stage0, t_scale0, kb_begin + k + 3);
+      k_block<BM, BN>(s, t_stage1, t_scale1, s.sb_ptr[(int64_t)(kb_begin + k + 1) * s.sb_sk], acc, t_stage0, t_scale0, kb_begin + k + 3);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
 
@@ -253,10 +256,10 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   }
 }
 
-template <int BM, bool SPLIT>
+template <int BM, bool SPLIT, int BN>
 __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmParams p) {
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
-  dma3_tile<BM, SPLIT>(p, tc.tile_m * BM, tc.tile_n * T_BN, tc.split);
+  dma3_tile<BM, SPLIT, BN>(p, tc.tile_m * BM, tc.tile_n * BN, tc.split);
 }
 
 // Grouped problems (see GroupedParams): the workgroup's token tile comes from the table the plan kernel wrote, the
@@ -269,29 +272,33 @@ __global__ __launch_bounds__(T_THREADS) void fp8_grouped_dma3_kernel(const Group
   dma3_tile<BM, false>(p, m0, tile_n * T_BN, 0);
 }
 
-template <int BM>
+template <int BM, int BN>
 int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + BM - 1) / BM;
-  p.tiles_n = (p.N + T_BN - 1) / T_BN;
+  p.tiles_n = (p.N + BN - 1) / BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits));
   if (p.splits > 1)
-    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true>), grid, dim3(T_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN>), grid, dim3(T_THREADS), 0, stream, p);
   else
-    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false>), grid, dim3(T_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN>), grid, dim3(T_THREADS), 0, stream, p);
   return check_launch(what);
 }
 
 }  // namespace
 
-// Token-tile height and split count for this kernel.  One workgroup per CU fits (three stages fill the LDS).
+// Tile shape (64 or 128 tokens x 256 or 128 channels) and split count for this kernel.  One workgroup per CU fits (the
+// LDS stages are sized for the widest tile).  Narrow channel tiles do half the multiplications of a block in 0.6 of the
+// time, but they double the workgroups without a K split, i.e. without fp32 partial sums: they win for few channels and
+// long K (K=18432 -> N=7168 at M=128: 52.7 -> 46.7 us; K=7168 -> N=4096 at M=512: 34.4 -> 24.5 us; N=576 at M=4096:
+// 35.7 -> 31.0 us) and lose where 256-channel tiles already give a round's worth of workgroups.
 //
 // The choice minimises a time model fitted to measurements on this part (24 shapes, M = 32 .. 4096, every tile height
 // and split count; it names the measured best or a choice within 5 % of it for 22 of them, within 12 % for the others):
 //   * a workgroup spends per K block the largest of
-//       - the tile's own time when operands come from L2: 0.88 us for 128 token rows, 0.58 us for 64 (x 1.2 in a round
-//         that keeps more than 200 CUs busy, x 1.3 for the INT8 kernel);
-//       - a latency floor when the weight comes from HBM (two blocks in flight per CU): 1.2 us / 1.0 us, times 1.2 for
-//         weight rows longer than 8 KB;
+//       - the tile's own time when operands come from L2: 0.88 us for 128 token rows, 0.58 us for 64 (0.52 / 0.40 with
+//         128 channels; x 1.2 in a round that keeps more than 200 CUs busy, x 1.3 for the INT8 kernel);
+//       - a latency floor when the weight comes from HBM (two blocks in flight per CU): 1.2 us / 1.0 us (0.7 / 0.51 with
+//         128 channels), times 1.2 for weight rows longer than 8 KB;
 //       - its share of the HBM stream: (concurrent workgroups) x (HBM bytes per workgroup and block) / 5.5 TB/s, where
 //         weight rows are shared in L2 by up to 8 token tiles and token rows by up to 8 channel tiles;
 //   * a workgroup runs kb_per + 2 blocks (pipeline fill), and rounds of up to 256 workgroups follow each other;
@@ -305,15 +312,17 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 // for preferring another kernel at M < 256 was set with it:
 //   balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2) * (0.65 for 64-row tiles at M > 128)
 namespace {
-double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int sp, bool is_int8) {
+double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int bn, int sp, bool is_int8) {
   constexpr double HBM_BYTES_PER_US = 5.5e6;
   const int64_t per = (kb_total + sp - 1) / sp;
-  const int64_t tm = (M + bm - 1) / bm, tn = (N + T_BN - 1) / T_BN;
-  // (the INT8 kernel of the same structure is 1.3x slower per block: measured on K=4096 -> N=28672 at M = 512 .. 1024)
-  const double t_tile = (bm == 128 ? 0.88 : 0.58) * (is_int8 ? 1.3 : 1.0);
-  const double hbm_per_block = (double)(T_BN * KSTEP) / (double)std::min<int64_t>(tm, 8) + (double)(bm * KSTEP) / (double)std::min<int64_t>(tn, 8);
-  // (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
-  const double t_latency = hbm_per_block >= 16384.0 ? (bm == 128 ? 1.2 : 1.0) * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
+  const int64_t tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn;
+  // the tile's own time per K block (the INT8 kernel of the same structure is 1.3x slower: measured on K=4096 -> N=28672)
+  const double t_tile = (bn == 256 ? (bm == 128 ? 0.88 : 0.58) : (bm == 128 ? 0.52 : 0.40)) * (is_int8 ? 1.3 : 1.0);
+  const double hbm_per_block = (double)(bn * KSTEP) / (double)std::min<int64_t>(tm, 8) + (double)(bm * KSTEP) / (double)std::min<int64_t>(tn, 8);
+  // latency floor while the weight streams from HBM: with 256 channels per tile when at most two token tiles share it,
+  // with 128 when nobody does (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
+  const bool streams = bn == 256 ? hbm_per_block >= 16384.0 : hbm_per_block >= (double)(bn * KSTEP);
+  const double t_latency = streams ? (bn == 256 ? (bm == 128 ? 1.2 : 1.0) : (bm == 128 ? 0.7 : 0.51)) * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
   double t = 0.0;
   for (int64_t left = tm * tn * sp; left > 0;) {
     const int64_t c = std::min<int64_t>(left, 256);
@@ -333,23 +342,26 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8) {
   const double useful = (double)N * K + (double)M * K + 2.0 * M * N;
   const int max_split = (N % 4 == 0) ? 16 : 1;  // the reduce kernel works on aligned quads of one row
   double best_time = 1e30;
-  pl.bm = 128, pl.splits = 1, pl.efficiency = 0.0;
-  for (int bm = 64; bm <= 128; bm += 64) {
-    if (M <= 64 && bm == 128) break;                 // a second half tile of padding rows buys nothing
-    if (M > 64 && M <= 128 && bm == 64) continue;    // two token tiles would stream the weight twice
-    const double tile_factor = (bm == 64 && M > 128) ? 0.65 : 1.0;
-    const int64_t tiles = ((M + bm - 1) / bm) * ((N + T_BN - 1) / T_BN);
-    for (int sp = 1; sp <= max_split; ++sp) {
-      const int64_t per = (kb_total + sp - 1) / sp;
-      if (sp > 1 && per < 4) break;
-      if ((kb_total + per - 1) / per != sp) continue;  // some split would get no work
-      const double t = dma3_model_us(M, N, kb_total, bm, sp, is_int8);
-      if (t < best_time) best_time = t, pl.splits = sp, pl.bm = bm;
-      const int64_t wgs = tiles * sp;
-      const int64_t rounds = (wgs + 255) / 256;
-      const double balance = (double)wgs / (double)(rounds * 256);
-      const double partial = sp > 1 ? 8.0 * sp * M * N : 0.0;
-      pl.efficiency = std::max(pl.efficiency, balance * useful / (useful + partial) * (double)per / (double)(per + 2) * tile_factor);
+  pl.bm = 128, pl.bn = T_BN, pl.splits = 1, pl.efficiency = 0.0;
+  for (int bn = T_BN; bn >= (is_int8 ? T_BN : 128); bn -= 128) {  // the INT8 kernel has 256-channel tiles only
+    for (int bm = 64; bm <= 128; bm += 64) {
+      if (M <= 64 && bm == 128) break;                 // a second half tile of padding rows buys nothing
+      if (M > 64 && M <= 128 && bm == 64) continue;    // two token tiles would stream the weight twice
+      const double tile_factor = (bm == 64 && M > 128) ? 0.65 : 1.0;
+      const int64_t tiles = ((M + bm - 1) / bm) * ((N + T_BN - 1) / T_BN);
+      for (int sp = 1; sp <= max_split; ++sp) {
+        const int64_t per = (kb_total + sp - 1) / sp;
+        if (sp > 1 && per < 4) break;
+        if ((kb_total + per - 1) / per != sp) continue;  // some split would get no work
+        const double t = dma3_model_us(M, N, kb_total, bm, bn, sp, is_int8);
+        if (t < best_time) best_time = t, pl.splits = sp, pl.bm = bm, pl.bn = bn;
+        if (bn != T_BN) continue;  // the byte-model score below is defined on 256-channel tiles
+        const int64_t wgs = tiles * sp;
+        const int64_t rounds = (wgs + 255) / 256;
+        const double balance = (double)wgs / (double)(rounds * 256);
+        const double partial = sp > 1 ? 8.0 * sp * M * N : 0.0;
+        pl.efficiency = std::max(pl.efficiency, balance * useful / (useful + partial) * (double)per / (double)(per + 2) * tile_factor);
+      }
     }
   }
   pl.kb_per_split = (int)((kb_total + pl.splits - 1) / pl.splits);
@@ -368,8 +380,9 @@ int launch_fp8_grouped_dma3(GroupedParams& gp, int bm, hipStream_t stream, const
   return check_launch(what);
 }
 
-int launch_fp8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what) {
-  return bm == 64 ? launch_bm<64>(p, stream, what) : launch_bm<128>(p, stream, what);
+int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what) {
+  if (bn == 128) return bm == 64 ? launch_bm<64, 128>(p, stream, what) : launch_bm<128, 128>(p, stream, what);
+  return bm == 64 ? launch_bm<64, 256>(p, stream, what) : launch_bm<128, 256>(p, stream, what);
 }
 
 }  // namespace mi355

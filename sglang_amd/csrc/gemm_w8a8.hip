@@ -450,7 +450,7 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
       }
     }
     if ((M >= 256 && M <= 1024) || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
-      r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = 256, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
+      r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = dp.bn, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
       return r;
     }
   }
@@ -558,7 +558,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
       rc = IS_FP8 ? launch_fp8_decode(p, r.groups_per_wg, stream, what) : launch_int8_decode(p, r.groups_per_wg, stream, what);
       break;
     case RK_DMA3:
-      rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, stream, what) : launch_int8_dma3(p, r.bm, stream, what);
+      rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, r.bn, stream, what) : launch_int8_dma3(p, r.bm, stream, what);
       break;
     case RK_PINGPONG: return IS_FP8 ? launch_fp8_pp(p, stream, what) : launch_int8_pp(p, stream, what);
     case RK_PIPELINED: return launch_fp8_pipelined(p, stream, what);
