@@ -224,7 +224,7 @@ __device__ __forceinline__ bool grouped_tile_of_block(const GroupedParams& gp, G
 }
 int launch_fp8_grouped_dma3(GroupedParams& gp, int bm, hipStream_t stream, const char* what);  // gemm_fp8_dma3.hip; bm: 64 or 128
 int launch_fp8_grouped_pp(GroupedParams& gp, hipStream_t stream, const char* what);            // gemm_fp8_pp.hip: 256-row tiles
-int launch_int8_dma3(GemmParams& p, int bm, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
+int launch_int8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
 
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases, direct-to-LDS loads,
 // 32x32x32 MFMA); gemm_int8_pp.hip.  Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.

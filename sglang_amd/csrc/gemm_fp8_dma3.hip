@@ -296,14 +296,14 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 // and split count; it names the measured best or a choice within 5 % of it for 22 of them, within 12 % for the others):
 //   * a workgroup spends per K block the largest of
 //       - the tile's own time when operands come from L2: 0.88 us for 128 token rows, 0.58 us for 64 (0.52 / 0.40 with
-//         128 channels; x 1.2 in a round that keeps more than 200 CUs busy, x 1.3 for the INT8 kernel);
+//         128 channels; x 1.2 in a round that keeps more than 200 CUs busy; the INT8 kernel: 1.14 / 0.71 / 0.64 / 0.44);
 //       - a latency floor when the weight comes from HBM (two blocks in flight per CU): 1.2 us / 1.0 us (0.7 / 0.51 with
-//         128 channels), times 1.2 for weight rows longer than 8 KB;
+//         128 channels; INT8: 0.96 / 0.68 / 0.59 / 0.54), times 1.2 for weight rows longer than 8 KB;
 //       - its share of the HBM stream: (concurrent workgroups) x (HBM bytes per workgroup and block) / 5.5 TB/s, where
 //         weight rows are shared in L2 by up to 8 token tiles and token rows by up to 8 channel tiles;
 //   * a workgroup runs kb_per + 2 blocks (pipeline fill), and rounds of up to 256 workgroups follow each other;
-//   * a split adds the fp32 partial tiles written and read back (8 * splits * M * N bytes at 5.5 TB/s) and 10 us for the
-//     second launch and its tail.
+//   * a split adds the fp32 partial tiles written and read back (8 * splits * M * N bytes at 5.5 TB/s) and
+//     8 + 0.25 * splits us for the second launch and its tail.
 // So 144 workgroups streaming a weight unsplit beat 432 that split K in three (measured at M = 32 and 64 on K = 7168 ->
 // N = 36864: 58 against 65 us): with all CUs busy the HBM stream, not the number of workgroups, is the limit, and the
 // partial sums only add traffic.
@@ -316,13 +316,17 @@ double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int bn, int
   constexpr double HBM_BYTES_PER_US = 5.5e6;
   const int64_t per = (kb_total + sp - 1) / sp;
   const int64_t tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn;
-  // the tile's own time per K block (the INT8 kernel of the same structure is 1.3x slower: measured on K=4096 -> N=28672)
-  const double t_tile = (bn == 256 ? (bm == 128 ? 0.88 : 0.58) : (bm == 128 ? 0.52 : 0.40)) * (is_int8 ? 1.3 : 1.0);
+  // the tile's own time per K block and the latency floor, in the order 128x256, 64x256, 128x128, 64x128 (the INT8 kernel
+  // of the same structure has its own: fitted to K=4096 -> N=4096..28672 and K=14336 -> N=4096 at 24..1024 tokens)
+  static constexpr double TILE_US[2][4] = {{0.88, 0.58, 0.52, 0.40}, {1.14, 0.71, 0.64, 0.44}};
+  static constexpr double LATENCY_US[2][4] = {{1.2, 1.0, 0.7, 0.51}, {0.96, 0.68, 0.59, 0.54}};
+  const int shape = (bn == 256 ? 0 : 2) + (bm == 128 ? 0 : 1);
+  const double t_tile = TILE_US[is_int8][shape];
   const double hbm_per_block = (double)(bn * KSTEP) / (double)std::min<int64_t>(tm, 8) + (double)(bm * KSTEP) / (double)std::min<int64_t>(tn, 8);
   // latency floor while the weight streams from HBM: with 256 channels per tile when at most two token tiles share it,
   // with 128 when nobody does (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
   const bool streams = bn == 256 ? hbm_per_block >= 16384.0 : hbm_per_block >= (double)(bn * KSTEP);
-  const double t_latency = streams ? (bn == 256 ? (bm == 128 ? 1.2 : 1.0) : (bm == 128 ? 0.7 : 0.51)) * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
+  const double t_latency = streams ? LATENCY_US[is_int8][shape] * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
   double t = 0.0;
   for (int64_t left = tm * tn * sp; left > 0;) {
     const int64_t c = std::min<int64_t>(left, 256);
@@ -331,7 +335,7 @@ double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int bn, int
     const double t_own = t_tile * (c > 200 ? 1.2 : 1.0);
     t += (double)(per + 2) * std::max(std::max(t_own, t_latency), (double)c * hbm_per_block / HBM_BYTES_PER_US);
   }
-  if (sp > 1) t += 8.0 * sp * (double)M * (double)N / HBM_BYTES_PER_US + 10.0;
+  if (sp > 1) t += 8.0 * sp * (double)M * (double)N / HBM_BYTES_PER_US + 8.0 + 0.25 * sp;
   return t;
 }
 }  // namespace
@@ -343,10 +347,9 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8) {
   const int max_split = (N % 4 == 0) ? 16 : 1;  // the reduce kernel works on aligned quads of one row
   double best_time = 1e30;
   pl.bm = 128, pl.bn = T_BN, pl.splits = 1, pl.efficiency = 0.0;
-  for (int bn = T_BN; bn >= (is_int8 ? T_BN : 128); bn -= 128) {  // the INT8 kernel has 256-channel tiles only
+  for (int bn = T_BN; bn >= 128; bn -= 128) {
     for (int bm = 64; bm <= 128; bm += 64) {
       if (M <= 64 && bm == 128) break;                 // a second half tile of padding rows buys nothing
-      if (M > 64 && M <= 128 && bm == 64) continue;    // two token tiles would stream the weight twice
       const double tile_factor = (bm == 64 && M > 128) ? 0.65 : 1.0;
       const int64_t tiles = ((M + bm - 1) / bm) * ((N + T_BN - 1) / T_BN);
       for (int sp = 1; sp <= max_split; ++sp) {

@@ -435,8 +435,10 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   if (M > 16 && (M <= 1024 || tiles_256 < NUM_CUS) && K % KSTEP == 0 && aligned && small_offsets) {
     // mid-M, or many tokens but too few channels for 256 x 256 tiles: three-stage direct-to-LDS kernel with 64- or 128-token
     // tiles, when its tiling fills the chip well enough
-    // Between 256 and 1024 tokens it beats the generic kernel even where its tiling fills the chip badly (measured on K=4096..7168 ->
-    // N=1536..6144: 25 us against 35..63 us); below that the generic kernel's small tiles win for few channels.
+    // Up to 1024 tokens it beats the generic kernel for every layer measured (K=1536..14336 -> N=576..28672 at 24..1024
+    // tokens: e.g. 9 against 25 us for K=2048 -> N=7168 at 128 tokens), its 64 x 128 tiles and K splits filling the chip
+    // where the channels alone do not; without splits (N not a multiple of 4) and above 1024 tokens the older
+    // chip-filling score decides.
     const Dma3Plan dp = dma3_plan(M, N, K, !is_fp8);
     // Between 129 and 1024 tokens the two-phase 256 x 256 kernel competes: a round of its tiles takes (K blocks) x 1.39 us
     // + 11 us (INT8: 1.46 us per block), whatever part of the tile is filled and however many CUs the round uses, so it
@@ -449,7 +451,7 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
         return r;
       }
     }
-    if ((M >= 256 && M <= 1024) || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
+    if ((M <= 1024 && N % 4 == 0) || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
       r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = dp.bn, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
       return r;
     }
@@ -558,7 +560,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
       rc = IS_FP8 ? launch_fp8_decode(p, r.groups_per_wg, stream, what) : launch_int8_decode(p, r.groups_per_wg, stream, what);
       break;
     case RK_DMA3:
-      rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, r.bn, stream, what) : launch_int8_dma3(p, r.bm, stream, what);
+      rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, r.bn, stream, what) : launch_int8_dma3(p, r.bm, r.bn, stream, what);
       break;
     case RK_PINGPONG: return IS_FP8 ? launch_fp8_pp(p, stream, what) : launch_int8_pp(p, stream, what);
     case RK_PIPELINED: return launch_fp8_pipelined(p, stream, what);

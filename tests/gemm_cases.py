@@ -18,11 +18,16 @@ FP8_ROUTE_SHAPES = [
     (250, 8192, 7296), (100, 16384, 3584), (500, 4096, 14336),
     # the same kernel with 256-channel tiles and a K split (long K, many channels), and with 128-channel tiles
     (65, 7168, 18432), (24, 36864, 14336), (100, 36864, 640), (40, 4096, 7168), (300, 4096, 7168), (1000, 4096, 2048),
+    (400, 4096, 16384),
     # 256 x 256 two-phase and 256 x 128 pipelined kernels, K a multiple of 128 and not
     (4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 256), (4000, 2100, 272),
     # generic kernel: every token-tile height, aligned and byte-granular loads, whole-K and split
     (7, 1088, 512), (16, 576, 7168), (1, 1088, 3884), (17, 384, 2304), (20, 256, 264), (33, 512, 512), (64, 128, 3884),
     (50, 300, 520), (127, 128, 4096), (130, 640, 896), (1500, 640, 1000), (130, 200, 300), (2048, 4224, 264),
+    # between 17 and 1024 tokens only K % 128 != 0 (or unaligned rows) leaves the mid-M kernel to the generic one
+    (20, 256, 2064), (33, 256, 272), (100, 256, 400), (100, 640, 2064),
+    # 128-channel tiles with a ragged last channel tile
+    (50, 3000, 4224),
 ]
 
 FP8_REQUIRED_VARIANTS = {
@@ -44,14 +49,20 @@ INT8_ROUTE_SHAPES = [
     (5, 66048, 512), (2, 133120, 384),
     (20, 8192, 4096), (40, 65536, 512), (200, 16384, 2048), (200, 32768, 1024), (300, 4096, 14336), (130, 8192, 7168),
     (100, 16384, 3584), (500, 4096, 14336),
+    # the mid-M kernel's 128-channel tiles (and 128 x 256 with a K split): ragged M, a ragged last channel tile
+    (700, 6144, 14336), (100, 6144, 7168), (100, 28672, 512), (40, 6144, 14336), (20, 2048, 4096), (20, 4096, 1024),
+    (50, 3000, 4224),
     (4096, 4096, 512), (4000, 4088, 1024),
     (1, 16, 512), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
+    # between 17 and 1024 tokens only K % 128 != 0 leaves the mid-M kernel to the generic one
+    (20, 256, 2064), (33, 256, 272), (100, 256, 400), (100, 640, 2064),
 ]
 
 INT8_REQUIRED_VARIANTS = {
     ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
     ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
+    ("dma3", 64, "whole", "bn128"), ("dma3", 64, "split", "bn128"), ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"),
     ("pingpong", "kfull"),
     ("generic", 16, "aligned", "whole"), ("generic", 32, "aligned", "split"), ("generic", 64, "aligned", "whole"),
     ("generic", 128, "aligned", "whole"), ("generic", 128, "aligned", "split"), ("generic", 256, "aligned", "whole"),
