@@ -30,14 +30,6 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
 typedef const __attribute__((address_space(4))) float* cfloat_ptr;
 
-// three stages: tiles (rows 0..BM-1 tokens, BM.. channels) and the tile's BM token scales
-__shared__ __attribute__((aligned(1024))) uint8_t t_stage0[(128 + T_BN) * KSTEP];
-__shared__ __attribute__((aligned(1024))) uint8_t t_stage1[(128 + T_BN) * KSTEP];
-__shared__ __attribute__((aligned(1024))) uint8_t t_stage2[(128 + T_BN) * KSTEP];
-__shared__ __attribute__((aligned(256))) float t_scale0[512];
-__shared__ __attribute__((aligned(256))) float t_scale1[512];
-__shared__ __attribute__((aligned(256))) float t_scale2[512];
-
 struct Frag {
   u32x4 lo, hi;
 };
@@ -195,6 +187,15 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   s.sa_sk = p.sa_sk;
   s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * T_WN, p.N - 1) / 128) * p.sb_sn);
   s.sb_sk = p.sb_sk;
+
+  // three stages: tiles (rows 0..BM-1 tokens, BM.. channels) and the tile's BM token scales, sized per tile shape: a
+  // 64 x 128 tile takes 73.5 KB, so two such workgroups share a CU's 160 KB
+  __shared__ __attribute__((aligned(1024))) uint8_t t_stage0[(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(1024))) uint8_t t_stage1[(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(1024))) uint8_t t_stage2[(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(256))) float t_scale0[BM];
+  __shared__ __attribute__((aligned(256))) float t_scale1[BM];
+  __shared__ __attribute__((aligned(256))) float t_scale2[BM];
 
   float acc[T_NT][MT][4];
 #pragma unroll

@@ -16,14 +16,10 @@ namespace {
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int U_THREADS = 512;
-constexpr int U_BN = 256;  // widest channel tile (sizes the LDS stages); the kernels take BN = 128 or 256
 
 typedef __attribute__((address_space(3))) void* lptr_t;
 typedef const __attribute__((address_space(3))) uint8_t* lds_cptr;
 
-__shared__ __attribute__((aligned(1024))) uint8_t u_stage0[(128 + U_BN) * KSTEP];
-__shared__ __attribute__((aligned(1024))) uint8_t u_stage1[(128 + U_BN) * KSTEP];
-__shared__ __attribute__((aligned(1024))) uint8_t u_stage2[(128 + U_BN) * KSTEP];
 
 __device__ __forceinline__ v4i lds16(lds_cptr p, int imm) {
   const u32x4 v = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(p + imm);
@@ -103,6 +99,11 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
   const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
   const int nkb = kb_end - kb_begin;
 
+  // three stages of (BM token rows + BN channel rows) x 128 bytes, sized per tile shape: a 64 x 128 tile takes 72 KB, so
+  // two such workgroups share a CU's 160 KB
+  __shared__ __attribute__((aligned(1024))) uint8_t u_stage0[(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(1024))) uint8_t u_stage1[(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(1024))) uint8_t u_stage2[(BM + BN) * KSTEP];
   U8State<BM, BN> s;
   s.wave = wave;
   s.kb_last = kb_end - 1;

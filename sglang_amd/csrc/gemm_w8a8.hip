@@ -435,23 +435,23 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   if (M > 16 && (M <= 1024 || tiles_256 < NUM_CUS) && K % KSTEP == 0 && aligned && small_offsets) {
     // mid-M, or many tokens but too few channels for 256 x 256 tiles: three-stage direct-to-LDS kernel with 64- or 128-token
     // tiles, when its tiling fills the chip well enough
-    // Up to 1024 tokens it beats the generic kernel for every layer measured (K=1536..14336 -> N=576..28672 at 24..1024
-    // tokens: e.g. 9 against 25 us for K=2048 -> N=7168 at 128 tokens), its 64 x 128 tiles and K splits filling the chip
-    // where the channels alone do not; without splits (N not a multiple of 4) and above 1024 tokens the older
+    // It beats the generic kernel for every layer measured (K=1536..18432 -> N=576..28672 at 24..4096 tokens: e.g. 9 against
+    // 25 us for K=2048 -> N=7168 at 128 tokens, 23 against 68 us for K=7168 -> N=576 at 2048), its 64 x 128 tiles and K
+    // splits filling the chip where the channels alone do not; without splits (N not a multiple of 4) the older
     // chip-filling score decides.
     const Dma3Plan dp = dma3_plan(M, N, K, !is_fp8);
-    // Between 129 and 1024 tokens the two-phase 256 x 256 kernel competes: a round of its tiles takes (K blocks) x 1.39 us
-    // + 11 us (INT8: 1.46 us per block), whatever part of the tile is filled and however many CUs the round uses, so it
-    // wins where the channels alone give it a round's worth of tiles (measured: K=7168 -> N=36864 at M=256: 89 against
-    // 141 us, M=1024: 260 against 308 us; INT8 K=4096 -> N=28672 at M=512: 59 against 94 us) and loses for few channels.
-    if (M > 128 && M <= 1024 && (is_fp8 || K % KSTEP == 0)) {
+    // Above 128 tokens the two-phase 256 x 256 kernel competes: a round of its tiles takes (K blocks) x 1.39 us + 11 us
+    // (INT8: 1.46 us per block), whatever part of the tile is filled and however many CUs the round uses, so it wins
+    // where the channels alone give it a round's worth of tiles (measured: K=7168 -> N=36864 at M=256: 89 against 141 us,
+    // M=1024: 260 against 308 us; INT8 K=4096 -> N=28672 at M=512: 59 against 94 us) and loses for few channels.
+    if (M > 128) {
       const double pp_us = (double)((tiles_256 + NUM_CUS - 1) / NUM_CUS) * ((double)(K / KSTEP) * (is_fp8 ? 1.39 : 1.46) + 11.0);
       if (pp_us < dp.time_us) {
         r.kernel = RK_PINGPONG, r.bm = 256, r.bn = 256, r.splits = 1, r.kb_per_split = (int)(K / KSTEP);
         return r;
       }
     }
-    if ((M <= 1024 && N % 4 == 0) || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
+    if (N % 4 == 0 || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
       r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = dp.bn, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
       return r;
     }

@@ -20,7 +20,8 @@ FP8_ROUTE_SHAPES = [
     (65, 7168, 18432), (24, 36864, 14336), (100, 36864, 640), (40, 4096, 7168), (300, 4096, 7168), (1000, 4096, 2048),
     (400, 4096, 16384),
     # 256 x 256 two-phase and 256 x 128 pipelined kernels, K a multiple of 128 and not
-    (4096, 4352, 512), (4000, 4300, 400), (4096, 2176, 256), (4000, 2100, 272),
+    # (the pipelined kernel takes whole-K shapes only where N % 4 != 0 rules the mid-M kernel's split reduce out)
+    (4096, 4352, 512), (4000, 4300, 400), (4096, 2178, 256), (4000, 2100, 272), (4096, 2176, 256),
     # generic kernel: every token-tile height, aligned and byte-granular loads, whole-K and split
     (7, 1088, 512), (16, 576, 7168), (1, 1088, 3884), (17, 384, 2304), (20, 256, 264), (33, 512, 512), (64, 128, 3884),
     (50, 300, 520), (127, 128, 4096), (130, 640, 896), (1500, 640, 1000), (130, 200, 300), (2048, 4224, 264),
