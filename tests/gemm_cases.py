@@ -27,8 +27,8 @@ FP8_ROUTE_SHAPES = [
     (50, 300, 520), (127, 128, 4096), (130, 640, 896), (1500, 640, 1000), (130, 200, 300), (2048, 4224, 264),
     # between 17 and 1024 tokens only K % 128 != 0 (or unaligned rows) leaves the mid-M kernel to the generic one
     (20, 256, 2064), (33, 256, 272), (100, 256, 400), (100, 640, 2064),
-    # 128-channel tiles with a ragged last channel tile
-    (50, 3000, 4224),
+    # 128-channel tiles with a ragged last channel tile; a handful of channels; a single K block
+    (50, 3000, 4224), (40, 8, 1024), (100, 16, 4096), (1000, 8, 128),
 ]
 
 FP8_REQUIRED_VARIANTS = {
@@ -52,7 +52,7 @@ INT8_ROUTE_SHAPES = [
     (100, 16384, 3584), (500, 4096, 14336),
     # the mid-M kernel's 128-channel tiles (and 128 x 256 with a K split): ragged M, a ragged last channel tile
     (700, 6144, 14336), (100, 6144, 7168), (100, 28672, 512), (40, 6144, 14336), (20, 2048, 4096), (20, 4096, 1024),
-    (50, 3000, 4224),
+    (50, 3000, 4224), (40, 8, 1024), (100, 16, 4096), (1000, 8, 128),
     (4096, 4096, 512), (4000, 4088, 1024),
     (1, 16, 512), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
     # between 17 and 1024 tokens only K % 128 != 0 leaves the mid-M kernel to the generic one
