@@ -226,6 +226,20 @@ int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, in
  */
 int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
 
+/* Per-token-group FP8 quantization with the whole row as ONE group: s[m] = max(absmax of row m, eps) / 448 and
+ * q = e4m3fn(clamp(x * (1 / s[m]), -448, 448)) (mode MI355_QUANT_RCP) or q = e4m3fn(clamp(x / s[m], -448, 448)) with a
+ * true division (mode MI355_QUANT_DIV).
+ *
+ * Replaces per_token_group_quant_fp8 called with group_size == K, which is how the reference quantizes the weights of a
+ * 16-bit checkpoint per output channel at load time (python/sglang/srt/layers/quantization/fp8.py:368-375:
+ * per_token_group_quant_fp8(layer.weight, layer.weight.shape[-1]), the Triton kernel fp8_kernel.py:122-161 = RCP), and
+ * sgl_per_token_group_quant_8bit with such a group (sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:25-114 = DIV).
+ * mi355_group_quant_8bit covers power-of-two groups of up to 2048 input bytes; this entry covers rows of any length
+ * that is a multiple of 16 bytes.
+ * x [M, K] contiguous f32/f16/bf16 (16-byte aligned), q [M, K] e4m3fn (8-byte aligned), s [M] fp32. */
+int mi355_row_group_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, float eps, int mode,
+                              void* stream);
+
 /*
  * Weight-side 128 x 128 block quantization (load time: re-quantizing a block-FP8 checkpoint to power-of-two scales).
  *   mi355_block_cast_to_fp8:  x [m, n] contiguous F32/F16/BF16 -> q [m, n] e4m3fn, s [ceil(m/128), ceil(n/128)] fp32

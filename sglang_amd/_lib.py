@@ -37,6 +37,7 @@ EXPORTS = (
     "mi355_int8_scaled_mm_plan",
     "mi355_per_token_quant_int8",
     "mi355_per_token_quant_fp8",
+    "mi355_row_group_quant_fp8",
     "mi355_per_tensor_quant_fp8",
     "mi355_silu_mul_group_quant_fp8",
     "mi355_block_cast_to_fp8",
@@ -109,6 +110,8 @@ def lib() -> ctypes.CDLL:
     L.mi355_per_token_quant_int8.restype = i32
     L.mi355_per_token_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
     L.mi355_per_token_quant_fp8.restype = i32
+    L.mi355_row_group_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64, ctypes.c_float, i32, vp]
+    L.mi355_row_group_quant_fp8.restype = i32
     L.mi355_per_tensor_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i32, vp, i64, vp]
     L.mi355_per_tensor_quant_fp8.restype = i32
     L.mi355_silu_mul_group_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64, i64, vp, i64, i64, vp]

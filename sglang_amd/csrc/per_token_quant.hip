@@ -6,6 +6,11 @@
 //         python/sglang/srt/layers/quantization/int8_kernel.py:47-50;
 //   FP8:  scale = absmax / 448 (no floor), q = e4m3fn(clamp(x * (1 / scale))) rounded to nearest even, a row of zeros
 //         gives scale 0 and zeros, as in sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-85.
+//   FP8, whole row as ONE quantization group (per_token_group_quant_fp8 with group_size == K, what the reference
+//         quantizes a 16-bit checkpoint's weights with at load time, python/sglang/srt/layers/quantization/fp8.py:368-375):
+//         scale = max(absmax, eps) / 448 and either q = e4m3fn(clamp(x * (1 / scale))), the arithmetic of the Triton kernel
+//         python/sglang/srt/layers/quantization/fp8_kernel.py:122-161, or q = e4m3fn(clamp(x / scale)) with a true
+//         division, the arithmetic of sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:25-114.
 // Rows of up to 8192 two-byte elements stay in registers between the two phases; longer rows are
 // re-read (from L2).
 // Two-byte inputs with rows of at most 8192 elements (every hidden size of the benchmark models) take a second kernel: one
@@ -66,8 +71,8 @@ __device__ __forceinline__ float row_scale(float amax, float& mul) {
   }
 }
 
-// One 16-byte vector of input -> 4 or 8 codes at d.
-template <int DT, bool FP8_OUT, bool STREAM>
+// One 16-byte vector of input -> 4 or 8 codes at d.  DIVIDE: `mul` is the scale and the elements are divided by it.
+template <int DT, bool FP8_OUT, bool STREAM, bool DIVIDE = false>
 __device__ __forceinline__ void emit_vector(const u32x4& raw, float mul, int8_t* d) {
   constexpr int VEC = (DT == MI355_F32) ? 4 : 8;
   float f[VEC];
@@ -79,7 +84,7 @@ __device__ __forceinline__ void emit_vector(const u32x4& raw, float mul, int8_t*
     if constexpr (FP8_OUT) {
       float t[4];
 #pragma unroll
-      for (int b = 0; b < 4; ++b) t[b] = fmaxf(fminf(f[4 * j + b] * mul, 448.0f), -448.0f);
+      for (int b = 0; b < 4; ++b) t[b] = fmaxf(fminf(DIVIDE ? f[4 * j + b] / mul : f[4 * j + b] * mul, 448.0f), -448.0f);
       int c = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
       c = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c, true);
       pk = (uint32_t)c;
@@ -131,8 +136,12 @@ __global__ __launch_bounds__(256) void per_token_quant_wave_kernel(const void* x
   }
 }
 
-template <int DT, bool FP8_OUT>
-__global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int8_t* q, float* s, int64_t K) {
+// ROW_GROUP (FP8 only): the row is one quantization group: absmax floored at eps; DIVIDE: elements are divided by the
+// scale instead of multiplied by its reciprocal.
+template <int DT, bool FP8_OUT, bool ROW_GROUP = false, bool DIVIDE = false>
+__global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int8_t* q, float* s, int64_t K, float eps) {
+  static_assert(FP8_OUT || !ROW_GROUP, "whole-row groups are built for FP8 codes");
+  static_assert(ROW_GROUP || !DIVIDE, "division is a mode of the whole-row group");
   constexpr int VEC = (DT == MI355_F32) ? 4 : 8;
   constexpr int KEEP = 4;  // vectors per thread kept in registers
   __shared__ float wave_max[4];
@@ -140,7 +149,7 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int
   const int64_t nvec = K / VEC;
   const u32x4* src = reinterpret_cast<const u32x4*>(x) + row * nvec;
   u32x4 keep[KEEP];
-  float amax = FP8_OUT ? 0.f : 1e-10f;
+  float amax = ROW_GROUP ? eps : (FP8_OUT ? 0.f : 1e-10f);
 #pragma unroll
   for (int i = 0; i < KEEP; ++i) {
     const int64_t v = threadIdx.x + 256 * i;
@@ -161,10 +170,14 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int
   __syncthreads();
   amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
   float mul;
-  const float scale = row_scale<FP8_OUT>(amax, mul);
+  float scale = row_scale<FP8_OUT>(amax, mul);
+  if constexpr (ROW_GROUP) {
+    scale = amax / 448.0f;  // amax >= eps > 0
+    mul = DIVIDE ? scale : 1.0f / scale;
+  }
   if (threadIdx.x == 0) s[row] = scale;
 
-  auto emit = [&](const u32x4& raw, int64_t v) { emit_vector<DT, FP8_OUT, false>(raw, mul, q + row * K + v * VEC); };
+  auto emit = [&](const u32x4& raw, int64_t v) { emit_vector<DT, FP8_OUT, false, DIVIDE>(raw, mul, q + row * K + v * VEC); };
 #pragma unroll
   for (int i = 0; i < KEEP; ++i) {
     const int64_t v = threadIdx.x + 256 * i;
@@ -179,8 +192,9 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int
 namespace mi355 {
 namespace {
 
-template <bool FP8_OUT>
-int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream) {
+template <bool FP8_OUT, bool ROW_GROUP = false, bool DIVIDE = false>
+int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream,
+                    float eps = 0.f) {
   clear_error();
   MI355_REQUIRE(M >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
   MI355_REQUIRE(x_dtype == MI355_F32 || x_dtype == MI355_F16 || x_dtype == MI355_BF16, MI355_ERR_INVALID_ARGUMENT,
@@ -194,7 +208,7 @@ int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float
   MI355_REQUIRE(M < (1ll << 31), MI355_ERR_INVALID_ARGUMENT, "%s: too many rows", what);
   hipStream_t st = static_cast<hipStream_t>(stream);
   int8_t* qq = static_cast<int8_t*>(q);
-  if (x_dtype != MI355_F32 && K <= 8192) {  // one wave per row
+  if (!ROW_GROUP && x_dtype != MI355_F32 && K <= 8192) {  // one wave per row
     const dim3 grid((unsigned)((M + 3) / 4));
     const int nv = (int)((K / 8 + 63) / 64);
 #define MI355_WAVE_ROWS(DT, NV) \
@@ -213,13 +227,13 @@ int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float
   }
   switch (x_dtype) {
     case MI355_F32:
-      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F32, FP8_OUT>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F32, FP8_OUT, ROW_GROUP, DIVIDE>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps);
       break;
     case MI355_F16:
-      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F16, FP8_OUT>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F16, FP8_OUT, ROW_GROUP, DIVIDE>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps);
       break;
     default:
-      hipLaunchKernelGGL((per_token_quant_kernel<MI355_BF16, FP8_OUT>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_BF16, FP8_OUT, ROW_GROUP, DIVIDE>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps);
   }
   return check_launch(what);
 }
@@ -235,4 +249,15 @@ extern "C" int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, f
 extern "C" int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K,
                                          void* stream) {
   return mi355::per_token_quant<true>("mi355_per_token_quant_fp8", x, x_dtype, q, s, M, K, stream);
+}
+
+extern "C" int mi355_row_group_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, float eps,
+                                         int mode, void* stream) {
+  const char* what = "mi355_row_group_quant_fp8";
+  mi355::clear_error();
+  MI355_REQUIRE(eps > 0.f, MI355_ERR_INVALID_ARGUMENT, "%s: eps must be positive (it is the floor of the row maximum)", what);
+  MI355_REQUIRE(mode == MI355_QUANT_DIV || mode == MI355_QUANT_RCP, MI355_ERR_INVALID_ARGUMENT,
+                "%s: mode must be MI355_QUANT_DIV or MI355_QUANT_RCP", what);
+  if (mode == MI355_QUANT_DIV) return mi355::per_token_quant<true, true, true>(what, x, x_dtype, q, s, M, K, stream, eps);
+  return mi355::per_token_quant<true, true, false>(what, x, x_dtype, q, s, M, K, stream, eps);
 }

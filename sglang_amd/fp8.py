@@ -98,8 +98,6 @@ class Fp8Linear(torch.nn.Module):
                  tp_rank: int = 0, tp_size: int = 1, params_dtype: torch.dtype = torch.bfloat16, bias: bool = False,
                  device: Optional[torch.device] = None) -> None:
         super().__init__()
-        if not quant_config.is_checkpoint_fp8_serialized:
-            raise NotImplementedError("quantizing a 16-bit checkpoint to FP8 at load time is not built; the checkpoint must be FP8")
         if parallel not in (None, "column", "row"):
             raise ValueError(f"parallel must be None, 'column' or 'row', got {parallel!r}")
         if not 0 <= tp_rank < tp_size:
@@ -128,9 +126,15 @@ class Fp8Linear(torch.nn.Module):
                     if v % block_n != 0:
                         raise ValueError(f"Weight output_partition_size = {v} is not divisible by weight quantization block_n = {block_n}.")
         P = lambda t: torch.nn.Parameter(t, requires_grad=False)
-        self.weight = P(torch.empty(n, k, dtype=FP8, device=device))
+        self.serialized = quant_config.is_checkpoint_fp8_serialized
+        self.weight = P(torch.empty(n, k, dtype=FP8 if self.serialized else params_dtype, device=device))
         lowest = torch.finfo(torch.float32).min  # "not loaded yet", as the reference marks scales
-        if self.block_quant:
+        if not self.serialized:
+            # a 16-bit checkpoint: the weight is loaded as it is and quantized in process_weights_after_loading
+            # (fp8.py:293-295, :368-383); Fp8Config refuses block quantization for such a checkpoint
+            self.weight_scale = None
+            self.input_scale = None
+        elif self.block_quant:
             self.weight_scale_inv = P(torch.full((_ceil_div(n, block_n), _ceil_div(k, block_k)), lowest, dtype=torch.float32, device=device))
             self.input_scale = None
         else:
@@ -190,7 +194,7 @@ class Fp8Linear(torch.nn.Module):
         one.  Missing weights or scales raise KeyError."""
         if len(prefixes) not in (1, len(self.output_sizes)):
             raise ValueError("one prefix, or one per merged projection")
-        names = ["weight"] + (["weight_scale_inv"] if self.block_quant else ["weight_scale"])
+        names = ["weight"] + ([] if not self.serialized else ["weight_scale_inv"] if self.block_quant else ["weight_scale"])
         if self.input_scale is not None:
             names.append("input_scale")
         if self.bias is not None:
@@ -203,10 +207,22 @@ class Fp8Linear(torch.nn.Module):
     # ------------------------------------------------------------------ after loading, forward
 
     def process_weights_after_loading(self, requant_ue8m0: bool = False) -> None:
-        """fp8.py:343-465 for FP8-serialized checkpoints.  Block-FP8: the tensors stay as loaded (or are re-quantized to
+        """fp8.py:343-465.  A 16-bit checkpoint is quantized here, per output channel.  Block-FP8: the tensors stay as loaded (or are re-quantized to
         power-of-two scales: weight_scale_inv becomes packed int32 exponents, fp8_utils.py:428-449).  Per-tensor: one
         scale per merged projection becomes one scale per output channel (what fp8_scaled_mm takes), the weight is kept
         as its [K, N] column-major view, a static input scale is the maximum over the merged projections."""
+        if not self.serialized:
+            # fp8.py:368-383, the branch of a platform with per-channel FP8 GEMMs: one quantization group per output
+            # channel (per_token_group_quant_fp8 with group_size = K), scales as [1, N], no static input scale
+            from .fp8_kernel import per_token_group_quant_fp8
+
+            w = self.weight.data.contiguous()
+            qweight, weight_scale = per_token_group_quant_fp8(w, w.shape[-1])
+            self.weight = torch.nn.Parameter(qweight.t(), requires_grad=False)
+            self.weight_scale = torch.nn.Parameter(weight_scale.t().contiguous(), requires_grad=False)
+            self.input_scale = None
+            self._processed = True
+            return
         lowest = torch.finfo(torch.float32).min
         scale = self.weight_scale_inv if self.block_quant else self.weight_scale
         if bool((scale.data == lowest).any()) or (self.input_scale is not None and bool((self.input_scale.data == lowest).any())):

@@ -104,6 +104,13 @@ def _per_token_group_quant_8bit_raw(
     else:
         assert not scale_ue8m0
         mode, s_row, s_col = _lib.QUANT_RCP, K // group_size, 1
+    if (group_size == K and dtype == fp8_dtype and not scale_ue8m0
+            and (group_size * x.element_size() > 2048 or group_size & (group_size - 1))):
+        # the whole row is one group (a weight quantized per output channel at load time, fp8.py:368-375): rows
+        # longer than the group kernel's 2048 bytes, or not a power of two
+        _lib.check(_lib.lib().mi355_row_group_quant_fp8(x.data_ptr(), ops._DT[x.dtype], x_q.data_ptr(), x_s.data_ptr(), M, K, eps,
+                                                        mode, torch.cuda.current_stream().cuda_stream))
+        return x_q, x_s
     kind = _lib.SCALE_UE8M0_PACKED if scale_ue8m0 else _lib.SCALE_F32
     _lib.check(
         _lib.lib().mi355_group_quant_8bit(

@@ -80,6 +80,15 @@ def _group_quant(input, output_q, output_s, group_size, eps, qmin, qmax, scale_u
     K = input.size(-1)
     M = input.numel() // K
     _require(K % group_size == 0, f"{op}: the last dimension must be divisible by group_size")
+    if (group_size == K and mode == _lib.QUANT_DIV and not scale_ue8m0 and output_q.dtype == torch.float8_e4m3fn
+            and (group_size * input.element_size() > 2048 or group_size & (group_size - 1)) and output_s.dtype == torch.float32
+            and (qmin, qmax) == (-448.0, 448.0)):
+        # the whole row is one group (a weight quantized per output channel at load time): rows longer than the group
+        # kernel's 2048 bytes, or not a power of two
+        _require(output_s.numel() == M and output_s.is_contiguous(), f"{op}: output_s must hold one contiguous scale per row")
+        check(lib().mi355_row_group_quant_fp8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), output_s.data_ptr(),
+                                              M, K, eps, _lib.QUANT_DIV, _stream()))
+        return
     # same test as per_token_group_quant_8bit.cu:153 / per_token_group_quant_8bit_v2.cu:426
     column_major = output_s.stride(0) < output_s.stride(1)
     if scale_ue8m0:

@@ -71,6 +71,13 @@ def test_newer_entry_points_validate_before_any_device_work():
     assert L.mi355_silu_mul_group_quant_fp8(p, _lib.F32, p, p, 1, 4, 128, None, 0, 4, None) == 1
     assert L.mi355_silu_mul_group_quant_fp8(p, _lib.BF16, p, p, 1, 4, 100, None, 0, 4, None) == 2
     assert L.mi355_silu_mul_group_quant_fp8(None, _lib.BF16, None, None, 0, 4, 128, None, 0, 4, None) == 0
+    # whole-row group quantizer: eps positive, a known mode, a float input type, rows of whole 16-byte vectors, empty tensor
+    R = L.mi355_row_group_quant_fp8
+    assert R(p, _lib.BF16, p, p, 4, 256, 0.0, _lib.QUANT_DIV, None) == 1 and b"eps" in L.mi355_last_error()
+    assert R(p, _lib.BF16, p, p, 4, 256, 1e-10, _lib.QUANT_MUL, None) == 1 and b"mode" in L.mi355_last_error()
+    assert R(p, _lib.I8, p, p, 4, 256, 1e-10, _lib.QUANT_RCP, None) == 1
+    assert R(p, _lib.BF16, p, p, 4, 100, 1e-10, _lib.QUANT_RCP, None) == 2
+    assert R(None, _lib.BF16, None, None, 0, 256, 1e-10, _lib.QUANT_DIV, None) == 0
     # weight-side block cast / dequant
     assert L.mi355_block_cast_to_fp8(p, _lib.I8, p, p, 128, 128, None) == 1
     assert L.mi355_block_cast_to_fp8(None, _lib.BF16, None, None, 0, 128, None) == 0

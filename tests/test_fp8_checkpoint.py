@@ -38,8 +38,9 @@ def test_config_parsing_and_errors(tmp_path):
         Fp8Config(True, "dynamic", weight_block_size=[128])
     with pytest.raises(ValueError, match="only supports dynamic activation"):
         Fp8Config(True, "static", weight_block_size=[128, 128])
-    with pytest.raises(NotImplementedError):
-        Fp8Linear(256, [256], Fp8Config(False, "dynamic"))
+    # a 16-bit checkpoint: the weight parameter keeps the checkpoint's type until process_weights_after_loading, no scales
+    layer = Fp8Linear(256, [256], Fp8Config(False, "dynamic"))
+    assert layer.weight.dtype == torch.bfloat16 and layer.weight_scale is None and layer.input_scale is None
 
 
 def test_block_alignment_checks_of_create_weights():

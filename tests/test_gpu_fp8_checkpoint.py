@@ -118,3 +118,30 @@ def test_per_tensor_static_checkpoint(gpu, oracle):
     sb = torch.cat([torch.full((n,), s) for n, s in zip(sizes, ws)])
     ref, mag = oracle.fp8_scaled_mm(q_o, w, scale.expand(M).contiguous(), sb, torch.float32, None, want_abs=True)
     _close(out, ref, mag)
+
+
+@pytest.mark.parametrize("K,sizes", [(7168, [256, 128]), (1024, [384])])
+def test_sixteen_bit_checkpoint_is_quantized_per_channel_at_load(gpu, oracle, K, sizes):
+    """fp8.py:368-383: a bf16 checkpoint under quantization="fp8": one quantization group per output channel
+    (per_token_group_quant_fp8 with group_size = K), dynamic per-token activations, fp8_scaled_mm."""
+    from sglang_amd.fp8 import Fp8Config, Fp8Linear
+
+    cfg = Fp8Config.from_config({"quant_method": "none", "activation_scheme": "dynamic"})
+    assert not cfg.is_checkpoint_fp8_serialized
+    g = torch.Generator().manual_seed(3)
+    M = 19
+    layer = Fp8Linear(K, sizes, cfg, device=gpu)
+    names = ["gate", "up"][:len(sizes)]
+    tensors = {f"{n}.weight": (torch.randn(sz, K, generator=g) * 0.02).to(torch.bfloat16) for n, sz in zip(names, sizes)}
+    layer.load_from(tensors, names)
+    layer.process_weights_after_loading()
+    w16 = torch.cat([tensors[f"{n}.weight"] for n in names])
+    wq_o, ws_o = oracle.group_quant(w16, K, mode="rcp", layout="row")
+    assert tuple(layer.weight.shape) == (K, sum(sizes)) and tuple(layer.weight_scale.shape) == (1, sum(sizes))
+    assert torch.equal(layer.weight.data.t().contiguous().cpu().view(torch.uint8), wq_o.view(torch.uint8))
+    assert torch.equal(layer.weight_scale.data.cpu().view(-1), ws_o.view(-1))
+    x = make_activation(M, K, seed=5)
+    out = layer(x.to(gpu))
+    q_o, s_o = oracle.per_token_quant_fp8(x)
+    ref, mag = oracle.fp8_scaled_mm(q_o, wq_o, s_o.view(-1), ws_o.view(-1), torch.float32, None, want_abs=True)
+    _close(out, ref, mag)

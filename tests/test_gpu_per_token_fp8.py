@@ -30,6 +30,24 @@ def test_per_token_quant_fp8_bits(gpu, oracle, dtype, M, K):
         assert float(s[1]) == 0.0 and not bool(q[1].view(torch.uint8).any())
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K", [(3, 7168), (130, 4096), (5, 2056), (2, 18432), (7, 1536)])
+@pytest.mark.parametrize("column_major", [False, True])
+def test_whole_row_group_quant_bits(gpu, oracle, dtype, M, K, column_major):
+    """per_token_group_quant_fp8 with group_size == K (a weight quantized per output channel at load time): rows longer than
+    the group kernel's groups, not powers of two; row-major scales multiply by the reciprocal, column-major ones divide."""
+    from sglang_amd.fp8_kernel import per_token_group_quant_fp8
+
+    x = make_activation(M, K, seed=M * 11 + K, dtype=dtype)
+    x[1] = 0  # a row of zeros: the floor eps keeps the scale positive, codes are zero
+    q, s = per_token_group_quant_fp8(x.to(gpu), K, column_major_scales=column_major)
+    q_o, s_o = oracle.group_quant(x, K, mode="div" if column_major else "rcp", layout="col" if column_major else "row")
+    assert q.dtype == FP8 and tuple(s.shape) == (M, 1)
+    assert torch.equal(s.cpu().contiguous().view(torch.int32), s_o.contiguous().view(torch.int32))
+    assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8))
+    assert float(s[1]) == pytest.approx(1e-10 / 448.0) and not bool(q[1].view(torch.uint8).any())
+
+
 def _rand_fp8(shape, g):
     return ((torch.rand(*shape, generator=g) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
 

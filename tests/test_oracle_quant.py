@@ -49,6 +49,20 @@ def test_matches_torch_fp32_arithmetic(oracle, dtype, mode, group):
     assert torch.equal(q.view(torch.uint8), q_t.view(torch.uint8))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["div", "rcp"])
+@pytest.mark.parametrize("K", [1536, 7168])
+def test_whole_row_groups_match_torch_fp32_arithmetic(oracle, dtype, mode, K):
+    """group == K (a weight quantized per output channel at load time): the same routine over one long group."""
+    x = make_activation(9, K, seed=K + 3, dtype=dtype)
+    x[2] = 0
+    q, s = oracle.group_quant(x, K, mode=mode)
+    q_t, s_t = _torch_group_quant(x, K, mode)
+    assert tuple(s.shape) == (9, 1)
+    assert torch.equal(s.view(torch.int32), s_t.view(torch.int32))
+    assert torch.equal(q.view(torch.uint8), q_t.view(torch.uint8))
+
+
 def test_modes_differ_somewhere_but_only_by_one_code(oracle):
     # guards against the three modes being wired to the same arithmetic
     x = make_activation(256, 2048, seed=3)
