@@ -170,12 +170,12 @@ int launch_fp8_pp_rowcol(GemmParams& p, hipStream_t stream, const char* what);
 // gemm_fp8_dma3.hip.  Needs 16-byte aligned rows, K % 128 == 0, row offsets below 4 GiB.  dma3_plan() gives the split it
 // wants; the caller sets p.splits, p.kb_per_split and p.ws accordingly.
 struct Dma3Plan {
-  int bm, bn, splits, kb_per_split;  // bn: 256, or 128 for the FP8 kernel when narrow tiles model faster
+  int bm, bn, splits, kb_per_split;  // bn: 256, 192 (FP8 only) or 128, whichever models fastest
   double efficiency;  // modelled fraction of the streaming time that is useful (balance, partial sums, pipeline fill)
   double time_us;     // modelled duration of the chosen plan
 };
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8 = false);
-int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);  // bm: 64 or 128, bn: 128 or 256, from dma3_plan()
+int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);  // bm: 64 or 128, bn: 128, 192 or 256, from dma3_plan()
 
 // Grouped problems on the tile bodies of the dense kernels: token rows of all experts stacked in one matrix, one weight
 // matrix per expert.  `g` describes expert 0 (a, out, b, sb, and sa = the re-laid-out token scales: M-major, every

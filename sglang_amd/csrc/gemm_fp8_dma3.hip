@@ -1,9 +1,11 @@
-// Blockwise-scaled FP8 GEMM for gfx950 with short token tiles: (64 or 128) x 256 macro tile, 8 waves (two per SIMD), THREE LDS stages.
+// Blockwise-scaled FP8 GEMM for gfx950 with short token tiles: (64 or 128) x (256, 192 or 128) macro tile, 8 waves (two per SIMD),
+// THREE LDS stages.
 //
 // For 16 < M <= 1024 a linear layer is between weight streaming and MFMA-bound; prefill shapes with few output channels
 // (M = 4096, N = 576 or 1536) do not give 256 x 256 tiles enough workgroups.  Both take this kernel.  The tile is short in the token dimension
-// (64 or 128 tokens) and wide in channels (256), so a stage of LDS is (BM + 256) x 128 B <= 48 KB and three stages fit in
-// the CU's 160 KB.  With three stages the direct-to-LDS loads of K block k+2 are issued while block k is multiplied and
+// (64 or 128 tokens) and wide in channels (256; 192 and 128 where those fill the chip better: 36864 channels are 144 tiles
+// of 256 but 192 of 192, 1536 channels x 4096 tokens are exactly 256 tiles of 128 x 192), so a stage of LDS is
+// (BM + BN) x 128 B <= 48 KB and three stages fit in the CU's 160 KB.  With three stages the direct-to-LDS loads of K block k+2 are issued while block k is multiplied and
 // only have to land before block k+2 is multiplied, two barriers later: the wait that precedes the barrier at the end of
 // iteration k covers block k+1 only.  The compiler cannot express that (its wait before a barrier covers every load it
 // knows about), so inside the loop the loads, the wait and the barrier are written as instructions:
@@ -48,7 +50,13 @@ struct Dma3State {
   uint32_t goff[LOADS];   // lane's byte offset from the matrix base (rows clamped); first BM/64 loads are token rows
   const float* sa_base;   // token scales, M-major: element (m, kb) at sa_base[kb * sa_sk + m]
   uint32_t sa_off;        // byte offset of the four scales this lane fetches (first BM / 32 lanes), clamped to the last valid quad
-  cfloat_ptr sb_ptr;      // &sb[nb, 0] of this wave's 128-channel block
+  // Weight-block scale rows.  A wave's channels are BN / 4 consecutive ones inside one 128-channel block, except for
+  // BN = 192, where 48 consecutive channels could straddle two blocks: there the wave's tile i is channels
+  // 64 i + 16 wave .. + 15 of the tile, so that tile i of every wave lies in the block of channel n0 + 64 i.
+  static constexpr bool INTERLEAVED = BN == 192;
+  static constexpr int SB = INTERLEAVED ? BN / 64 : 1;
+  static constexpr int W_STRIDE = INTERLEAVED ? 64 * 128 : 16 * 128;  // bytes between a wave's consecutive channel tiles in a stage
+  cfloat_ptr sb_ptr[SB];  // &sb[nb, 0] of the wave's (tile's) 128-channel block
   int64_t sa_sk, sb_sk;
   int wave, kb_last;
   uint32_t tok_off[2], ch_off[2], sc_off;
@@ -84,12 +92,14 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM, BN>& s, int i, uin
 
 // One K block out of `cur`; the loads of block kb_next go out over the first LOADS + 1 steps into `nxt`.
 template <int BM, int BN>
-__device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_t* cur, const float* sc_cur, float sbv,
-                                        float (&acc)[BN / 64][BM / 32][4], uint8_t* nxt, float* sc_nxt, int kb_next) {
+__device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_t* cur, const float* sc_cur,
+                                        const float (&sbv)[Dma3State<BM, BN>::SB], float (&acc)[BN / 64][BM / 32][4], uint8_t* nxt,
+                                        float* sc_nxt, int kb_next) {
   constexpr int MT = BM / 32, T_NT = BN / 64, LOADS = Dma3State<BM, BN>::LOADS;  // a wave owns BN / 4 channels = T_NT tiles of 16
+  constexpr int SB = Dma3State<BM, BN>::SB, W_STRIDE = Dma3State<BM, BN>::W_STRIDE;
   static_assert(LOADS + 1 <= MT * T_NT, "one load per step");
   Frag w[T_NT], tokb[2];
-  float scb[2];
+  float scb[2][SB];
   const lds_cptr ch0 = (lds_cptr)cur + s.ch_off[0], ch1 = (lds_cptr)cur + s.ch_off[1];
   const lds_cptr tk0 = (lds_cptr)cur + s.tok_off[0], tk1 = (lds_cptr)cur + s.tok_off[1];
   w[0].lo = lds16(ch0, 0);
@@ -97,7 +107,8 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
   tokb[0].lo = lds16(tk0, 0);
   tokb[0].hi = lds16(tk1, 0);
   const float* scp = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(sc_cur) + s.sc_off);
-  scb[0] = scp[0] * sbv;
+#pragma unroll
+  for (int b = 0; b < SB; ++b) scb[0][b] = scp[0] * sbv[b];
   __builtin_amdgcn_sched_barrier(0);
 
   v4f part[2];
@@ -110,17 +121,20 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
     if (t > 0) {
       const int pj = (t - 1) / T_NT, pi = (t - 1) % T_NT;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[(t - 1) & 1][v], scb[pj & 1], acc[pi][pj][v]);
+      for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[(t - 1) & 1][v], scb[pj & 1][SB > 1 ? pi : 0], acc[pi][pj][v]);
     }
     if (t + 1 < T_NT) {  // remaining weight fragments, one per step
-      w[t + 1].lo = lds16(ch0, (t + 1) * 2048);
-      w[t + 1].hi = lds16(ch1, (t + 1) * 2048);
+      w[t + 1].lo = lds16(ch0, (t + 1) * W_STRIDE);
+      w[t + 1].hi = lds16(ch1, (t + 1) * W_STRIDE);
     }
     if (i == 0 && j + 1 < MT) {  // next token tile
       tokb[(j + 1) & 1].lo = lds16(tk0, (j + 1) * 2048);
       tokb[(j + 1) & 1].hi = lds16(tk1, (j + 1) * 2048);
     }
-    if (i == 1 && j + 1 < MT) scb[(j + 1) & 1] = scp[(j + 1) * 16] * sbv;
+    if (i == 1 && j + 1 < MT) {
+#pragma unroll
+      for (int b = 0; b < SB; ++b) scb[(j + 1) & 1][b] = scp[(j + 1) * 16] * sbv[b];
+    }
     if (t <= LOADS) issue_one<BM, BN>(s, t, nxt, sc_nxt, kb_next);
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -128,7 +142,7 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
     constexpr int t = MT * T_NT - 1;
     constexpr int pj = t / T_NT, pi = t % T_NT;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[t & 1][v], scb[pj & 1], acc[pi][pj][v]);
+    for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[t & 1][v], scb[pj & 1][SB > 1 ? pi : 0], acc[pi][pj][v]);
   }
 }
 
@@ -145,8 +159,10 @@ __device__ __forceinline__ void wait_and_barrier() {
 // One BM x 256 output tile at (m0, n0), K blocks of split `split`, by the whole workgroup.
 template <int BM, bool SPLIT, int BN = T_BN>
 __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, int split) {
-  static_assert(BN == 128 || BN == 256, "channel tile");
+  static_assert(BN == 128 || BN == 192 || BN == 256, "channel tile");
   constexpr int WM = BM / 2, MT = WM / 16, T_WN = BN / 4, T_NT = T_WN / 16, LOADS = Dma3State<BM, BN>::LOADS;
+  constexpr bool INTERLEAVED = Dma3State<BM, BN>::INTERLEAVED;
+  constexpr int SB = Dma3State<BM, BN>::SB;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -173,7 +189,7 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
       else
         s.goff[i] = (uint32_t)((int64_t)min(n0 + row - BM, p.N - 1) * p.ldb + chunk_byte);
     }
-    const int trow = wave_m * WM + l16, crow = BM + wave_n * T_WN + l16;
+    const int trow = wave_m * WM + l16, crow = BM + wave_n * (INTERLEAVED ? 16 : T_WN) + l16;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       s.tok_off[h] = trow * KSTEP + (((q + 4 * h) ^ (trow & 7)) << 4);
@@ -185,7 +201,11 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   s.sa_base = p.sa;
   s.sa_off = (uint32_t)min(m0 + wave * (BM / 8) + (lane & (BM / 32 - 1)) * 4, (p.M - 1) & ~3) * 4u;
   s.sa_sk = p.sa_sk;
-  s.sb_ptr = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(n0 + wave_n * T_WN, p.N - 1) / 128) * p.sb_sn);
+#pragma unroll
+  for (int b = 0; b < SB; ++b) {
+    const int first = INTERLEAVED ? n0 + 64 * b : n0 + wave_n * T_WN;  // first channel of the wave's tile(s) with this scale
+    s.sb_ptr[b] = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(first, p.N - 1) / 128) * p.sb_sn);
+  }
   s.sb_sk = p.sb_sk;
 
   // three stages: tiles (rows 0..BM-1 tokens, BM.. channels) and the tile's BM token scales, sized per tile shape: a
@@ -213,11 +233,16 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   wait_and_barrier<LOADS + 1>();  // block 0 has landed everywhere
 
   // ---- three blocks per trip over the three stages; iteration k multiplies block k, requests block k + 2
+  auto sb_of = [&](int kb, float (&v)[SB]) {
+#pragma unroll
+    for (int b = 0; b < SB; ++b) v[b] = s.sb_ptr[b][(int64_t)kb * s.sb_sk];
+  };
   int k = 0;
   for (; k + 2 < nkb; k += 3) {
-    const float sb0 = s.sb_ptr[(int64_t)(kb_begin + k) * s.sb_sk];
-    const float sb1 = s.sb_ptr[(int64_t)(kb_begin + k + 1) * s.sb_sk];
-    const float sb2 = s.sb_ptr[(int64_t)(kb_begin + k + 2) * s.sb_sk];
+    float sb0[SB], sb1[SB], sb2[SB];
+    sb_of(kb_begin + k, sb0);
+    sb_of(kb_begin + k + 1, sb1);
+    sb_of(kb_begin + k + 2, sb2);
     k_block<BM, BN>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2);
     wait_and_barrier<LOADS + 1>();
     k_block<BM, BN>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3);
@@ -226,10 +251,15 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
     wait_and_barrier<LOADS + 1>();
   }
   if (k < nkb) {  // one or two blocks left, in stages 0 and 1
-    k_block<BM, BN>(s, t_stage0, t_scale0, s.sb_ptr[(int64_t)(kb_begin + k) * s.sb_sk], acc, t_stage2, t_scale2, kb_begin + k + 2);
+    float sb0[SB];
+    sb_of(kb_begin + k, sb0);
+    k_block<BM, BN>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2);
     wait_and_barrier<LOADS + 1>();
-    if (k + 1 < nkb)
-      k_block<BM, BN>(s, t_stage1, t_scale1, s.sb_ptr[(int64_t)(kb_begin + k + 1) * s.sb_sk], acc, t_stage0, t_scale0, kb_begin + k + 3);
+    if (k + 1 < nkb) {
+      float sb1[SB];
+      sb_of(kb_begin + k + 1, sb1);
+      k_block<BM, BN>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
 
@@ -241,7 +271,7 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
     if (m >= p.M) continue;
 #pragma unroll
     for (int i = 0; i < T_NT; ++i) {
-      const int n = n0 + wave_n * T_WN + i * 16 + 4 * q;
+      const int n = n0 + (INTERLEAVED ? i * 64 + wave_n * 16 : wave_n * T_WN + i * 16) + 4 * q;
       if (n >= p.N) continue;
       const int nvalid = min(4, p.N - n);
       if constexpr (SPLIT) {
@@ -297,8 +327,8 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 // and split count; it names the measured best or a choice within 5 % of it for 22 of them, within 12 % for the others):
 //   * a workgroup spends per K block the largest of
 //       - the tile's own time when operands come from L2: 0.88 us for 128 token rows, 0.58 us for 64 (0.52 / 0.40 with
-//         128 channels; x 1.2 in a round that keeps more than 200 CUs busy; the INT8 kernel: 1.14 / 0.71 / 0.64 / 0.44);
-//       - a latency floor when the weight comes from HBM (two blocks in flight per CU): 1.2 us / 1.0 us (0.7 / 0.51 with
+//         128 channels, 0.68 / 0.50 with 192; x 1.2 in a round that keeps more than 200 CUs busy; the INT8 kernel: 1.14 / 0.71 / 0.64 / 0.44);
+//       - a latency floor when the weight comes from HBM (two blocks in flight per CU): 1.2 us / 1.0 us (1.0 / 0.75 with 192 channels, 0.7 / 0.51 with
 //         128 channels; INT8: 0.96 / 0.68 / 0.59 / 0.54), times 1.2 for weight rows longer than 8 KB;
 //       - its share of the HBM stream: (concurrent workgroups) x (HBM bytes per workgroup and block) / 5.5 TB/s, where
 //         weight rows are shared in L2 by up to 8 token tiles and token rows by up to 8 channel tiles;
@@ -317,16 +347,16 @@ double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int bn, int
   constexpr double HBM_BYTES_PER_US = 5.5e6;
   const int64_t per = (kb_total + sp - 1) / sp;
   const int64_t tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn;
-  // the tile's own time per K block and the latency floor, in the order 128x256, 64x256, 128x128, 64x128 (the INT8 kernel
+  // the tile's own time per K block and the latency floor, in the order 128x256, 64x256, 128x128, 64x128, 128x192, 64x192 (the INT8 kernel
   // of the same structure has its own: fitted to K=4096 -> N=4096..28672 and K=14336 -> N=4096 at 24..1024 tokens)
-  static constexpr double TILE_US[2][4] = {{0.88, 0.58, 0.52, 0.40}, {1.14, 0.71, 0.64, 0.44}};
-  static constexpr double LATENCY_US[2][4] = {{1.2, 1.0, 0.7, 0.51}, {0.96, 0.68, 0.59, 0.54}};
-  const int shape = (bn == 256 ? 0 : 2) + (bm == 128 ? 0 : 1);
+  static constexpr double TILE_US[2][6] = {{0.88, 0.58, 0.52, 0.40, 0.68, 0.50}, {1.14, 0.71, 0.64, 0.44, 0.0, 0.0}};
+  static constexpr double LATENCY_US[2][6] = {{1.2, 1.0, 0.7, 0.51, 1.0, 0.75}, {0.96, 0.68, 0.59, 0.54, 0.0, 0.0}};
+  const int shape = (bn == 256 ? 0 : bn == 128 ? 2 : 4) + (bm == 128 ? 0 : 1);  // ..., 128x192, 64x192 (FP8 only)
   const double t_tile = TILE_US[is_int8][shape];
   const double hbm_per_block = (double)(bn * KSTEP) / (double)std::min<int64_t>(tm, 8) + (double)(bm * KSTEP) / (double)std::min<int64_t>(tn, 8);
-  // latency floor while the weight streams from HBM: with 256 channels per tile when at most two token tiles share it,
-  // with 128 when nobody does (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
-  const bool streams = bn == 256 ? hbm_per_block >= 16384.0 : hbm_per_block >= (double)(bn * KSTEP);
+  // latency floor while the weight streams from HBM: with 256 or 192 channels per tile when at most two token tiles share
+  // it, with 128 when nobody does (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
+  const bool streams = hbm_per_block >= (bn == 192 ? 12288.0 : 16384.0);
   const double t_latency = streams ? LATENCY_US[is_int8][shape] * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
   double t = 0.0;
   for (int64_t left = tm * tn * sp; left > 0;) {
@@ -348,7 +378,8 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8) {
   const int max_split = (N % 4 == 0) ? 16 : 1;  // the reduce kernel works on aligned quads of one row
   double best_time = 1e30;
   pl.bm = 128, pl.bn = T_BN, pl.splits = 1, pl.efficiency = 0.0;
-  for (int bn = T_BN; bn >= 128; bn -= 128) {
+  for (int bn = T_BN; bn >= 128; bn -= 64) {
+    if (bn == 192 && is_int8) continue;  // the INT8 kernel's 32-channel MFMA tiles do not divide 192 / 4
     for (int bm = 64; bm <= 128; bm += 64) {
       if (M <= 64 && bm == 128) break;                 // a second half tile of padding rows buys nothing
       const double tile_factor = (bm == 64 && M > 128) ? 0.65 : 1.0;
@@ -386,6 +417,7 @@ int launch_fp8_grouped_dma3(GroupedParams& gp, int bm, hipStream_t stream, const
 
 int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what) {
   if (bn == 128) return bm == 64 ? launch_bm<64, 128>(p, stream, what) : launch_bm<128, 128>(p, stream, what);
+  if (bn == 192) return bm == 64 ? launch_bm<64, 192>(p, stream, what) : launch_bm<128, 192>(p, stream, what);
   return bm == 64 ? launch_bm<64, 256>(p, stream, what) : launch_bm<128, 256>(p, stream, what);
 }
 

@@ -12,13 +12,15 @@ FP8_ROUTE_SHAPES = [
     # an uneven last workgroup (16640 = 130 groups), short last K ranges (4480 = 35 blocks, 2176 = 17 blocks)
     (1, 128, 128), (3, 256, 512), (1, 512, 7168), (16, 2048, 7168), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432),
     (7, 33280, 4096), (5, 66048, 512), (2, 133120, 384),
-    # three-stage mid-M kernel: 64 / 128 token tiles x 256 / 128 channel tiles, whole-K and split, ragged M, K blocks per
+    # three-stage mid-M kernel: 64 / 128 token tiles x 256 / 192 / 128 channel tiles, whole-K and split, ragged M, K blocks per
     # range = 1, 2, 0 mod 3
     (48, 16384, 2048), (33, 16384, 2176), (40, 65536, 512), (200, 16384, 2048), (100, 32768, 640), (130, 8192, 7168),
     (250, 8192, 7296), (100, 16384, 3584), (500, 4096, 14336),
     # the same kernel with 256-channel tiles and a K split (long K, many channels), and with 128-channel tiles
     (65, 7168, 18432), (24, 36864, 14336), (100, 36864, 640), (40, 4096, 7168), (300, 4096, 7168), (1000, 4096, 2048),
-    (400, 4096, 16384),
+    (400, 4096, 16384), (100, 65536, 512), (130, 4096, 7168),
+    # 192-channel tiles (a wave's three channel tiles are 64 channels apart): whole-K and split, a ragged last tile
+    (100, 36864, 512), (20, 36864, 1024), (130, 3072, 7168), (300, 3072, 14336), (130, 1000, 896),
     # 256 x 256 two-phase and 256 x 128 pipelined kernels, K a multiple of 128 and not
     # (the pipelined kernel takes whole-K shapes only where N % 4 != 0 rules the mid-M kernel's split reduce out)
     (4096, 4352, 512), (4000, 4300, 400), (4096, 2178, 256), (4000, 2100, 272), (4096, 2176, 256),
@@ -36,6 +38,7 @@ FP8_REQUIRED_VARIANTS = {
     ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
     ("dma3", 64, "whole", "bn128"), ("dma3", 64, "split", "bn128"), ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"),
+    ("dma3", 64, "whole", "bn192"), ("dma3", 64, "split", "bn192"), ("dma3", 128, "whole", "bn192"), ("dma3", 128, "split", "bn192"),
     ("pingpong", "kfull"), ("pingpong", "ktail"), ("pipelined", "kfull"), ("pipelined", "ktail"),
     ("generic", 16, "aligned", "whole"), ("generic", 16, "aligned", "split"), ("generic", 16, "bytes", "split"),
     ("generic", 32, "aligned", "split"), ("generic", 32, "bytes", "whole"),
@@ -86,7 +89,7 @@ def variant_of(plan: dict, K: int):
         g = plan["groups_per_wg"]
         return (k, sp, f"gpw{g}" if g < 3 else "gpw3+")
     if k == "dma3":
-        return (k, plan["bm"], sp) if plan["bn"] == 256 else (k, plan["bm"], sp, "bn128")
+        return (k, plan["bm"], sp) if plan["bn"] == 256 else (k, plan["bm"], sp, f"bn{plan['bn']}")
     if k in ("pingpong", "pipelined"):
         return (k, "kfull" if K % 128 == 0 else "ktail")
     return (k, plan["bm"], "aligned" if plan["aligned"] else "bytes", sp)
