@@ -176,3 +176,13 @@ def test_host_checks_reject_bad_operands_with_reference_wording():
     with pytest.raises(NotImplementedError):
         ops.sgl_per_token_group_quant_8bit_v2(torch.zeros(4, 256), a, torch.zeros(4, 2), 128, 1e-10, -448.0, 448.0,
                                               False, True, None)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path is a one-GPU path: bench.py says so instead of launching ranks."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "ONE GPU" in (r.stdout + r.stderr)
