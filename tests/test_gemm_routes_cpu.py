@@ -122,3 +122,6 @@ def test_mid_m_plans_are_consistent():
                 kb = -(-K // 128)
                 assert p["splits"] >= 1 and p["kb_per_split"] >= 1
                 assert p["kb_per_split"] * p["splits"] >= kb and p["kb_per_split"] * (p["splits"] - 1) < kb, (kind, M, N, K, p)
+                if p["kernel"] == "dma3":  # the tile shapes that are compiled: 192 channels for FP8 only, splits need N % 4 == 0
+                    assert p["bm"] in (64, 128) and p["bn"] in ((128, 192, 256) if kind == "fp8" else (128, 256)), (kind, M, N, K, p)
+                    assert p["splits"] == 1 or N % 4 == 0
