@@ -1,0 +1,84 @@
+"""The shape grids of the reference's own operator tests, run through the operators under the reference's names.
+
+sgl-kernel/tests/test_fp8_blockwise_gemm.py:62-85 runs fp8_blockwise_scaled_mm over M x N x K x out_dtype with operands
+drawn uniformly from the whole e4m3fn range, scales ~ N(0, 1e-3) (either sign) laid out M-major, and accepts
+rtol 0.02 / atol 1 against scale-then-multiply in fp32; sgl-kernel/tests/test_int8_gemm.py:20-49 runs int8_scaled_mm over
+M x N x K x bias x out_dtype with int8(N(0, 5)) operands, N(0, 1) scales of either sign and a bias of N(0, 10).
+
+The same grids, operand distributions and (for FP8) the same criterion are used here; the comparison values are built
+with torch on the GPU, as the reference's tests build theirs.  FP8 is floating point, so the reference's tolerance
+applies; the INT8 result is held to the bits: exact integer accumulators (an fp64 matmul is exact at these sizes), then the
+epilogue f32(acc) * (sb[n] * sa[m]) + bias, each step rounded once.  Cases above 2^36 multiply-accumulates are left to
+the curated full-size tests (tests/test_gpu_fp8_gemm.py, tests/test_gpu_int8_gemm.py, tests/test_gpu_config_shapes.py).
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+MAX_MACS = 1 << 36
+
+FP8_M = [1, 3, 5, 127, 128, 512, 1024, 4096]
+FP8_N = [128, 512, 1024, 4096, 8192, 14080]
+FP8_K = [512, 1024, 4096, 8192, 14080, 16384]
+INT8_M = [1, 16, 32, 64, 128, 512, 1024, 4096, 8192]
+INT8_N = [16, 128, 512, 1024, 4096, 8192, 16384]
+INT8_K = [512, 1024, 4096, 8192, 16384]
+
+
+def _m_major(t):
+    return t.t().contiguous().t()
+
+
+@pytest.mark.parametrize("N", FP8_N)
+@pytest.mark.parametrize("K", FP8_K)
+def test_fp8_blockwise_scaled_mm_reference_grid(gpu, N, K):
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    g = torch.Generator(device=gpu).manual_seed(N * 31 + K)
+    w = ((torch.rand(N, K, generator=g, device=gpu) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
+    sb = _m_major(torch.randn(K // 128, N // 128, generator=g, device=gpu) * 0.001)  # shaped like mat_b: [K / 128, N / 128]
+    wb = w.float() * sb.t().repeat_interleave(128, 0).repeat_interleave(128, 1)
+    ran = 0
+    for M in FP8_M:
+        if M * N * K > MAX_MACS:
+            continue
+        print(f"case fp8 M={M} N={N} K={K}", flush=True)
+        a = ((torch.rand(M, K, generator=g, device=gpu) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
+        sa = _m_major(torch.randn(M, K // 128, generator=g, device=gpu) * 0.001)
+        want32 = (a.float() * sa.repeat_interleave(128, 1)) @ wb.t()
+        for out_dtype in (torch.bfloat16, torch.float16):
+            out = fp8_blockwise_scaled_mm(a, w.t(), sa, sb, out_dtype)
+            assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
+            torch.testing.assert_close(out, want32.to(out_dtype), rtol=0.02, atol=1)
+        ran += 1
+    assert ran >= 5  # every (N, K) pair runs at least the five smallest token counts
+
+
+@pytest.mark.parametrize("N", INT8_N)
+@pytest.mark.parametrize("K", INT8_K)
+def test_int8_scaled_mm_reference_grid(gpu, N, K):
+    from sglang_amd.sgl_kernel import int8_scaled_mm
+
+    g = torch.Generator(device=gpu).manual_seed(N * 17 + K)
+    w = (torch.randn(N, K, generator=g, device=gpu) * 5).round().clamp(-128, 127).to(torch.int8)
+    sb = torch.randn(N, generator=g, device=gpu)
+    w64 = w.double()
+    ran = 0
+    for M in INT8_M:
+        if M * N * K > MAX_MACS:
+            continue
+        print(f"case int8 M={M} N={N} K={K}", flush=True)
+        a = (torch.randn(M, K, generator=g, device=gpu) * 5).round().clamp(-128, 127).to(torch.int8)
+        sa = torch.randn(M, generator=g, device=gpu)
+        acc = (a.double() @ w64.t()).to(torch.float32)            # exact integers, rounded once to fp32 like (float)acc
+        scaled = acc * (sb.view(1, N) * sa.view(M, 1))            # f32(acc) * (sb * sa), each product rounded once
+        for out_dtype in (torch.bfloat16, torch.float16):
+            bias = (torch.randn(N, generator=g, device=gpu) * 10).to(out_dtype)
+            for b in (None, bias):
+                out = int8_scaled_mm(a, w.t(), sa, sb, out_dtype, b)
+                want = (scaled if b is None else scaled + b.float().view(1, N)).to(out_dtype)
+                assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
+                assert torch.equal(out.view(torch.int16), want.view(torch.int16)), (M, N, K, out_dtype, b is not None)
+        ran += 1
+    assert ran >= 5  # every (N, K) pair runs at least the five smallest token counts
