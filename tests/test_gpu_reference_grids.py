@@ -82,3 +82,44 @@ def test_int8_scaled_mm_reference_grid(gpu, N, K):
                 assert torch.equal(out.view(torch.int16), want.view(torch.int16)), (M, N, K, out_dtype, b is not None)
         ran += 1
     assert ran >= 5  # every (N, K) pair runs at least the five smallest token counts
+
+
+# ---- sgl-kernel/tests/test_per_token_group_quant_8bit.py:22-59: tokens x hidden x group x {fp8, int8} x four scale layouts,
+# through sglang_per_token_group_quant_8bit(enable_v2=True) as that test calls it.  There the CUDA kernel is compared with
+# the Triton kernel under a tolerance; here codes and scales must equal the CPU oracle's bit for bit, so the inputs are
+# capped at 2^21 elements per case (the full-size configuration has its own test in tests/test_gpu_group_quant.py).
+QUANT_TOKENS = [1, 4, 16, 64, 127, 128, 512, 1024, 4096, 8192]
+QUANT_HIDDEN = [128, 256, 384, 512, 1024, 1536, 1664, 2048, 4096, 7168, 16384]
+QUANT_LAYOUTS = ["row", "col", "col_aligned", "ue8m0"]
+
+
+@pytest.mark.parametrize("hidden", QUANT_HIDDEN)
+@pytest.mark.parametrize("group", [16, 32, 64, 128])
+def test_per_token_group_quant_8bit_reference_grid(gpu, oracle, hidden, group):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_8bit
+    from sglang_amd.workloads import make_activation
+
+    ran = 0
+    for tokens in QUANT_TOKENS:
+        if tokens * hidden > (1 << 21):
+            continue
+        x = make_activation(tokens, hidden, seed=tokens * 13 + hidden + group, zero_group_frac=0.02, group=group)
+        xg = x.to(gpu)
+        for dst in (FP8, torch.int8):
+            for layout in QUANT_LAYOUTS:
+                if (layout == "ue8m0" and group != 128) or (dst == torch.int8 and layout != "row"):
+                    continue  # the combinations the reference's test skips too
+                print(f"case quant tokens={tokens} hidden={hidden} group={group} {dst} {layout}", flush=True)
+                q, s = sglang_per_token_group_quant_8bit(
+                    xg, group, dst, column_major_scales=layout != "row", scale_tma_aligned=layout in ("col_aligned", "ue8m0"),
+                    scale_ue8m0=layout == "ue8m0", enable_v2=True)
+                q_o, s_o = oracle.group_quant(x, group, mode="mul", layout=layout, dst_dtype=dst)
+                assert q.dtype == dst and tuple(s.shape) == tuple(s_o.shape) and s.dtype == s_o.dtype
+                assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8)), (tokens, hidden, group, dst, layout)
+                if layout == "ue8m0":
+                    n = 4 * s.shape[1]
+                    assert torch.equal(oracle.unpack_ue8m0(s.cpu(), n), oracle.unpack_ue8m0(s_o, n))
+                else:
+                    assert torch.equal(s.cpu().contiguous().view(torch.int32), s_o.contiguous().view(torch.int32))
+                ran += 1
+    assert ran >= 12
