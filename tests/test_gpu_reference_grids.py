@@ -123,3 +123,51 @@ def test_per_token_group_quant_8bit_reference_grid(gpu, oracle, hidden, group):
                     assert torch.equal(s.cpu().contiguous().view(torch.int32), s_o.contiguous().view(torch.int32))
                 ran += 1
     assert ran >= 12
+
+
+# ---- sgl-kernel/tests/test_per_token_quant_fp8.py:37-53 and test_per_tensor_quant_fp8.py:39-66: fp16 inputs uniform in
+# [0, 1), tokens x hidden incl. 1368 (rows of 171 16-byte vectors); per-tensor both dynamic and with a given scale.  Those
+# tests re-derive the codes from the kernel's own scale under a tolerance; here codes and scales equal the oracle's bits.
+@pytest.mark.parametrize("tokens", [128, 256, 512])
+@pytest.mark.parametrize("hidden", [512, 1368, 2048, 4096])
+def test_per_token_and_per_tensor_quant_fp8_reference_grid(gpu, oracle, tokens, hidden):
+    from sglang_amd.sgl_kernel import sgl_per_tensor_quant_fp8, sgl_per_token_quant_fp8
+
+    g = torch.Generator().manual_seed(tokens + hidden)
+    x = torch.rand(tokens, hidden, generator=g).to(torch.float16)
+    xg = x.to(gpu)
+    q = torch.empty(tokens, hidden, dtype=FP8, device=gpu)
+    s = torch.zeros(tokens, dtype=torch.float32, device=gpu)
+    sgl_per_token_quant_fp8(xg, q, s)
+    q_o, s_o = oracle.per_token_quant_fp8(x)
+    assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8)) and torch.equal(s.cpu().view(torch.int32), s_o.view(-1).view(torch.int32))
+    for given in (None, torch.rand(1, generator=g)):
+        scale = torch.zeros(1, dtype=torch.float32, device=gpu) if given is None else given.to(gpu)
+        sgl_per_tensor_quant_fp8(xg, q, scale, given is not None)
+        q_o, s_o = oracle.per_tensor_quant_fp8(x, given)
+        assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8)), (tokens, hidden, given)
+        assert torch.equal(scale.cpu().view(torch.int32), s_o.view(torch.int32))
+
+
+# ---- sgl-kernel/tests/test_fp8_gemm.py:39-45: fp8_scaled_mm over M x N x K x bias x out_dtype, full-range codes, per-token
+# and per-channel scales ~ N(0, 1e-3), bias ~ N(0, 1) in the output type; the reference's formula and its rtol 0.02 / atol 1.
+@pytest.mark.parametrize("N", [16, 128, 512, 1024, 4096])
+@pytest.mark.parametrize("K", [512, 1024, 4096, 8192, 16384])
+def test_fp8_scaled_mm_reference_grid(gpu, N, K):
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
+
+    g = torch.Generator(device=gpu).manual_seed(N * 7 + K)
+    w = ((torch.rand(N, K, generator=g, device=gpu) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
+    sb = torch.randn(N, generator=g, device=gpu) * 0.001
+    w32 = w.float()
+    for M in (1, 128, 512, 1024, 4096):
+        print(f"case fp8_scaled_mm M={M} N={N} K={K}", flush=True)
+        a = ((torch.rand(M, K, generator=g, device=gpu) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
+        sa = torch.randn(M, generator=g, device=gpu) * 0.001
+        scaled = (a.float() @ w32.t()) * sa.view(-1, 1) * sb.view(1, -1)
+        for out_dtype in (torch.bfloat16, torch.float16):
+            bias = torch.randn(N, generator=g, device=gpu).to(out_dtype)
+            for b in (None, bias):
+                out = fp8_scaled_mm(a, w.t(), sa, sb, out_dtype, b)
+                want = scaled.to(out_dtype) if b is None else scaled.to(out_dtype) + b.view(1, -1)
+                torch.testing.assert_close(out, want, rtol=0.02, atol=1)
