@@ -171,3 +171,42 @@ def test_fp8_scaled_mm_reference_grid(gpu, N, K):
                 out = fp8_scaled_mm(a, w.t(), sa, sb, out_dtype, b)
                 want = scaled.to(out_dtype) if b is None else scaled.to(out_dtype) + b.view(1, -1)
                 torch.testing.assert_close(out, want, rtol=0.02, atol=1)
+
+
+# ---- python/sglang/test/test_block_fp8.py:326-398 (TestW8A8BlockFP8Matmul), both of its grids: the generic one with ragged
+# N = 7748 and K = 3884 / 5120 / 256 and fp32 / fp16 / bf16 outputs, and the DeepSeek-V3 one; full-range codes, scales
+# uniform in [0, 1e-2), row-major token scales, through fp8_kernel.w8a8_block_fp8_matmul; its criterion
+# mean|out - ref| / mean|ref| < 0.001 against the broadcast-scale fp32 product.
+GENERIC_NK = [(N, K) for N in (128, 512, 1024, 4096, 7748, 13824) for K in (256, 4096, 5120, 3884, 13824)]
+DSV3_NK = [(2112, 7168), (1536, 7168), (3072, 1536), (24576, 7168), (4096, 512), (7168, 2048), (4608, 7168), (512, 7168),
+           (7168, 2304), (7168, 512)]
+
+
+def _block_matmul_case(gpu, N, K, Ms, out_dtypes):
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
+
+    g = torch.Generator(device=gpu).manual_seed(N + K)
+    nt, kt = -(-N // 128), -(-K // 128)
+    w = ((torch.rand(N, K, generator=g, device=gpu) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
+    Bs = torch.rand(nt, kt, generator=g, device=gpu) * 1e-2
+    wb = w.float() * Bs.repeat_interleave(128, 0)[:N].repeat_interleave(128, 1)[:, :K]
+    for M in Ms:
+        print(f"case block matmul M={M} N={N} K={K}", flush=True)
+        a = ((torch.rand(M, K, generator=g, device=gpu) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
+        As = torch.rand(M, kt, generator=g, device=gpu) * 1e-2
+        ref32 = (a.float() * As.repeat_interleave(128, 1)[:, :K]) @ wb.t()
+        for out_dtype in out_dtypes:
+            out = w8a8_block_fp8_matmul(a, w, As, Bs, [128, 128], out_dtype)
+            ref = ref32.to(out_dtype).float()
+            assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
+            assert float((out.float() - ref).abs().mean() / ref.abs().mean()) < 0.001, (M, N, K, out_dtype)
+
+
+@pytest.mark.parametrize("N,K", GENERIC_NK)
+def test_w8a8_block_fp8_matmul_generic_grid(gpu, N, K):
+    _block_matmul_case(gpu, N, K, [1, 7, 83, 512, 2048], [torch.float32, torch.half, torch.bfloat16])
+
+
+@pytest.mark.parametrize("N,K", DSV3_NK)
+def test_w8a8_block_fp8_matmul_deepseek_grid(gpu, N, K):
+    _block_matmul_case(gpu, N, K, [64, 128, 512, 1024, 4096], [torch.bfloat16])
