@@ -210,3 +210,31 @@ def test_w8a8_block_fp8_matmul_generic_grid(gpu, N, K):
 @pytest.mark.parametrize("N,K", DSV3_NK)
 def test_w8a8_block_fp8_matmul_deepseek_grid(gpu, N, K):
     _block_matmul_case(gpu, N, K, [64, 128, 512, 1024, 4096], [torch.bfloat16])
+
+
+# ---- python/sglang/test/test_block_fp8.py:51-92 (TestPerTokenGroupQuantFP8) and :118-158 (TestStaticQuantFP8): inputs uniform
+# in [0, 1) in fp16 / bf16 / fp32, tokens x hidden incl. 5120 and 13824, groups of 64 .. 512.  The reference compares with a
+# torch restatement under rtol 0.15; here the codes and scales equal the oracle's bits (cases above 2^23 elements left out).
+@pytest.mark.parametrize("dtype", [torch.half, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("hidden", [512, 4096, 5120, 13824])
+def test_python_level_quantizer_grids(gpu, oracle, dtype, hidden):
+    from sglang_amd.fp8_kernel import per_token_group_quant_fp8, static_quant_fp8
+
+    for tokens in (7, 83, 2048):
+        if tokens * hidden > (1 << 23):
+            continue
+        g = torch.Generator().manual_seed(tokens + hidden)
+        x = torch.rand(tokens, hidden, generator=g).to(dtype)
+        xg = x.to(gpu)
+        for group in (64, 128, 256, 512):
+            print(f"case group quant tokens={tokens} hidden={hidden} group={group} {dtype}", flush=True)
+            q, s = per_token_group_quant_fp8(xg, group)
+            q_o, s_o = oracle.group_quant(x, group, mode="rcp", layout="row")
+            assert tuple(s.shape) == (tokens, hidden // group)
+            assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8)), (tokens, hidden, group, dtype)
+            assert torch.equal(s.cpu().view(torch.int32), s_o.view(torch.int32))
+        x_s = (x.float().max() / 448.0).reshape(1)
+        q, s = static_quant_fp8(xg, x_s.to(gpu))
+        q_o, _ = oracle.per_tensor_quant_fp8(x, x_s)
+        assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8)), (tokens, hidden, dtype, "static")
+        assert float(s) == float(x_s)
