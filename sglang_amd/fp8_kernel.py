@@ -354,8 +354,8 @@ def prepare_block_fp8_matmul_inputs(
     block_size: List[int],
     output_dtype: torch.dtype = torch.float16,
 ):
-    """Shape contract of fp8_kernel.py:999-1044 (fp32 scales; packed integer scales are a
-    DeepGEMM-only input there and are rejected here)."""
+    """Shape contract of fp8_kernel.py:999-1044: fp32 scales, or int32 words holding four UE8M0 exponent bytes along K
+    (``As`` [..., ceil(ceil(K/bk)/4)], ``Bs`` [N, ceil(ceil(K/bk)/4)], one row of words per weight row)."""
     assert len(block_size) == 2
     block_n, block_k = block_size[0], block_size[1]
 
@@ -365,6 +365,8 @@ def prepare_block_fp8_matmul_inputs(
 
     if As.dtype == torch.float:
         assert ceil_div(A.shape[-1], block_k) == As.shape[-1]
+    elif As.dtype == torch.int:
+        assert ceil_div(ceil_div(A.shape[-1], block_k), 4) == As.shape[-1], f"{A.shape=} {As.shape=} {block_size=}"
     else:
         raise NotImplementedError
 
@@ -378,6 +380,9 @@ def prepare_block_fp8_matmul_inputs(
     if Bs.dtype == torch.float:
         assert ceil_div(N, block_n) == Bs.shape[0]
         assert ceil_div(K, block_k) == Bs.shape[1]
+    elif Bs.dtype == torch.int:
+        assert N == Bs.shape[0], f"{B.shape=} {Bs.shape=} {block_size=}"
+        assert ceil_div(ceil_div(K, block_k), 4) == Bs.shape[1], f"{B.shape=} {Bs.shape=} {block_size=}"
     else:
         raise NotImplementedError
 
@@ -385,6 +390,13 @@ def prepare_block_fp8_matmul_inputs(
     C = A.new_empty(C_shape, dtype=output_dtype)
 
     return M, N, K, C
+
+
+def _unpack_ue8m0_words(words: torch.Tensor, groups: int) -> torch.Tensor:
+    """int32 words [..., ceil(groups/4)] with exponent byte j of word w belonging to K group 4 w + j -> fp32 powers of two
+    [..., groups] (the inverse of the packing of per_token_group_quant_8bit_v2.cu:84-90, :305-329)."""
+    bytes_ = torch.stack([(words >> (8 * j)) & 0xFF for j in range(4)], dim=-1).reshape(*words.shape[:-1], -1)[..., :groups]
+    return (bytes_.to(torch.int32) << 23).view(torch.float32)
 
 
 def w8a8_block_fp8_matmul(
@@ -397,7 +409,9 @@ def w8a8_block_fp8_matmul(
 ) -> torch.Tensor:
     """Block-wise quantized matmul, fp8_kernel.py:1068-1164.  ``B`` is the weight ``[N, K]`` as
     stored, ``Bs`` its ``[ceil(N/128), ceil(K/128)]`` scales, ``As`` the per-token-group scales of
-    ``A``; N and K may be ragged with respect to the 128x128 blocks."""
+    ``A``; N and K may be ragged with respect to the 128x128 blocks.  Scales packed as UE8M0 exponent bytes in int32
+    words (the DeepGEMM operand format, :1016-1019, :1034-1039) are taken as they are when both operands carry them - the
+    matrix instruction applies the exponents - and are expanded to fp32 first when only one side is packed."""
     M, N, K, C = prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size, output_dtype)
     if list(block_size) != [128, 128]:
         raise NotImplementedError("only 128x128 weight blocks with 1x128 activation groups are built")
@@ -405,7 +419,18 @@ def w8a8_block_fp8_matmul(
     assert output_dtype in (torch.float16, torch.bfloat16, torch.float32)
     if M == 0:
         return C
-    ops.block_fp8_matmul(A.view(M, K), B, As.reshape(M, As.shape[-1]), Bs, C.view(M, N))
+    As2d = As.reshape(M, As.shape[-1]) if As.dim() != 2 else As
+    kb = ceil_div(K, 128)
+    if As.dtype == torch.int32 and Bs.dtype == torch.int32 and output_dtype != torch.float32:
+        if M > 1 and As2d.stride(0) != 1:
+            # the kernels read a token's words with stride 1 along tokens (the layout the quantizer writes)
+            As2d = As2d.t().contiguous().t()
+        return ops.fp8_blockwise_mm_ue8m0(A.view(M, K), B, As2d, Bs, output_dtype).view(C.shape)
+    if As.dtype == torch.int32:
+        As2d = _unpack_ue8m0_words(As2d, kb)
+    if Bs.dtype == torch.int32:
+        Bs = _unpack_ue8m0_words(Bs[::128], kb)
+    ops.block_fp8_matmul(A.view(M, K), B, As2d, Bs, C.view(M, N))
     return C
 
 

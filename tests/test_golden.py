@@ -8,6 +8,8 @@ import numpy as np
 import pytest
 import torch
 
+from fp8_tolerance import check_fp8_gemm, magnitudes
+
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "qlinear_golden.npz")
 FP8 = torch.float8_e4m3fn
 
@@ -24,6 +26,18 @@ def _bf16(t):
 
 def _f32(t):
     return t.view(torch.float32)
+
+
+def _dequant_rows(q_u8, s_f32):
+    """codes [R, K] with one scale per 128-wide K group [R, K/128] -> fp32 (the fixtures hold no sum of magnitudes; it is
+    formed here from their operands with plain torch, without the oracle)."""
+    return q_u8.view(FP8).float() * s_f32.repeat_interleave(128, dim=1)[:, : q_u8.shape[1]]
+
+
+def _dequant_blocks(q_u8, s_f32):
+    """codes [N, K] with one scale per 128 x 128 block [N/128, K/128] -> fp32."""
+    n, k = q_u8.shape
+    return q_u8.view(FP8).float() * s_f32.repeat_interleave(128, dim=0)[:n].repeat_interleave(128, dim=1)[:, :k]
 
 
 def test_oracle_reproduces_quant_fixtures(oracle, gold):
@@ -87,9 +101,9 @@ def test_gpu_reproduces_gemm_fixtures(gpu, gold):
     aq, asc = gold["gemm_a_q"].view(FP8).to(gpu), _f32(gold["gemm_a_s_f32"]).to(gpu)
     wq, ws = gold["gemm_w_q"].view(FP8).to(gpu), _f32(gold["gemm_w_s_f32"]).to(gpu)
     ref = _f32(gold["gemm_out_f32"])
-    out = w8a8_block_fp8_matmul(aq, wq, asc, ws, [128, 128], torch.float32).cpu()
-    # floating point: |err| <= 1e-2 |ref| + 1e-4 * (sum of |terms|), here bounded by K * max|term| ~ row scale
-    assert bool(((out - ref).abs() <= 1e-2 * ref.abs() + 1e-4 * ref.abs().max()).all())
+    out = w8a8_block_fp8_matmul(aq, wq, asc, ws, [128, 128], torch.float32)
+    mag = magnitudes(_dequant_rows(gold["gemm_a_q"], _f32(gold["gemm_a_s_f32"])), _dequant_blocks(gold["gemm_w_q"], _f32(gold["gemm_w_s_f32"])))
+    check_fp8_gemm(out, ref, mag, "gemm fixture")
     a, w = gold["int8_a"].to(gpu), gold["int8_w"].to(gpu)
     assert torch.equal(ops.int8_mm_raw_accumulators(a, w.t()).cpu(), gold["int8_acc"])
     out = int8_scaled_mm(a, w.t(), _f32(gold["int8_sa_f32"]).to(gpu), _f32(gold["int8_sb_f32"]).to(gpu), torch.bfloat16,
@@ -159,11 +173,12 @@ def test_gpu_reproduces_the_other_fixtures(gpu, more):
     assert torch.equal(wq.cpu().view(torch.uint8), more["cast_q"]) and torch.equal(ws.cpu().view(torch.int32), more["cast_s_f32"])
     back = block_quant_dequant(wq, ws, [128, 128], torch.bfloat16)
     assert torch.equal(back.cpu().view(torch.int16), more["cast_back_bf16"])
-    # floating point: |err| <= 1e-2 |ref| + 1e-4 * (sum of |terms|), bounded here by the largest |ref| of the matrix
     ref = _f32(more["smm_out_f32"])
     out = fp8_scaled_mm(more["ptq_fp8_q"].view(FP8).to(gpu), more["smm_w_q"].view(FP8).to(gpu).t(), _f32(more["ptq_fp8_s_f32"]).to(gpu),
-                        _f32(more["smm_sb_f32"]).to(gpu), torch.bfloat16, None).float().cpu()
-    assert bool(((out - ref).abs() <= 1e-2 * ref.abs() + 2.0 ** -8 * ref.abs() + 1e-4 * ref.abs().max()).all())
+                        _f32(more["smm_sb_f32"]).to(gpu), torch.bfloat16, None)
+    mag = magnitudes(more["ptq_fp8_q"].view(FP8).float() * _f32(more["ptq_fp8_s_f32"]).reshape(-1, 1),
+                     more["smm_w_q"].view(FP8).float() * _f32(more["smm_sb_f32"]).reshape(-1, 1))
+    check_fp8_gemm(out, ref, mag, "fp8_scaled_mm fixture")
     E, T, N, K = 3, 9, 128, 256
     outg = torch.full((T, N), 7.0, dtype=torch.bfloat16, device=gpu)
     strides = torch.full((E,), K, dtype=torch.int64, device=gpu)
@@ -173,4 +188,8 @@ def test_gpu_reproduces_the_other_fixtures(gpu, more):
         more["grp_offsets"].to(gpu), torch.empty(1 << 20, dtype=torch.uint8, device=gpu))
     ref = _f32(more["grp_out_f32"])
     got = outg.float().cpu()
-    assert bool(((got - ref).abs() <= 1e-2 * ref.abs() + 2.0 ** -8 * ref.abs() + 1e-4 * ref.abs().max()).all())
+    ga = _dequant_rows(more["grp_a_q"], _f32(more["grp_a_s_f32"]))
+    for e, (r0, m) in enumerate(zip(more["grp_offsets"].tolist(), more["grp_sizes"][:, 0].tolist())):
+        if m:
+            mag = magnitudes(ga[r0:r0 + m], _dequant_blocks(more["grp_w_q"][e], _f32(more["grp_w_s_f32"])[e]))
+            check_fp8_gemm(got[r0:r0 + m], ref[r0:r0 + m], mag, f"grouped fixture, expert {e}")

@@ -10,6 +10,7 @@ step; both are covered, and so are K extents whose last exponent word is only pa
 import pytest
 import torch
 
+from fp8_tolerance import check_fp8_gemm
 from sglang_amd.workloads import make_activation, make_fp8_weight
 
 pytestmark = pytest.mark.gpu
@@ -62,9 +63,7 @@ def test_ue8m0_gemm_against_oracle(gpu, oracle, M, N, K):
     g = torch.Generator().manual_seed(M)
     rows = torch.arange(M) if M <= 256 else torch.cat([torch.tensor([0, 127, 128, 255, 256, M - 1]), torch.randperm(M, generator=g)[:26]])
     ref, mag = _reference(oracle, x_q, sa_words, w2, sb_words, rows)
-    err = (out[rows.to(gpu)].float().cpu() - ref).abs()
-    tol = 1e-2 * ref.abs() + 1e-4 * mag
-    assert bool((err <= tol).all()), float((err - tol).max())
+    check_fp8_gemm(out[rows.to(gpu)], ref, mag, f"M={M} N={N} K={K}")
 
 
 @pytest.mark.parametrize("M,N,K", [(4096, 4352, 1152), (16, 2048, 1024), (200, 16384, 640)])
@@ -113,10 +112,40 @@ def test_deepgemm_linear_wrapper(gpu, oracle, M):
     sb = torch.exp2(_unpack_bytes(sb_words, K // 128).float() - 127.0)[::128].contiguous()
     rows = torch.arange(M) if M <= 64 else torch.tensor([0, 1, 255, 256, 4095])
     ref, mag = oracle.fp8_blockwise_mm(q_o[rows].contiguous(), w2.cpu(), sa[rows].contiguous(), sb, torch.float32, want_abs=True)
-    ref = ref + bias.float()[None, :]
-    err = (out.reshape(M, N)[rows.to(gpu)].float().cpu() - ref).abs()
-    tol = 1e-2 * ref.abs() + 1e-4 * mag + 2.0 ** -8 * ref.abs()
-    assert bool((err <= tol).all()), float((err - tol).max())
+    # the wrapper rounds the product to bf16 and then adds the bias (fp8_utils.py:250-254): up to half a unit in the last place of the product, 2^-8 of it
+    check_fp8_gemm(out.reshape(M, N)[rows.to(gpu)], ref + bias.float()[None, :], mag, "deepgemm linear", extra=2.0 ** -8 * ref.abs())
     # an fp32 block scale tensor (a checkpoint that was not re-quantized) takes the ordinary block-FP8 linear
     out2 = deepgemm_w8a8_block_fp8_linear_with_fallback(x.to(gpu), w_q.to(gpu), [128, 128], w_s.to(gpu), None, None)
     assert tuple(out2.shape) == (M, N)
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 4352, 512), (16, 2048, 1024), (6, 640, 1152), (200, 1024, 640)])
+def test_w8a8_block_fp8_matmul_takes_packed_scales(gpu, oracle, M, N, K):
+    """python/sglang/srt/layers/quantization/fp8_kernel.py:1016-1019, :1034-1039: `w8a8_block_fp8_matmul` and
+    `prepare_block_fp8_matmul_inputs` accept scales packed as UE8M0 exponent bytes in int32 words, [..., ceil(K/512)] for
+    the activation and [N, ceil(K/512)] for the weight.  With both operands packed the result is the UE8M0 kernel's, bit
+    for bit, for 2-D and batched activations and for token words that are not packed along tokens; with one side packed
+    and the other fp32 the packed side is expanded first and the result is held against the oracle."""
+    from sglang_amd.fp8_kernel import prepare_block_fp8_matmul_inputs, w8a8_block_fp8_matmul, w8a8_block_fp8_matmul_deepgemm
+
+    x_q, sa_words, w2, sb_words = _operands(M, N, K, gpu, 5 * M + N + K)
+    assert sa_words.dtype == torch.int32 and tuple(sa_words.shape) == (M, (K // 128 + 3) // 4)
+    assert prepare_block_fp8_matmul_inputs(x_q, w2, sa_words, sb_words, [128, 128], torch.bfloat16)[:3] == (M, N, K)
+    want = w8a8_block_fp8_matmul_deepgemm(x_q, w2, sa_words, sb_words, [128, 128], torch.bfloat16)
+    got = w8a8_block_fp8_matmul(x_q, w2, sa_words, sb_words, [128, 128], torch.bfloat16)
+    assert got.dtype == torch.bfloat16 and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # words stored row-major instead of along tokens, and a leading batch dimension
+    got = w8a8_block_fp8_matmul(x_q.view(2, M // 2, K), w2, sa_words.contiguous().view(2, M // 2, -1), sb_words, [128, 128], torch.bfloat16)
+    assert tuple(got.shape) == (2, M // 2, N) and torch.equal(got.view(M, N).view(torch.int16), want.view(torch.int16))
+    g = torch.Generator().manual_seed(M)
+    rows = torch.arange(M) if M <= 256 else torch.cat([torch.tensor([0, 255, 256, M - 1]), torch.randperm(M, generator=g)[:28]])
+    ref, mag = _reference(oracle, x_q, sa_words, w2, sb_words, rows)
+    KB = K // 128
+    sa_f32 = torch.exp2(_unpack_bytes(sa_words, KB).float() - 127.0).to(gpu)
+    sb_f32 = torch.exp2(_unpack_bytes(sb_words, KB).float() - 127.0)[::128].contiguous().to(gpu)
+    for As, Bs in ((sa_words, sb_f32), (sa_f32, sb_words)):
+        mixed = w8a8_block_fp8_matmul(x_q, w2, As, Bs, [128, 128], torch.float16)
+        assert mixed.dtype == torch.float16
+        check_fp8_gemm(mixed[rows.to(gpu)], ref, mag, f"mixed scales M={M} N={N} K={K}")
+    with pytest.raises(AssertionError):
+        w8a8_block_fp8_matmul(x_q, w2, sa_words[:, :0], sb_words, [128, 128], torch.bfloat16)

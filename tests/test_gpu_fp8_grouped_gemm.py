@@ -9,6 +9,7 @@ product) is reproduced in test_reference_acceptance_criterion with this package'
 import pytest
 import torch
 
+from fp8_tolerance import check_fp8_gemm
 pytestmark = pytest.mark.gpu
 FP8 = torch.float8_e4m3fn
 
@@ -41,12 +42,7 @@ def _call(gpu, a, w, sa, sw, sizes, offsets, out_dtype, out=None, workspace_byte
 
 
 def _check_expert(out_rows, ref, mag, what):
-    out_rows = out_rows.float().cpu()
-    assert bool(torch.isfinite(out_rows).all()), what
-    err = (out_rows - ref).abs()
-    tol = 1e-2 * ref.abs() + 1e-4 * mag + 2.0 ** -8 * ref.abs()
-    bad = err > tol
-    assert not bool(bad.any()), f"{what}: {int(bad.sum())} elements out of tolerance, worst {float((err - tol).max())}"
+    check_fp8_gemm(out_rows, ref, mag, what)
 
 
 def _problem(sizes, N, K, seed, gap=0):

@@ -4,6 +4,7 @@ fp8_scaled_mm (|out - ref| <= 1e-2 * |ref| + 1e-4 * mag as in tests/test_gpu_per
 import pytest
 import torch
 
+from fp8_tolerance import check_fp8_gemm
 from sglang_amd.workloads import make_activation
 
 pytestmark = pytest.mark.gpu
@@ -109,6 +110,4 @@ def test_apply_fp8_linear_paths(gpu, oracle, path):
     assert tuple(out.shape) == (5, 9, N) and out.dtype == torch.bfloat16
     ref, mag = oracle.fp8_scaled_mm(q_o, w, sa.contiguous(), ws, torch.float32, None, want_abs=True)
     ref = ref + bias.float()[None, :]
-    err = (out.reshape(M, N).float().cpu() - ref).abs()
-    tol = 1e-2 * ref.abs() + 1e-4 * mag + 2.0 ** -8 * ref.abs()  # plus the bf16 rounding of the output
-    assert bool((err <= tol).all()), float((err - tol).max())
+    check_fp8_gemm(out.reshape(M, N), ref, mag, path)

@@ -5,6 +5,7 @@ criterion rtol 0.02 / atol 1 against its torch formula, sgl-kernel/tests/test_fp
 import pytest
 import torch
 
+from fp8_tolerance import check_fp8_gemm
 from sglang_amd.workloads import make_activation
 
 pytestmark = pytest.mark.gpu
@@ -77,13 +78,8 @@ def test_fp8_scaled_mm(gpu, oracle, M, N, K, with_bias, out_dtype):
     ref, mag = oracle.fp8_scaled_mm(a[rows].contiguous(), w, sa[rows], sb, torch.float32, None, want_abs=True)
     if with_bias:
         ref = ref + bias.float()[None, :]
-    got = out[rows.to(gpu)].float().cpu()
-    assert bool(torch.isfinite(got).all())
-    err = (got - ref).abs()
-    tol = 1e-2 * ref.abs() + 1e-4 * mag + (2.0 ** -8 * bias.float().abs()[None, :] if with_bias else 0)
-    if out_dtype == torch.float16:
-        tol = tol + 2.0 ** -24  # one step of the fp16 subnormal grid: the products of two 1e-3 scales reach down there
-    assert bool((err <= tol).all()), float((err - tol).max())
+    # fp16 only: one step of the subnormal grid, the products of two 1e-3 scales reach down there
+    check_fp8_gemm(out[rows.to(gpu)], ref, mag, f"M={M} N={N} K={K}", extra=2.0 ** -24 if out_dtype == torch.float16 else 0.0)
     # the reference's own test: torch formula, bias added after the cast
     o = (a[rows].float() @ w.float().T) * sa[rows].view(-1, 1) * sb.view(1, -1)
     o = o.to(out_dtype)
@@ -128,7 +124,6 @@ def test_apply_fp8_linear(gpu, oracle, shape, N, K):
     xq, xs = oracle.per_token_quant_fp8(x.view(M, K))
     ref, mag = oracle.fp8_scaled_mm(xq, w_q, xs, w_s, torch.float32, None, want_abs=True)
     ref = ref + bias.float()[None, :]
-    err = (out.float().cpu().view(M, N) - ref).abs()
-    assert bool((err <= 1e-2 * ref.abs() + 1e-4 * mag + 2.0 ** -8 * bias.float().abs()[None, :]).all())
+    check_fp8_gemm(out.view(M, N), ref, mag, "apply_fp8_linear")
     full = x.view(M, K).float() @ w.T + bias.float()
     assert float((out.float().cpu().view(M, N) - full).norm() / full.norm()) < 0.05
