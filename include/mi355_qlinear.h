@@ -181,6 +181,19 @@ int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, const float* sa
                                    int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo, void* stream);
 
 /*
+ * Measurement aid, not an operator (no counterpart in the reference): the large-M kernel of mi355_fp8_blockwise_mm with
+ * the global loads of its K loop taken out.  K blocks 0 and 1 and the token scales of blocks 0..3 are fetched once;
+ * every later K block multiplies those again, so the matrix instructions, promotion FMAs, LDS reads, barriers and the
+ * epilogue are the operator's, on the operator's operand values, and `out` is NOT the product.  Timed beside the
+ * operator on the same buffers it gives the ceiling the schedule and the chip's sustained clock set once memory is out
+ * of the picture (bench.py --workload fp8_ceiling).  Accepts only shapes the operator runs on that kernel, with K a
+ * multiple of 128 (at least 512) and M-major token scales (sa_sm == 1, sa_sk % 4 == 0, 16-byte aligned base).
+ */
+int mi355_fp8_blockwise_mm_kloop_ceiling(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                         int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                         int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo, void* stream);
+
+/*
  * Per-token x per-channel INT8 GEMM:  acc = sum_k a[m,k] * b[n,k] exactly in int32;
  *   out[m,n] = cast( f32(acc) * (sb[n] * sa[m]) + f32(bias[n]) ).
  * Replaces int8_scaled_mm (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; epilogue order of

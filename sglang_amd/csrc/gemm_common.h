@@ -17,6 +17,13 @@ constexpr int KSTEP = 128;   // bytes of K per row and stage
 constexpr int THREADS = 256;
 constexpr int GROUP_M = 8;    // M-tiles per group in the tile order
 
+// ---- measured constants of the dispatcher's time models (the shapes and runs they come from are listed with the
+// models that use them; tests/test_gemm_routes_cpu.py holds the benchmark shapes on their kernels under +-10 % changes)
+constexpr int NUM_CUS = 256;
+// two-phase 256 x 256 kernels: a round of tiles takes (K blocks) * US_PER_KBLOCK + US_PER_TILE, whatever part of the
+// tile is filled (K sweep at M = 4096, N = 36864: slope and intercept of the tile time)
+constexpr double PP_FP8_US_PER_KBLOCK = 1.39, PP_INT8_US_PER_KBLOCK = 1.46, PP_US_PER_TILE = 11.0;
+
 struct GemmParams {
   const uint8_t* a;  // tokens   [M, K], row stride lda
   const uint8_t* b;  // channels [N, K], row stride ldb
@@ -157,6 +164,8 @@ int launch_fp8_pipelined(GemmParams& p, hipStream_t stream, const char* what);
 // Large-M blockwise FP8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases);
 // gemm_fp8_pp.hip.  Same requirements.
 int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what);
+// The K loop of launch_fp8_pp without its global loads: a measurement aid (see gemm_fp8_pp.hip).  K % 128 == 0.
+int launch_fp8_pp_noload(GemmParams& p, hipStream_t stream, const char* what);
 // The same kernel for packed power-of-two (UE8M0) scales on both operands, applied by the MFMA itself: p.sa / p.sb point
 // to 32-bit words of four exponent bytes (see fp8_gemm_pp_kernel).  K % 128 == 0.
 int launch_fp8_pp_ue8m0(GemmParams& p, hipStream_t stream, const char* what);

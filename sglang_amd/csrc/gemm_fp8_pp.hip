@@ -286,8 +286,11 @@ __device__ __forceinline__ void row_col_epilogue(const GemmParams& p, int m, int
 //                 (n, kw) at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb; the MFMA applies them;
 //   SM_EPILOGUE   one scale per token (p.row_scale) and per channel (p.col_scale), applied once, after the K loop, as
 //                 row_scale * (col_scale * acc) + bias; the K loop accumulates in the MFMA with unit scales.
+// NOLOAD (a measurement aid, never the product): K blocks 0 and 1 and the token scales of blocks 0..3 are fetched once and
+// every later K block multiplies those again, so the loop is the product's instruction stream on the product's operand
+// values minus its global loads; what it leaves out is what the loads cost.
 // One 256 x 256 output tile at (m0, n0) by the whole workgroup.
-template <bool KFULL, int SM>
+template <bool KFULL, int SM, bool NOLOAD = false>
 __device__ __forceinline__ void pp_tile(const GemmParams& p, const int m0, const int n0) {
   constexpr bool UE8M0 = SM == SM_UE8M0;
   constexpr bool HW_SCALE = SM != SM_BLOCK_F32;  // scale operands of the MFMA instead of promotion FMAs
@@ -354,7 +357,14 @@ __device__ __forceinline__ void pp_tile(const GemmParams& p, const int m0, const
   issue_set_b<KFULL>(s, g_stage0, 0);
   issue_set_a<KFULL, UE8M0>(s, g_stage1, 1);
   float sb_cur = s.sb_ptr[0];
-  asm volatile("s_waitcnt vmcnt(7)\n\ts_barrier" ::: "memory");  // block 0 is in LDS (set A of block 1 may be in flight)
+  if constexpr (NOLOAD) {
+    issue_set_b<KFULL>(s, g_stage1, 1);
+    issue_scales<UE8M0>(s, 2);
+    issue_scales<UE8M0>(s, 3);
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(7)\n\ts_barrier" ::: "memory");  // block 0 is in LDS (set A of block 1 may be in flight)
+  }
   if (grp == 1) compute_end();  // group 1 runs one phase behind group 0
 
   // One K block: M0, C0, M1, C1.  `cur` holds block kb; `nxt` takes set B of block kb + 1, `cur` set A of block kb + 2.
@@ -364,14 +374,14 @@ __device__ __forceinline__ void pp_tile(const GemmParams& p, const int m0, const
     const int w_scale = UE8M0 ? (int)(__float_as_uint(sbv) >> ((kb & 3) * 8)) : 127;
     if constexpr (!HW_SCALE) retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
     read_operands<0, SM>(s, cur, sc_cur, sbv, kb, w, tok, scb);
-    issue_set_b<KFULL>(s, nxt, kb + 1);
+    if constexpr (!NOLOAD) issue_set_b<KFULL>(s, nxt, kb + 1);
     memory_end();
     if constexpr (HW_SCALE) compute_ue8m0<0>(w, tok, scb, w_scale, acc);
     else compute<0>(w, tok, scb, acc, pd);
     compute_end();
     if constexpr (!HW_SCALE) retire<0>(pd, acc);
     read_operands<1, SM>(s, cur, sc_cur, sbv, kb, w, tok, scb);
-    issue_set_a<KFULL, UE8M0>(s, cur, kb + 2);
+    if constexpr (!NOLOAD) issue_set_a<KFULL, UE8M0>(s, cur, kb + 2);
     memory_end();
     if constexpr (HW_SCALE) compute_ue8m0<1>(w, tok, scb, w_scale, acc);
     else compute<1>(w, tok, scb, acc, pd);
@@ -423,10 +433,10 @@ __device__ __forceinline__ void pp_tile(const GemmParams& p, const int m0, const
   }
 }
 
-template <bool KFULL, int SM>
+template <bool KFULL, int SM, bool NOLOAD = false>
 __global__ __launch_bounds__(G_THREADS) void fp8_gemm_pp_kernel(const GemmParams p) {
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
-  pp_tile<KFULL, SM>(p, tc.tile_m * G_BM, tc.tile_n * G_BN);
+  pp_tile<KFULL, SM, NOLOAD>(p, tc.tile_m * G_BM, tc.tile_n * G_BN);
 }
 
 // Grouped problems (see GroupedParams): the workgroup's token tile comes from the table the plan kernel wrote, the
@@ -457,6 +467,15 @@ int launch_fp8_pp(GemmParams& p, hipStream_t stream, const char* what) {
     hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, SM_BLOCK_F32>), grid, dim3(G_THREADS), 0, stream, p);
   else
     hipLaunchKernelGGL((fp8_gemm_pp_kernel<false, SM_BLOCK_F32>), grid, dim3(G_THREADS), 0, stream, p);
+  return check_launch(what);
+}
+
+// The K loop of launch_fp8_pp without its global loads (NOLOAD above): a measurement aid.  K % 128 == 0, K >= 512.
+int launch_fp8_pp_noload(GemmParams& p, hipStream_t stream, const char* what) {
+  p.tiles_m = (p.M + G_BM - 1) / G_BM;
+  p.tiles_n = (p.N + G_BN - 1) / G_BN;
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  hipLaunchKernelGGL((fp8_gemm_pp_kernel<true, SM_BLOCK_F32, true>), grid, dim3(G_THREADS), 0, stream, p);
   return check_launch(what);
 }
 

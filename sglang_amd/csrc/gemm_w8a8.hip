@@ -321,8 +321,6 @@ struct Plan {
 // tiles, two workgroups per CU) does better
 constexpr double DMA3_MIN_EFFICIENCY = 0.30;
 
-constexpr int NUM_CUS = 256;
-
 // Tile and split selection.  Large token counts are MFMA-bound and want the biggest tile; small ones
 // stream the weight once and want enough workgroups in flight to cover HBM latency.
 Plan make_plan(int64_t M, int64_t N, int64_t K) {
@@ -445,7 +443,7 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
     // where the channels alone give it a round's worth of tiles (measured: K=7168 -> N=36864 at M=256: 89 against 141 us,
     // M=1024: 260 against 308 us; INT8 K=4096 -> N=28672 at M=512: 59 against 94 us) and loses for few channels.
     if (M > 128) {
-      const double pp_us = (double)((tiles_256 + NUM_CUS - 1) / NUM_CUS) * ((double)(K / KSTEP) * (is_fp8 ? 1.39 : 1.46) + 11.0);
+      const double pp_us = (double)((tiles_256 + NUM_CUS - 1) / NUM_CUS) * ((double)(K / KSTEP) * (is_fp8 ? PP_FP8_US_PER_KBLOCK : PP_INT8_US_PER_KBLOCK) + PP_US_PER_TILE);
       if (pp_us < dp.time_us) {
         r.kernel = RK_PINGPONG, r.bm = 256, r.bn = 256, r.splits = 1, r.kb_per_split = (int)(K / KSTEP);
         return r;
@@ -764,6 +762,24 @@ extern "C" int mi355_fp8_blockwise_mm_ue8m0(const void* a, const void* b, const 
   p.sa = sa_f, p.sa_sm = 1, p.sa_sk = ldm;
   p.sb = sb_f, p.sb_sn = KB, p.sb_sk = 1;
   return run_gemm<true>(p, static_cast<uint8_t*>(workspace) + head, workspace_bytes_given - head, st, what);
+}
+
+extern "C" int mi355_fp8_blockwise_mm_kloop_ceiling(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                                    int out_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                                    int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo,
+                                                    void* stream) {
+  const char* what = "mi355_fp8_blockwise_mm_kloop_ceiling";
+  GemmParams p;
+  bool empty;
+  const int rc = fp8_mm_params(what, a, b, sa, sb, out, out_dtype, M, N, K, lda, ldb, sa_sm, sa_sk, sb_sn, sb_sk, ldo, p, empty);
+  if (rc != MI355_OK || empty) return rc;
+  p.kb_total = (p.K + KSTEP - 1) / KSTEP;
+  const Route r = choose_route(true, p.M, p.N, p.K, p.lda, p.ldb, operands_aligned(p));
+  MI355_REQUIRE(r.kernel == RK_PINGPONG && K % KSTEP == 0 && K >= 4 * KSTEP && fp8_scales_conform(p), MI355_ERR_UNSUPPORTED,
+                "%s: only for shapes that take the two-phase kernel, K a multiple of 128 and at least 512, token scales M-major "
+                "with a pitch that is a multiple of four floats and a 16-byte aligned base", what);
+  p.splits = 1, p.kb_per_split = p.kb_total;
+  return launch_fp8_pp_noload(p, static_cast<hipStream_t>(stream), what);
 }
 
 extern "C" int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, const float* sa, const float* sb, void* out,
