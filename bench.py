@@ -18,6 +18,10 @@ Infinity Cache.
   fp8_ue8m0:M:K:N  the same linear with power-of-two (UE8M0) scales on both operands
   fp8_linear:M:K:N  a whole block-FP8 linear, bf16 in -> bf16 out, one call (fp8_linear2: quantizer call + GEMM call)
   fp8_grouped:E:ROWS:K:N  grouped FP8 GEMM of E experts with ROWS token rows each (mixture-of-experts)
+  fp8_ceiling[:M:K:N]  the large-M FP8 kernel with the global loads of its K loop taken out, on the headline's operands
+               (what schedule and sustained clock allow once memory is out of the picture; the result is not the product)
+  mfma_stream  the kernels' fp8 matrix-instruction streams with all operands in registers, on every CU at once: what the
+               chip's power management lets the matrix pipes sustain on the benchmark's operand values (and on zeros)
   copy         a plain 256 MiB device copy (calibration of the HBM traffic counters)
   silu_quant   silu(gate) * up fused in front of the group quantizer (packed UE8M0 scales)
   per_token_fp8 / per_token_int8 / per_tensor_fp8 / block_cast   the other quantizers of the path
@@ -113,18 +117,19 @@ def _cpu_time_boxed(fn, seconds=10.0):
 
 
 def _roofline(flops, nbytes, st, peak_ops, unit_ops):
-    """Which roof binds (time at peak MFMA rate vs time at peak HBM rate) and the achieved fraction of it.  The
-    duration is the median of the per-launch HIP-event times; for launches under 0.1 ms, where the two event records
-    around a launch cost a visible share of it, the smaller of that median and the average over the event-bracketed
-    run of back-to-back launches (which still holds the launch gaps and, for split K, the reduce kernel)."""
-    ms = st["median"] if st["median"] >= 0.1 else min(st["median"], st["b2b"])
+    """Which roof binds (time at peak MFMA rate vs time at peak HBM rate) and the achieved fraction of it.  ONE basis
+    for every row: `achieved` and `frac` use the MEDIAN of the per-launch HIP-event durations.  `frac_b2b` is the same
+    fraction on the average over the event-bracketed run of back-to-back launches, printed beside it: for launches of
+    tens of microseconds the two event records around each launch cost a visible share of the median, while the
+    back-to-back figure hides the tail of one launch behind the head of the next."""
+    ms = st["median"]
     if flops / (peak_ops * 1e12) >= nbytes / (HBM_PEAK_GBS * 1e9):
         a = flops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "achieved": a, "peak": peak_ops, "unit": unit_ops, "frac": a / peak_ops, "traffic": None,
-                "per_launch": flops}
+                "per_launch": flops, "basis": "median launch", "frac_b2b": flops / (st["b2b"] * 1e-3) / 1e12 / peak_ops}
     a = nbytes / (ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": a / HBM_PEAK_GBS, "traffic": None,
-            "per_launch": nbytes}
+            "per_launch": nbytes, "basis": "median launch", "frac_b2b": nbytes / (st["b2b"] * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
 # ------------------------------------------------------------------------------------------ quantizer
@@ -401,6 +406,95 @@ def bench_fp8_grouped_gemm(E, m_per, K, N, steps, warmup):
     }
 
 
+def bench_fp8_ceiling(M, K, N, steps, warmup):
+    """The large-M FP8 kernel with the global loads of its K loop taken out (mi355_fp8_blockwise_mm_kloop_ceiling), on the
+    operands of bench_fp8_gemm.  `value` is what the matrix instructions, promotion FMAs, LDS reads, barriers and epilogue
+    of the operator sustain on these operand values when nothing is fetched inside the loop; the operator itself is timed
+    in the same call on the same buffers ("operator_ms")."""
+    import torch
+
+    from sglang_amd import _lib, fp8_kernel
+    from sglang_amd.workloads import fp8_gemm_algorithmic_bytes, gemm_flops, make_activation
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(N * 10007 + K)
+    nbuf = 2
+    ws, wss = zip(*[device_block_fp8_weight(N, K, gen, dev) for _ in range(nbuf)])
+    x = make_activation(M, K).to(dev)
+    x_q, x_s = fp8_kernel.per_token_group_quant_fp8(x, 128, column_major_scales=True)
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nbuf)]
+    wsb = L.mi355_fp8_blockwise_mm_workspace_bytes(M, N, K)
+    wsbuf = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+    common = [(x_q.data_ptr(), ws[i].data_ptr(), x_s.data_ptr(), wss[i].data_ptr(), outs[i].data_ptr(), _lib.BF16, M, N, K,
+               x_q.stride(0), ws[i].stride(0), x_s.stride(0), x_s.stride(1), wss[i].stride(0), wss[i].stride(1),
+               outs[i].stride(0)) for i in range(nbuf)]
+
+    def operator(i):
+        _lib.check(L.mi355_fp8_blockwise_mm(*common[i], wsbuf.data_ptr(), wsb, stream))
+
+    def ceiling(i):
+        _lib.check(L.mi355_fp8_blockwise_mm_kloop_ceiling(*common[i], stream))
+
+    _, ms_op, b2b_op = _time_launches(operator, nbuf, steps, warmup)
+    wall, ms, b2b = _time_launches(ceiling, nbuf, steps, warmup)
+    st, st_op = _stats(ms, b2b), _stats(ms_op, b2b_op)
+    flops, nbytes = gemm_flops(M, N, K), fp8_gemm_algorithmic_bytes(M, N, K)
+    return {
+        "workload": f"fp8_ceiling M={M} K={K} N={N} (the large-M FP8 kernel without the global loads of its K loop; not the product)",
+        "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
+        "dtype": "fp8(e4m3fn) MFMA, f32 accumulate", "kernel": "pingpong, K-loop loads removed",
+        "roofline": _roofline(flops, nbytes, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
+        "operator_ms": st_op, "operator_frac": flops / (st_op["median"] * 1e-3) / 1e12 / FP8_PEAK_TFLOPS,
+    }
+
+
+def bench_mfma_stream(steps, warmup):
+    """The fp8 matrix-instruction streams of the large-M kernels with every operand in registers (mi355_probe_fp8_mfma_stream),
+    256 workgroups of 8 waves: fp32-scale stream (C = 0 + four promotion FMAs), in-place stream, MFMA only; each on operand
+    values distributed like the benchmark's (quantized N(0,1) activations x block-quantized N(0, 0.02) weights) and on zeros."""
+    import torch
+
+    from sglang_amd import _lib, fp8_kernel
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    n = 8 * 4 * 64 * 32
+    x = torch.randn(n // 128, 128, generator=gen, device=dev).to(torch.bfloat16)
+    a_real, _ = fp8_kernel.per_token_group_quant_fp8(x, 128)
+    w_q, _ = device_block_fp8_weight(n // 128, 128, gen, dev)
+    zeros = torch.zeros(n, dtype=torch.uint8, device=dev)
+    out = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    iters = 2000
+    flops = 256.0 * 8 * iters * 16 * 2 * 16 * 16 * 128
+    rows = []
+    for data, (pa, pb) in (("benchmark operand values", (a_real, w_q)), ("zeros", (zeros, zeros))):
+        for mode, name in ((0, "C=0 + 4 promotion FMAs per MFMA (fp32-scale kernel)"), (1, "accumulate in place (UE8M0 kernel)"),
+                           (2, "MFMA only")):
+            def step(i, mode=mode, pa=pa, pb=pb):
+                _lib.check(L.mi355_probe_fp8_mfma_stream(mode, 256, iters, pa.data_ptr(), pb.data_ptr(), out.data_ptr(), stream))
+
+            wall, ms, b2b = _time_launches(step, 1, max(10, steps // 2), 3)
+            st = _stats(ms, b2b)
+            tf = flops / (st["median"] * 1e-3) / 1e12
+            rows.append({"stream": name, "operands": data, "ms": st["median"], "TFLOP/s": tf, "frac": tf / FP8_PEAK_TFLOPS,
+                         # two waves per SIMD issue 32-cycle instructions back to back: the clock at which the time fits
+                         "clock_GHz_if_pipe_full": 2.0 * iters * 16 * 32 / (st["median"] * 1e-3) / 1e9})
+    head = rows[0]
+    st = {"median": head["ms"], "p20_p80": [head["ms"], head["ms"]], "b2b": head["ms"]}
+    return {
+        "workload": "mfma_stream (fp8 16x16x128 matrix instructions, operands in registers, 256 workgroups x 8 waves; not a GEMM)",
+        "value": head["TFLOP/s"], "unit": "TFLOP/s", "ms_per_step": head["ms"], "kernel_ms": st,
+        "dtype": "fp8(e4m3fn) MFMA, f32 accumulate", "kernel": "mfma_stream",
+        "roofline": _roofline(flops, 0.0, st, FP8_PEAK_TFLOPS, "TFLOP/s"), "streams": rows,
+    }
+
+
 def bench_fp8_linear(M, K, N, steps, warmup, two_step):
     """A whole block-FP8 linear from bf16 activations to bf16 output: the one-call entry point (at decode sizes the GEMM
     kernel quantizes in its prologue), or, with two_step, quantizer call + GEMM call as the reference's wrappers do."""
@@ -652,6 +746,10 @@ def _short(rec):
            "bound": ro["bound"], "frac": ro["frac"]}
     if "kernel" in rec:
         row["kern"] = rec["kernel"]
+    if "operator_frac" in rec:
+        row["operator_frac_same_call"] = rec["operator_frac"]
+    if "streams" in rec:
+        row["streams"] = [{"s": x["stream"], "on": x["operands"], "frac": x["frac"], "GHz": x["clock_GHz_if_pipe_full"]} for x in rec["streams"]]
     for k in ("cpu_baseline", "cpu_torch_native", "cpu_w8a16_shape"):
         if k in rec:
             row[k] = {"v": rec[k]["value"], "u": rec[k]["unit"], "cores": rec[k]["cores"], "kind": rec[k]["kind"],
@@ -698,6 +796,15 @@ def main():
         rec = bench_quant(S, W, wl == "quant_ue8m0", cpu)
     elif wl == "copy":
         rec = bench_copy(S, W)
+    elif wl == "mfma_stream":
+        rec = bench_mfma_stream(S, W)
+    elif wl.startswith("fp8_ceiling"):
+        parts = wl.split(":")
+        K, N = DSV3_MLP["gate_up"]
+        M = 4096
+        if len(parts) == 4:
+            M, K, N = int(parts[1]), int(parts[2]), int(parts[3])
+        rec = bench_fp8_ceiling(M, K, N, S, W)
     elif wl == "silu_quant":
         rec = bench_silu_quant(S, W)
     elif wl in ("per_token_fp8", "per_token_int8", "per_tensor_fp8", "block_cast"):
@@ -731,6 +838,8 @@ def main():
         K, N = DSV3_MLP["gate_up"]
         rec = bench_fp8_gemm("gate_up", 4096, K, N, S, W, cpu)
         if full:
+            also.append(bench_fp8_ceiling(4096, K, N, S, W))
+            also.append(bench_mfma_stream(S, W))
             also.append(bench_fp8_ue8m0_gemm("gate_up", 4096, K, N, S, W))
             also.append(bench_silu_quant(S, W))
             # expert GEMMs of DeepSeek-R1 (shapes of the reference's grouped-GEMM benchmark): prefill TP=8, prefill EP=16, decode EP=8
@@ -760,7 +869,7 @@ def main():
         "dtype": rec["dtype"], "data": DATA, "config": {"workload": rec["workload"]},
         "roofline": rec["roofline"], "kernel_ms": rec["kernel_ms"],
     }
-    for k in ("kernel", "cpu_baseline", "cpu_torch_native"):
+    for k in ("kernel", "cpu_baseline", "cpu_torch_native", "operator_ms", "operator_frac", "streams"):
         if k in rec:
             line[k] = rec[k]
     if also:

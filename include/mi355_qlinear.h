@@ -194,6 +194,16 @@ int mi355_fp8_blockwise_mm_kloop_ceiling(const void* a, const void* b, const flo
                                          int64_t sa_sm, int64_t sa_sk, int64_t sb_sn, int64_t sb_sk, int64_t ldo, void* stream);
 
 /*
+ * Measurement aid, not an operator (no counterpart in the reference): the fp8 matrix-instruction stream of the large-M
+ * kernels with every operand in registers (no LDS, no global loads, no barriers), `workgroups` workgroups of 8 waves,
+ * `iters` rounds of 16 instructions of 2 * 16 * 16 * 128 FLOP per wave.  mode 0: C = 0 and four promotion FMAs per result
+ * (the fp32-scale kernel's compute phase); 1: accumulating in place (the UE8M0 kernel's); 2: C = 0, no vector arithmetic.
+ * a, b: 8 * 4 * 64 * 32 = 65536 bytes of e4m3fn operand values each (the timing depends on them through the chip's power
+ * management); out: workgroups * 512 floats.  bench.py --workload mfma_stream reports the rates.
+ */
+int mi355_probe_fp8_mfma_stream(int mode, int workgroups, int iters, const void* a, const void* b, void* out, void* stream);
+
+/*
  * Per-token x per-channel INT8 GEMM:  acc = sum_k a[m,k] * b[n,k] exactly in int32;
  *   out[m,n] = cast( f32(acc) * (sb[n] * sa[m]) + f32(bias[n]) ).
  * Replaces int8_scaled_mm (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; epilogue order of

@@ -27,6 +27,7 @@ EXPORTS = (
     "mi355_fp8_blockwise_mm",
     "mi355_fp8_blockwise_mm_noalloc",
     "mi355_fp8_blockwise_mm_kloop_ceiling",
+    "mi355_probe_fp8_mfma_stream",
     "mi355_fp8_blockwise_mm_ue8m0_workspace_bytes",
     "mi355_fp8_blockwise_mm_ue8m0",
     "mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes",
@@ -96,6 +97,8 @@ def lib() -> ctypes.CDLL:
     L.mi355_fp8_blockwise_mm_noalloc.restype = i32
     L.mi355_fp8_blockwise_mm_kloop_ceiling.argtypes = [vp, vp, vp, vp, vp, i32] + [i64] * 10 + [vp]
     L.mi355_fp8_blockwise_mm_kloop_ceiling.restype = i32
+    L.mi355_probe_fp8_mfma_stream.argtypes = [i32, i32, i32, vp, vp, vp, vp]
+    L.mi355_probe_fp8_mfma_stream.restype = i32
     L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes.argtypes = [i64, i64, i64, i64]
     L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes.restype = sz
     L.mi355_fp8_blockwise_scaled_grouped_mm_plan.argtypes = [i64, i64, i64, i64, ctypes.c_char_p, sz]
