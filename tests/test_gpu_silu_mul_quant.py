@@ -102,3 +102,27 @@ def test_unsupported_combinations_raise(gpu):
         sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, fuse_silu_and_mul=True, enable_v2=True)
     with pytest.raises(NotImplementedError):  # masked without the fused activation
         sglang_per_token_group_quant_fp8(x, 128, masked_m=torch.zeros(1, dtype=torch.int32, device=gpu), enable_v2=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_every_gate_value(gpu, oracle, dtype):
+    """The kernel looks T(silu(gate)) up in a table computed at build time: every one of the 65536 gate bit patterns of
+    either input type (infinities and NaNs aside) must give the oracle's value.  With up = 1 the quantized value is
+    T(silu(gate)) itself; with up = -3 the product's rounding is exercised too."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    T, H = 512, 128
+    gate = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype).clone()
+    gate[~torch.isfinite(gate.float())] = 0
+    for up in (1.0, -3.0):
+        x = torch.empty(T, 2 * H, dtype=dtype)
+        x[:, :H] = gate.view(T, H)
+        x[:, H:] = up
+        q, s = sglang_per_token_group_quant_fp8(x.to(gpu), 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True,
+                                                fuse_silu_and_mul=True, enable_v2=True)
+        v = oracle.silu_mul(x)
+        q_o, s_o = oracle.group_quant(v, 128, mode="mul", layout="ue8m0")
+        assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8))
+        dense = torch.empty(tuple(s.shape), dtype=torch.int32)
+        dense.copy_(s.cpu())
+        assert torch.equal(dense.view(torch.uint8).reshape(T, -1)[:, :1], oracle.unpack_ue8m0(s_o, 1))
