@@ -233,6 +233,20 @@ int mi355_fp8_blockwise_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, ch
 int mi355_int8_scaled_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len);
 
 /*
+ * Host-only: the measured constants of the dispatcher's time models (sglang_amd/csrc/route_constants.h holds the table and
+ * where each number comes from) and the plan a shape would get with ONE constant multiplied by `factor`.  No counterpart
+ * in the reference, whose dispatch ladders hold their thresholds inline (fp8_blockwise_gemm_kernel.cu:181-195,
+ * int8_gemm_kernel.cu:603-661); here a test perturbs every constant by +-10 % and checks that the benchmark shapes stay on
+ * their kernels.  The perturbed copy is local to the calling thread and gone when the call returns.
+ *   constant_index  0 .. mi355_route_constant_count() - 1;  is_fp8 nonzero for the FP8 GEMM, zero for the INT8 GEMM
+ */
+int mi355_route_constant_count(void);
+const char* mi355_route_constant_name(int index);
+double mi355_route_constant_value(int index);
+int mi355_gemm_plan_perturbed(int is_fp8, int64_t M, int64_t N, int64_t K, int aligned, int constant_index, double factor,
+                              char* buf, size_t buf_len);
+
+/*
  * Per-token INT8 activation quantization: absmax = max(1e-10, max |x[m,:]|), s[m] = absmax / 127,
  * q = round-half-away-from-zero(x * (127 / absmax)).
  * Replaces per_token_quant_int8 (python/sglang/srt/layers/quantization/int8_kernel.py:28-89, without cal_sum).

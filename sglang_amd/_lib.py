@@ -37,6 +37,10 @@ EXPORTS = (
     "mi355_int8_scaled_mm",
     "mi355_fp8_blockwise_mm_plan",
     "mi355_int8_scaled_mm_plan",
+    "mi355_route_constant_count",
+    "mi355_route_constant_name",
+    "mi355_route_constant_value",
+    "mi355_gemm_plan_perturbed",
     "mi355_per_token_quant_int8",
     "mi355_per_token_quant_fp8",
     "mi355_row_group_quant_fp8",
@@ -134,6 +138,13 @@ def lib() -> ctypes.CDLL:
     L.mi355_fp8_block_linear_workspace_bytes.restype = sz
     L.mi355_fp8_block_linear.argtypes = [vp, i32, vp, vp, i64, i64, vp, vp, i32] + [i64] * 5 + [vp, sz, vp]
     L.mi355_fp8_block_linear.restype = i32
+    L.mi355_route_constant_count.restype = i32
+    L.mi355_route_constant_name.argtypes = [i32]
+    L.mi355_route_constant_name.restype = ctypes.c_char_p
+    L.mi355_route_constant_value.argtypes = [i32]
+    L.mi355_route_constant_value.restype = ctypes.c_double
+    L.mi355_gemm_plan_perturbed.argtypes = [i32, i64, i64, i64, i32, i32, ctypes.c_double, ctypes.c_char_p, sz]
+    L.mi355_gemm_plan_perturbed.restype = i32
     got = L.mi355_qlinear_abi_version()
     if got != ABI_VERSION:
         raise ImportError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}: rebuild it")
@@ -147,6 +158,23 @@ def gemm_plan(kind: str, M: int, N: int, K: int, aligned: bool = True) -> dict:
     fn = {"fp8": lib().mi355_fp8_blockwise_mm_plan, "int8": lib().mi355_int8_scaled_mm_plan}[kind]
     buf = ctypes.create_string_buffer(256)
     check(fn(M, N, K, int(aligned), buf, len(buf)))
+    out = {}
+    for item in buf.value.decode().split():
+        k, v = item.split("=")
+        out[k] = v if k == "kernel" else int(v)
+    return out
+
+
+def route_constants() -> dict:
+    """The dispatcher's measured time-model constants, name -> value, in table order."""
+    L = lib()
+    return {L.mi355_route_constant_name(i).decode(): L.mi355_route_constant_value(i) for i in range(L.mi355_route_constant_count())}
+
+
+def gemm_plan_perturbed(kind: str, M: int, N: int, K: int, constant: int, factor: float, aligned: bool = True) -> dict:
+    """`gemm_plan` with the `constant`-th entry of the dispatcher's constants table multiplied by `factor`."""
+    buf = ctypes.create_string_buffer(256)
+    check(lib().mi355_gemm_plan_perturbed(int(kind == "fp8"), M, N, K, int(aligned), constant, factor, buf, len(buf)))
     out = {}
     for item in buf.value.decode().split():
         k, v = item.split("=")

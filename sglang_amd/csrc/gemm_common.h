@@ -4,6 +4,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "route_constants.h"
 
 namespace mi355 {
 
@@ -17,12 +18,7 @@ constexpr int KSTEP = 128;   // bytes of K per row and stage
 constexpr int THREADS = 256;
 constexpr int GROUP_M = 8;    // M-tiles per group in the tile order
 
-// ---- measured constants of the dispatcher's time models (the shapes and runs they come from are listed with the
-// models that use them; tests/test_gemm_routes_cpu.py holds the benchmark shapes on their kernels under +-10 % changes)
 constexpr int NUM_CUS = 256;
-// two-phase 256 x 256 kernels: a round of tiles takes (K blocks) * US_PER_KBLOCK + US_PER_TILE, whatever part of the
-// tile is filled (K sweep at M = 4096, N = 36864: slope and intercept of the tile time)
-constexpr double PP_FP8_US_PER_KBLOCK = 1.39, PP_INT8_US_PER_KBLOCK = 1.46, PP_US_PER_TILE = 11.0;
 
 struct GemmParams {
   const uint8_t* a;  // tokens   [M, K], row stride lda

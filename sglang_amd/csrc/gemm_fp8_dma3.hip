@@ -344,29 +344,28 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 //   balance * useful_bytes / (useful_bytes + partial_bytes) * kb_per / (kb_per + 2) * (0.65 for 64-row tiles at M > 128)
 namespace {
 double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int bn, int sp, bool is_int8) {
-  constexpr double HBM_BYTES_PER_US = 5.5e6;
+  const RouteConstants& rc = route_constants();
+  const double HBM_BYTES_PER_US = rc.dma3_hbm_bytes_per_us;
   const int64_t per = (kb_total + sp - 1) / sp;
   const int64_t tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn;
-  // the tile's own time per K block and the latency floor, in the order 128x256, 64x256, 128x128, 64x128, 128x192, 64x192 (the INT8 kernel
-  // of the same structure has its own: fitted to K=4096 -> N=4096..28672 and K=14336 -> N=4096 at 24..1024 tokens)
-  static constexpr double TILE_US[2][6] = {{0.88, 0.58, 0.52, 0.40, 0.68, 0.50}, {1.14, 0.71, 0.64, 0.44, 0.0, 0.0}};
-  static constexpr double LATENCY_US[2][6] = {{1.2, 1.0, 0.7, 0.51, 1.0, 0.75}, {0.96, 0.68, 0.59, 0.54, 0.0, 0.0}};
+  // the tile's own time per K block and the latency floor, in the order 128x256, 64x256, 128x128, 64x128, 128x192, 64x192
+  // (the INT8 kernel of the same structure has its own); the numbers and where they come from: route_constants.h
   const int shape = (bn == 256 ? 0 : bn == 128 ? 2 : 4) + (bm == 128 ? 0 : 1);  // ..., 128x192, 64x192 (FP8 only)
-  const double t_tile = TILE_US[is_int8][shape];
+  const double t_tile = rc.dma3_tile_us[is_int8][shape];
   const double hbm_per_block = (double)(bn * KSTEP) / (double)std::min<int64_t>(tm, 8) + (double)(bm * KSTEP) / (double)std::min<int64_t>(tn, 8);
   // latency floor while the weight streams from HBM: with 256 or 192 channels per tile when at most two token tiles share
-  // it, with 128 when nobody does (rows more than 8 KB apart: measured 1.2x on K = 18432 against K = 7168)
+  // it, with 128 when nobody does (rows more than 8 KB apart cost more)
   const bool streams = hbm_per_block >= (bn == 192 ? 12288.0 : 16384.0);
-  const double t_latency = streams ? LATENCY_US[is_int8][shape] * (kb_total > 64 ? 1.2 : 1.0) : 0.0;
+  const double t_latency = streams ? rc.dma3_latency_us[is_int8][shape] * (kb_total > 64 ? rc.dma3_long_row_factor : 1.0) : 0.0;
   double t = 0.0;
   for (int64_t left = tm * tn * sp; left > 0;) {
     const int64_t c = std::min<int64_t>(left, 256);
     left -= c;
-    // with (nearly) every CU multiplying, the clock drops: 1.2x on the tile's own time (measured on multi-round shapes)
-    const double t_own = t_tile * (c > 200 ? 1.2 : 1.0);
+    // with (nearly) every CU multiplying, the clock drops
+    const double t_own = t_tile * (c > 200 ? rc.dma3_busy_chip_factor : 1.0);
     t += (double)(per + 2) * std::max(std::max(t_own, t_latency), (double)c * hbm_per_block / HBM_BYTES_PER_US);
   }
-  if (sp > 1) t += 8.0 * sp * (double)M * (double)N / HBM_BYTES_PER_US + 8.0 + 0.25 * sp;
+  if (sp > 1) t += 8.0 * sp * (double)M * (double)N / HBM_BYTES_PER_US + rc.dma3_split_fixed_us + rc.dma3_split_per_split_us * sp;
   return t;
 }
 }  // namespace
@@ -382,7 +381,7 @@ Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8) {
     if (bn == 192 && is_int8) continue;  // the INT8 kernel's 32-channel MFMA tiles do not divide 192 / 4
     for (int bm = 64; bm <= 128; bm += 64) {
       if (M <= 64 && bm == 128) break;                 // a second half tile of padding rows buys nothing
-      const double tile_factor = (bm == 64 && M > 128) ? 0.65 : 1.0;
+      const double tile_factor = (bm == 64 && M > 128) ? route_constants().dma3_small_tile_factor : 1.0;
       const int64_t tiles = ((M + bm - 1) / bm) * ((N + T_BN - 1) / T_BN);
       for (int sp = 1; sp <= max_split; ++sp) {
         const int64_t per = (kb_total + sp - 1) / sp;

@@ -317,10 +317,6 @@ struct Plan {
   int bm, bn, splits, kb_per_split;
 };
 
-// below this modelled efficiency of the three-stage mid-M kernel's best tiling the generic kernel (128-wide channel
-// tiles, two workgroups per CU) does better
-constexpr double DMA3_MIN_EFFICIENCY = 0.30;
-
 // Tile and split selection.  Large token counts are MFMA-bound and want the biggest tile; small ones
 // stream the weight once and want enough workgroups in flight to cover HBM latency.
 Plan make_plan(int64_t M, int64_t N, int64_t K) {
@@ -443,13 +439,14 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
     // where the channels alone give it a round's worth of tiles (measured: K=7168 -> N=36864 at M=256: 89 against 141 us,
     // M=1024: 260 against 308 us; INT8 K=4096 -> N=28672 at M=512: 59 against 94 us) and loses for few channels.
     if (M > 128) {
-      const double pp_us = (double)((tiles_256 + NUM_CUS - 1) / NUM_CUS) * ((double)(K / KSTEP) * (is_fp8 ? PP_FP8_US_PER_KBLOCK : PP_INT8_US_PER_KBLOCK) + PP_US_PER_TILE);
+      const RouteConstants& rc = route_constants();
+      const double pp_us = (double)((tiles_256 + NUM_CUS - 1) / NUM_CUS) * ((double)(K / KSTEP) * (is_fp8 ? rc.pp_fp8_us_per_kblock : rc.pp_int8_us_per_kblock) + rc.pp_us_per_tile);
       if (pp_us < dp.time_us) {
         r.kernel = RK_PINGPONG, r.bm = 256, r.bn = 256, r.splits = 1, r.kb_per_split = (int)(K / KSTEP);
         return r;
       }
     }
-    if (N % 4 == 0 || dp.efficiency >= DMA3_MIN_EFFICIENCY) {
+    if (N % 4 == 0 || dp.efficiency >= route_constants().dma3_min_efficiency) {
       r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = dp.bn, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
       return r;
     }
@@ -578,6 +575,22 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
   return check_launch(what);
 }
 
+// ---- the constants table: defaults, the per-thread override of a perturbed plan query, names
+const RouteConstants g_route_defaults{};
+thread_local const RouteConstants* g_route_override = nullptr;
+const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
+    "pp_fp8_us_per_kblock", "pp_int8_us_per_kblock", "pp_us_per_tile", "dma3_hbm_bytes_per_us",
+    "dma3_tile_us[fp8][128x256]", "dma3_tile_us[fp8][64x256]", "dma3_tile_us[fp8][128x128]", "dma3_tile_us[fp8][64x128]",
+    "dma3_tile_us[fp8][128x192]", "dma3_tile_us[fp8][64x192]",
+    "dma3_tile_us[int8][128x256]", "dma3_tile_us[int8][64x256]", "dma3_tile_us[int8][128x128]", "dma3_tile_us[int8][64x128]",
+    "dma3_tile_us[int8][unused]", "dma3_tile_us[int8][unused2]",
+    "dma3_latency_us[fp8][128x256]", "dma3_latency_us[fp8][64x256]", "dma3_latency_us[fp8][128x128]", "dma3_latency_us[fp8][64x128]",
+    "dma3_latency_us[fp8][128x192]", "dma3_latency_us[fp8][64x192]",
+    "dma3_latency_us[int8][128x256]", "dma3_latency_us[int8][64x256]", "dma3_latency_us[int8][128x128]", "dma3_latency_us[int8][64x128]",
+    "dma3_latency_us[int8][unused]", "dma3_latency_us[int8][unused2]",
+    "dma3_busy_chip_factor", "dma3_long_row_factor", "dma3_split_fixed_us", "dma3_split_per_split_us", "dma3_min_efficiency",
+    "dma3_small_tile_factor"};
+
 int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len, const char* what) {
   clear_error();
   MI355_REQUIRE(buf != nullptr && buf_len > 0, MI355_ERR_INVALID_ARGUMENT, "%s: no buffer", what);
@@ -592,9 +605,33 @@ int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, ch
 }
 
 }  // namespace
+
+const RouteConstants& route_constants() { return g_route_override ? *g_route_override : g_route_defaults; }
+const char* route_constant_name(int index) {
+  return index >= 0 && index < ROUTE_CONSTANT_COUNT ? ROUTE_CONSTANT_NAMES[index] : nullptr;
+}
 }  // namespace mi355
 
 using namespace mi355;
+
+extern "C" int mi355_route_constant_count(void) { return ROUTE_CONSTANT_COUNT; }
+extern "C" const char* mi355_route_constant_name(int index) { return route_constant_name(index); }
+extern "C" double mi355_route_constant_value(int index) {
+  return index >= 0 && index < ROUTE_CONSTANT_COUNT ? reinterpret_cast<const double*>(&g_route_defaults)[index] : 0.0;
+}
+extern "C" int mi355_gemm_plan_perturbed(int is_fp8, int64_t M, int64_t N, int64_t K, int aligned, int constant_index, double factor,
+                                         char* buf, size_t buf_len) {
+  const char* what = "mi355_gemm_plan_perturbed";
+  clear_error();
+  MI355_REQUIRE(constant_index >= 0 && constant_index < ROUTE_CONSTANT_COUNT && factor > 0.0, MI355_ERR_INVALID_ARGUMENT,
+                "%s: constant index 0..%d and a positive factor", what, ROUTE_CONSTANT_COUNT - 1);
+  RouteConstants rc = g_route_defaults;
+  reinterpret_cast<double*>(&rc)[constant_index] *= factor;
+  g_route_override = &rc;
+  const int status = describe_route(is_fp8 != 0, M, N, K, aligned, buf, buf_len, what);
+  g_route_override = nullptr;
+  return status;
+}
 
 extern "C" size_t mi355_fp8_blockwise_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return workspace_bytes(M, N, K, true);

@@ -1,0 +1,43 @@
+// Every measured constant of the dispatcher's time models, in one place.
+//
+// choose_route (gemm_w8a8.hip) and dma3_plan (gemm_fp8_dma3.hip) pick a kernel, a tile and a K split by comparing
+// modelled times.  The models' coefficients were fitted to timings on MI355X; they are data, not logic, so they live in
+// this table, each with the measurement it comes from (the rocprofv3 summaries of the same shapes are under profiles/).
+// Run-to-run and box-to-box spread of these timings is +-3 %; tests/test_gemm_routes_cpu.py perturbs every entry by
+// +-10 % through mi355_gemm_plan_perturbed and holds the benchmark shapes on their kernels, or names the measured times
+// of both candidates where a shape sits on a boundary.
+#pragma once
+
+namespace mi355 {
+
+struct RouteConstants {
+  // ---- two-phase 256 x 256 kernels (gemm_fp8_pp.hip, gemm_int8_pp.hip): a round of tiles takes
+  //      (K blocks) * us_per_kblock + us_per_tile, whatever part of the tile is filled and however many CUs the round uses.
+  //      K sweep at M = 4096, N = 36864 (K = 128 ... 14336): slope and intercept of the tile time.
+  double pp_fp8_us_per_kblock = 1.39;
+  double pp_int8_us_per_kblock = 1.46;  // K = 4096 -> N = 28672 at M = 4096: 32 K blocks in 57 us per round
+  double pp_us_per_tile = 11.0;         // launch to first MFMA 2.7 + convert and stage 2.4 + output burst 5 + rest
+  // ---- three-stage kernels with 64- or 128-token tiles (gemm_fp8_dma3.hip, gemm_int8_dma3.hip).  Per K block a
+  //      workgroup takes the largest of: its tile's own time, a latency floor while its weight rows stream from HBM, its
+  //      share of the chip's streaming rate.  Fitted to a sweep of 24 shapes x every (tile, split) (FP8) and to
+  //      K = 4096 -> N = 4096 ... 28672, K = 14336 -> N = 4096 at 24 ... 1024 tokens (INT8).
+  double dma3_hbm_bytes_per_us = 5.5e6;  // streaming rate of the 8-rows x 128-B access shape with two blocks in flight per CU
+  // order: 128x256, 64x256, 128x128, 64x128, 128x192, 64x192 (token x channel tile); [0] FP8, [1] INT8 (no 192-wide tiles)
+  double dma3_tile_us[2][6] = {{0.88, 0.58, 0.52, 0.40, 0.68, 0.50}, {1.14, 0.71, 0.64, 0.44, 0.0, 0.0}};
+  double dma3_latency_us[2][6] = {{1.2, 1.0, 0.7, 0.51, 1.0, 0.75}, {0.96, 0.68, 0.59, 0.54, 0.0, 0.0}};
+  double dma3_busy_chip_factor = 1.2;    // on the tile's own time in a round that keeps > 200 CUs multiplying: the clock drops
+  double dma3_long_row_factor = 1.2;     // on the latency floor for weight rows longer than 8 KB (K = 18432 against K = 7168)
+  double dma3_split_fixed_us = 8.0;      // a K split costs its fp32 partial traffic plus fixed + per_split * splits us
+  double dma3_split_per_split_us = 0.25; //   (reduce launch and its pass over the partial tiles)
+  double dma3_min_efficiency = 0.30;     // below this byte-model score of its best tiling (no split possible: N % 4 != 0)
+                                         //   the generic kernel does better
+  double dma3_small_tile_factor = 0.65;  // the byte-model score of 64-token tiles above 128 tokens
+};
+constexpr int ROUTE_CONSTANT_COUNT = sizeof(RouteConstants) / sizeof(double);
+static_assert(sizeof(RouteConstants) == ROUTE_CONSTANT_COUNT * sizeof(double), "the table is read as an array of doubles");
+
+// The table the calling thread's dispatcher uses: the defaults above, or the perturbed copy a plan query installed.
+const RouteConstants& route_constants();
+const char* route_constant_name(int index);
+
+}  // namespace mi355

@@ -38,6 +38,72 @@ def test_every_variant_is_one_the_library_can_name():
         assert not extra, f"{kind}: variants reached but not listed as required: {sorted(extra, key=str)}"
 
 
+# Tile and split alternatives that a +-10 % change of one time-model constant reaches on a benchmark shape, with the
+# median launch time of each in microseconds on MI355X (40 launches after 8 warm-up launches, HIP events around each
+# launch, the alternative forced by a build of the dispatcher whose plan is overridden; configuration operands).  The first
+# entry of each shape is the dispatcher's own choice.  A boundary is acceptable when both sides of it cost about the same.
+RECORDED_BOUNDARIES = {
+    ("fp8", (128, 7168, 18432)): {(128, 128, 4): 48.8, (64, 128, 2): 50.0, (128, 192, 6): 52.7},
+    ("fp8", (4096, 1536, 7168)): {(128, 192, 1): 63.0, (128, 256, 1): 65.8},
+    ("fp8", (4096, 576, 7168)): {(64, 192, 1): 45.7, (128, 128, 1): 47.0},
+    ("int8", (256, 28672, 4096)): {(128, 256, 1): 56.2, (128, 128, 1): 61.2},
+    ("int8", (256, 4096, 14336)): {(128, 128, 4): 48.9, (64, 256, 4): 49.9, (128, 128, 3): 47.4},
+}
+BOUNDARY_COST = 1.10  # the slower side of a recorded boundary may cost at most this much more than the dispatcher's choice
+
+
+def test_benchmark_shapes_hold_their_kernels_when_a_constant_moves():
+    """Every measured constant of the dispatcher's time models (sglang_amd/csrc/route_constants.h) is changed by -10 % and
+    +10 %, one at a time.  No benchmark shape may move to another kernel.  Within the mid-M kernel a shape may move to
+    another tile or split only where both have been timed on the GPU and recorded above, and the recorded times must show
+    that the move costs less than BOUNDARY_COST: then the constant's uncertainty (timings spread +-3 %) cannot cost more
+    than that.  A new constant, or a changed one, that puts a benchmark shape on an unmeasured boundary fails here."""
+    from sglang_amd import _lib
+
+    names = list(_lib.route_constants())
+    assert len(names) == _lib.lib().mi355_route_constant_count() and len(set(names)) == len(names)
+    tile = lambda p: (p["bm"], p["bn"], p["splits"])
+    moved = set()
+    for kind, config in (("fp8", FP8_DECODE_CONFIG + FP8_PREFILL_CONFIG), ("int8", INT8_CONFIG)):
+        for shape in config:
+            base = plan_for(kind, *shape)
+            for i, name in enumerate(names):
+                for factor in (0.9, 1.1):
+                    p = _lib.gemm_plan_perturbed(kind, *shape, i, factor)
+                    assert p["kernel"] == base["kernel"], f"{kind} {shape}: {name} x {factor} moves {base['kernel']} -> {p['kernel']}"
+                    if tile(p) == tile(base):
+                        continue
+                    rec = RECORDED_BOUNDARIES.get((kind, shape))
+                    assert rec is not None and tile(base) in rec and tile(p) in rec, \
+                        f"{kind} {shape}: {name} x {factor} moves tile {tile(base)} -> {tile(p)}: time both and record them"
+                    assert next(iter(rec)) == tile(base), f"{kind} {shape}: the recorded choice {next(iter(rec))} is not the plan's {tile(base)}"
+                    assert rec[tile(p)] <= BOUNDARY_COST * rec[tile(base)], (kind, shape, name, factor, rec)
+                    moved.add((kind, shape, tile(p)))
+    # the record holds nothing stale: every recorded alternative is one a perturbation reaches
+    for (kind, shape), rec in RECORDED_BOUNDARIES.items():
+        for t in list(rec)[1:]:
+            assert (kind, shape, t) in moved, f"{kind} {shape}: recorded alternative {t} is no longer reached"
+
+
+def test_perturbed_plan_query():
+    import ctypes
+
+    from sglang_amd import _lib
+
+    L = _lib.lib()
+    n = L.mi355_route_constant_count()
+    assert n == 34 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
+    assert _lib.route_constants()["pp_fp8_us_per_kblock"] == 1.39
+    buf = ctypes.create_string_buffer(256)
+    assert L.mi355_gemm_plan_perturbed(1, 128, 7168, 18432, 1, n, 1.1, buf, len(buf)) == 1
+    assert L.mi355_gemm_plan_perturbed(1, 128, 7168, 18432, 1, 0, 0.0, buf, len(buf)) == 1
+    # a factor of one is the plain query, and the perturbed copy does not outlive its call
+    for kind, shape in (("fp8", (128, 7168, 18432)), ("int8", (256, 4096, 14336)), ("fp8", (4096, 36864, 7168))):
+        assert _lib.gemm_plan_perturbed(kind, *shape, 3, 1.0) == _lib.gemm_plan(kind, *shape)
+    far = _lib.gemm_plan_perturbed("fp8", 256, 36864, 7168, 0, 10.0)  # a two-phase kernel ten times slower loses
+    assert far["kernel"] == "dma3" and _lib.gemm_plan("fp8", 256, 36864, 7168)["kernel"] == "pingpong"
+
+
 def test_plan_query_rejects_bad_arguments():
     import ctypes
 
