@@ -63,6 +63,15 @@ enum {
 
 int mi355_qlinear_abi_version(void);
 
+/*
+ * Optional set-up of the current device: resolves the device addresses of the library's two built-in device arrays (the
+ * scratch of mi355_fp8_blockwise_mm_noalloc and a constant of mi355_fp8_scaled_mm).  Those entry points do the same on
+ * their first call on a device; a caller that captures them into a HIP graph calls this first, once per device with that
+ * device current, because the first look-up may load the code object and is refused during a capture.  No counterpart in
+ * the reference (torch extensions are initialised by their import).  Idempotent and thread-safe.
+ */
+int mi355_qlinear_init(void);
+
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the next call. */
 const char* mi355_last_error(void);
 

@@ -21,6 +21,7 @@ NOALLOC_SCRATCH_BYTES = 32 << 20
 
 EXPORTS = (
     "mi355_qlinear_abi_version",
+    "mi355_qlinear_init",
     "mi355_last_error",
     "mi355_group_quant_8bit",
     "mi355_fp8_blockwise_mm_workspace_bytes",

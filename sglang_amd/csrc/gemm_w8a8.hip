@@ -677,27 +677,46 @@ constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)MI355_NOALLOC_SCRATCH_BYTES;
 static __device__ __align__(256) uint8_t scratch[NOALLOC_SCRATCH_BYTES];
 
 constexpr int MAX_DEVICES = 64;
-std::mutex scratch_mutex;
-void* scratch_ptr[MAX_DEVICES];  // guarded by scratch_mutex
+std::mutex symbol_mutex;
+void* scratch_ptr[MAX_DEVICES];     // guarded by symbol_mutex
+void* unit_scale_ptr[MAX_DEVICES];  // guarded by symbol_mutex
 
-int scratch_of_current_device(void** ptr, const char* what) {
+// A weight-block scale of one for the per-token x per-channel FP8 GEMM, which runs on the blockwise kernels: every block
+// reads this same float (strides 0).
+static __device__ __align__(16) float unit_scale[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+
+// Device addresses of the two arrays above on the current device, looked up on first use (or by mi355_qlinear_init) and
+// kept.  The first lookup on a device may make the runtime load the code object, which allocates: it is refused while
+// `stream` is being captured into a graph, where the caller is told to initialise the device before the capture.
+int symbols_of_current_device(void** scratch_out, const float** unit_out, hipStream_t stream, bool check_capture, const char* what) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
     set_error("%s: cannot identify the current device (%s, device %d)", what, hipGetErrorString(e), dev);
     return MI355_ERR_LAUNCH;
   }
-  std::lock_guard<std::mutex> lock(scratch_mutex);
-  if (scratch_ptr[dev] == nullptr) {
-    void* p = nullptr;
+  std::lock_guard<std::mutex> lock(symbol_mutex);
+  if (scratch_ptr[dev] == nullptr || unit_scale_ptr[dev] == nullptr) {
+    if (check_capture) {
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      e = hipStreamIsCapturing(stream, &capturing);
+      if (e != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        set_error("%s: device %d is not initialised and the stream is being captured: call mi355_qlinear_init() on this device "
+                  "before the capture (%s)", what, dev, hipGetErrorString(e));
+        return MI355_ERR_LAUNCH;
+      }
+    }
+    void *p = nullptr, *q = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || p == nullptr) {
-      set_error("%s: cannot resolve the scratch array on device %d: %s", what, dev, hipGetErrorString(e));
+    if (e == hipSuccess) e = hipGetSymbolAddress(&q, HIP_SYMBOL(unit_scale));
+    if (e != hipSuccess || p == nullptr || q == nullptr) {
+      set_error("%s: cannot resolve the library's device arrays on device %d: %s", what, dev, hipGetErrorString(e));
       return MI355_ERR_LAUNCH;
     }
-    scratch_ptr[dev] = p;
+    scratch_ptr[dev] = p, unit_scale_ptr[dev] = q;
   }
-  *ptr = scratch_ptr[dev];
+  if (scratch_out) *scratch_out = scratch_ptr[dev];
+  if (unit_out) *unit_out = static_cast<const float*>(unit_scale_ptr[dev]);
   return MI355_OK;
 }
 
@@ -837,42 +856,17 @@ extern "C" int mi355_fp8_blockwise_mm_noalloc(const void* a, const void* b, cons
                 what, (long long)M, (long long)N, (long long)K, need, NOALLOC_SCRATCH_BYTES);
   void* ws = nullptr;
   if (need > 0) {
-    rc = scratch_of_current_device(&ws, what);
+    rc = symbols_of_current_device(&ws, nullptr, static_cast<hipStream_t>(stream), true, what);
     if (rc != MI355_OK) return rc;
   }
   // every partial sum that the reduce kernel reads is written by this call first, so nothing has to be cleared
   return run_gemm<true>(p, ws, need > 0 ? NOALLOC_SCRATCH_BYTES : 0, static_cast<hipStream_t>(stream), what);
 }
 
-namespace {
-
-// A weight-block scale of one for the per-token x per-channel FP8 GEMM, which runs on the blockwise kernels: every block
-// reads this same float (strides 0).  Device address looked up once per device, like the scratch array above.
-static __device__ __align__(16) float unit_scale[4] = {1.f, 1.f, 1.f, 1.f};
-void* unit_scale_ptr[MAX_DEVICES];  // guarded by scratch_mutex
-
-int unit_scale_of_current_device(const float** ptr, const char* what) {
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
-    set_error("%s: cannot identify the current device (%s, device %d)", what, hipGetErrorString(e), dev);
-    return MI355_ERR_LAUNCH;
-  }
-  std::lock_guard<std::mutex> lock(scratch_mutex);
-  if (unit_scale_ptr[dev] == nullptr) {
-    void* q = nullptr;
-    e = hipGetSymbolAddress(&q, HIP_SYMBOL(unit_scale));
-    if (e != hipSuccess || q == nullptr) {
-      set_error("%s: cannot resolve a device constant on device %d: %s", what, dev, hipGetErrorString(e));
-      return MI355_ERR_LAUNCH;
-    }
-    unit_scale_ptr[dev] = q;
-  }
-  *ptr = static_cast<const float*>(unit_scale_ptr[dev]);
-  return MI355_OK;
+extern "C" int mi355_qlinear_init(void) {
+  clear_error();
+  return symbols_of_current_device(nullptr, nullptr, nullptr, false, "mi355_qlinear_init");
 }
-
-}  // namespace
 
 extern "C" size_t mi355_fp8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return workspace_bytes(M, N, K, true);
@@ -887,7 +881,7 @@ extern "C" int mi355_fp8_scaled_mm(const void* a, const void* b, const float* sa
                 "%s: out_dtype must be bfloat16 or float16", what);
   const float* one = nullptr;
   if (M > 0 && N > 0) {
-    const int rc1 = unit_scale_of_current_device(&one, what);
+    const int rc1 = symbols_of_current_device(nullptr, &one, static_cast<hipStream_t>(stream), true, what);
     if (rc1 != MI355_OK) return rc1;
   }
   GemmParams p;

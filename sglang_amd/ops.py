@@ -50,7 +50,16 @@ SCHEMAS = {
 }
 
 
+_ready_devices = set()
+
+
 def _stream() -> int:
+    """The current HIP stream; on a device's first use, the library's per-device set-up (it must not fall inside a graph
+    capture, which the first launch of a process otherwise might)."""
+    dev = torch.cuda.current_device()
+    if dev not in _ready_devices:
+        check(lib().mi355_qlinear_init())
+        _ready_devices.add(dev)
     return torch.cuda.current_stream().cuda_stream
 
 

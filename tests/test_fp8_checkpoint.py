@@ -52,10 +52,69 @@ def test_block_alignment_checks_of_create_weights():
         Fp8Linear(512, [384], cfg, parallel="column", tp_rank=0, tp_size=2)
     with pytest.raises(ValueError, match="input_size_per_partition = 192 is not divisible"):
         Fp8Linear(384, [256], cfg, parallel="row", tp_rank=1, tp_size=2)
+
+
+def test_method_registers_the_checkpoint_names_on_the_layer():
+    """fp8.py:277-341: `weight`, `weight_scale_inv` / `weight_scale`, `input_scale` are parameters of `layer` itself, each
+    with the `weight_loader` the layer handed in; a loader that walks `named_parameters()` finds the checkpoint's keys."""
+    cfg = Fp8Config.from_config(BLOCK_CFG)
     layer = torch.nn.Module()
-    Fp8LinearMethod(cfg).create_weights(layer, 512, [256, 256], 512, 1024, torch.bfloat16, tp_rank=1)
-    assert layer.fp8.parallel == "column" and layer.fp8.tp_size == 2 and tuple(layer.fp8.weight.shape) == (512, 512)
-    assert tuple(layer.fp8.weight_scale_inv.shape) == (4, 4) and layer.logical_widths == [256, 256]
+    calls = []
+
+    def loader(param, loaded_weight, loaded_shard_id=None):
+        calls.append(loaded_shard_id)
+        param.data.copy_(loaded_weight)
+
+    method = Fp8LinearMethod(cfg, tp_size=2)
+    method.create_weights(layer, 512, [256, 256], 512, 1024, torch.bfloat16, weight_loader=loader)
+    names = dict(layer.named_parameters())
+    assert set(names) == {"weight", "weight_scale_inv"} and layer.input_scale is None
+    assert tuple(layer.weight.shape) == (512, 512) and layer.weight.dtype == FP8 and tuple(layer.weight_scale_inv.shape) == (4, 4)
+    assert (layer.weight.input_dim, layer.weight.output_dim) == (1, 0) and layer.weight_scale_inv.weight_loader is loader
+    assert layer.logical_widths == [256, 256] and layer.input_size_per_partition == 512 and layer.output_size_per_partition == 512
+    assert layer.orig_dtype == torch.bfloat16
+    with pytest.raises(RuntimeError, match="never loaded"):
+        method.process_weights_after_loading(layer)
+    g = torch.Generator().manual_seed(5)
+    ckpt = _proj(512, 512, g, "mlp.gate_up_proj")
+    for name, param in layer.named_parameters():
+        param.weight_loader(param, ckpt[f"mlp.gate_up_proj.{name}"])
+    assert calls == [None, None] and torch.equal(_bytes(layer.weight.data), _bytes(ckpt["mlp.gate_up_proj.weight"]))
+    method.process_weights_after_loading(layer)
+    # the column-parallel check needs tp_size: the same sizes on one rank are a merged layer only
+    with pytest.raises(ValueError, match="output_partition_size = 192 is not divisible"):
+        Fp8LinearMethod(cfg, tp_size=2).create_weights(torch.nn.Module(), 512, [192], 512, 384, torch.bfloat16)
+    Fp8LinearMethod(cfg, tp_size=1).create_weights(torch.nn.Module(), 512, [192], 512, 192, torch.bfloat16)
+    # per-tensor static: scales per merged projection, default loader, channelwise after loading
+    static = Fp8LinearMethod(Fp8Config.from_config({"quant_method": "fp8", "activation_scheme": "static"}))
+    layer = torch.nn.Module()
+    static.create_weights(layer, 128, [64, 32], 128, 96, torch.bfloat16)
+    assert set(dict(layer.named_parameters())) == {"weight", "weight_scale", "input_scale"}
+    layer.weight.weight_loader(layer.weight, torch.zeros(96, 128).to(FP8))
+    layer.weight_scale.weight_loader(layer.weight_scale, torch.tensor([0.5, 0.25]))
+    layer.input_scale.weight_loader(layer.input_scale, torch.tensor([2.0, 3.0]))
+    static.process_weights_after_loading(layer)
+    assert tuple(layer.weight.shape) == (128, 96) and tuple(layer.weight_scale.shape) == (96, 1)
+    assert layer.weight_scale[:64].eq(0.5).all() and layer.weight_scale[64:].eq(0.25).all() and float(layer.input_scale) == 3.0
+
+
+def test_layer_loads_through_named_parameters():
+    cfg = Fp8Config.from_config(BLOCK_CFG)
+    g = torch.Generator().manual_seed(6)
+    ckpt = {**_proj(512, 384, g, "q"), **_proj(256, 384, g, "k"), **_proj(256, 384, g, "v")}
+    layer = Fp8Linear(384, [512, 256, 256], cfg, parallel="column", tp_rank=1, tp_size=2, bias=True)
+    assert [n for n, _ in layer.named_parameters()] == ["weight", "weight_scale_inv", "bias"]
+    for shard, proj in enumerate("qkv"):
+        ckpt[f"{proj}.bias"] = torch.randn(ckpt[f"{proj}.weight"].shape[0], generator=g).to(torch.bfloat16)
+        for name, param in layer.named_parameters():
+            param.weight_loader(param, ckpt[f"{proj}.{name}"], shard)
+    want = torch.cat([ckpt["q.weight"][256:], ckpt["k.weight"][128:], ckpt["v.weight"][128:]])
+    assert torch.equal(_bytes(layer.weight.data), _bytes(want))
+    want_s = torch.cat([ckpt["q.weight_scale_inv"][2:], ckpt["k.weight_scale_inv"][1:], ckpt["v.weight_scale_inv"][1:]])
+    assert torch.equal(layer.weight_scale_inv.data, want_s)
+    assert torch.equal(layer.bias.data, torch.cat([ckpt["q.bias"][256:], ckpt["k.bias"][128:], ckpt["v.bias"][128:]]))
+    with pytest.raises(KeyError, match="does not belong"):
+        layer.weight_loader(torch.nn.Parameter(torch.zeros(1)), torch.zeros(1))
 
 
 def test_merged_projection_from_a_safetensors_checkpoint(tmp_path):
