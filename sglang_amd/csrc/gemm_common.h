@@ -244,4 +244,14 @@ int decode_groups_per_wg(int64_t N, int splits);  // consecutive 128-channel gro
 int launch_fp8_decode(GemmParams& p, int groups_per_wg, hipStream_t stream, const char* what);
 int launch_int8_decode(GemmParams& p, int groups_per_wg, hipStream_t stream, const char* what);  // same kernel, int8 MFMA, int32 partials
 
+// Decode (M <= 16) GEMMs for small weights (gemm_decode_wavesplit.hip): 16 channels per workgroup, K split over its waves
+// and summed inside the workgroup - one launch, no workspace.  K % 128 == 0, N % 16 == 0, 16-byte aligned rows.
+struct WavesplitShape {
+  int waves, blocks_per_round;
+};
+WavesplitShape wavesplit_shape(int64_t K);
+bool wavesplit_supported(int64_t M, int64_t N, int64_t K);
+int launch_fp8_wavesplit(GemmParams& p, hipStream_t stream, const char* what);
+int launch_int8_wavesplit(GemmParams& p, hipStream_t stream, const char* what);
+
 }  // namespace mi355

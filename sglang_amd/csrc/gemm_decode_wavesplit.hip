@@ -1,0 +1,159 @@
+// Decode (M <= 16) GEMMs for gfx950 when the weight is small - blockwise-scaled FP8 and per-token x per-channel INT8:
+// K is split over the WAVES of a workgroup, and the sum is finished inside the workgroup.
+//
+// The streaming decode kernel (gemm_fp8_decode.hip) gives a workgroup 128 channels and 8 K blocks; a weight of a few MB
+// (K = 7168 -> N = 2048: 14 MB) then makes ~100 workgroups, half the CUs stay empty, and a second launch adds the K
+// ranges.  Both cost more than the traffic itself: 6.1 us + 2.8 us for a weight that leaves HBM in 2 us.  Here a workgroup
+// owns 16 channels - one MFMA tile for the <= 16 tokens - over ALL of K; its W waves take K blocks w, w + W, w + 2 W, ...
+// so that neighbouring waves read neighbouring 128-byte pieces of the same weight rows.  A wave requests every block of
+// its share at once, straight into registers in MFMA operand layout (two 16-byte pieces per lane and block for the
+// weight, two for the tokens, which come from L2 after the first workgroups touched them), multiplies them as they
+// arrive, and the W partial tiles are added through LDS in wave order by wave 0, which applies the epilogue and stores.
+// No workspace, no second launch, N / 16 workgroups, and the whole weight is requested within the first microsecond.
+//
+// A wave's share is KBW blocks per round (all requested before the first is used); longer K takes several rounds, whose
+// start-up gaps the other workgroups on the CU fill (~80 registers: six waves per SIMD).
+// Blocks past the end of K are fetched from the last valid block and multiply a zero scale (FP8) or zeroed tokens (INT8).
+// Requires K % 128 == 0, N % 16 == 0, 16-byte aligned rows.  FP8 sums differ from the streaming kernel's in the order of
+// the additions only (per wave in K order, then over waves); INT8 results are exact either way.
+#include "gemm_common.h"
+
+namespace mi355 {
+namespace {
+
+struct Frag {
+  u32x4 lo, hi;
+};
+__device__ __forceinline__ v8i as_v8i(const Frag& f) {
+  return v8i{(int)f.lo.x, (int)f.lo.y, (int)f.lo.z, (int)f.lo.w, (int)f.hi.x, (int)f.hi.y, (int)f.hi.z, (int)f.hi.w};
+}
+
+template <bool IS_FP8, int W, int KBW>
+__global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmParams p) {
+  using AccT = typename std::conditional<IS_FP8, float, int>::type;
+  typedef AccT acc4 __attribute__((ext_vector_type(4)));
+  __shared__ acc4 red[W][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & 15, q = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int tok = min(l16, p.M - 1);  // lanes past M repeat the last token; their results are never stored
+  // operand layout of the 16 x 16 x 128 MFMA: lane (row l16, quarter q) holds bytes [16 q, +16) and [64 + 16 q, +16) of the row's block
+  const uint8_t* wrow = p.b + (int64_t)(n0 + l16) * p.ldb + q * 16;
+  const uint8_t* trow = p.a + (int64_t)tok * p.lda + q * 16;
+  const float* sa_row = IS_FP8 ? p.sa + (int64_t)tok * p.sa_sm : nullptr;
+  const float* sb_row = IS_FP8 ? p.sb + (int64_t)(n0 >> 7) * p.sb_sn : nullptr;  // wave-uniform
+
+  acc4 acc = {0, 0, 0, 0};
+  const int rounds = (p.kb_total + W * KBW - 1) / (W * KBW);
+  for (int r = 0; r < rounds; ++r) {
+    Frag wf[KBW], tf[KBW];
+    float sav[KBW], sbv[KBW];
+#pragma unroll
+    for (int j = 0; j < KBW; ++j) {
+      const int kb = (r * KBW + j) * W + wave;  // wave-uniform
+      const int kc = min(kb, p.kb_total - 1);
+      wf[j].lo = *reinterpret_cast<const u32x4*>(wrow + (int64_t)kc * KSTEP);
+      wf[j].hi = *reinterpret_cast<const u32x4*>(wrow + (int64_t)kc * KSTEP + 64);
+      tf[j].lo = *reinterpret_cast<const u32x4*>(trow + (int64_t)kc * KSTEP);
+      tf[j].hi = *reinterpret_cast<const u32x4*>(trow + (int64_t)kc * KSTEP + 64);
+      if constexpr (IS_FP8) {
+        sav[j] = sa_row[(int64_t)kc * p.sa_sk];
+        sbv[j] = sb_row[(int64_t)kc * p.sb_sk];
+      }
+    }
+    // every request of the round is out before the first result is used: without this fence the scheduler pairs each
+    // block's loads with its MFMA to save registers, and the wave waits out one memory latency per block
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < KBW; ++j) {
+      const bool valid = (r * KBW + j) * W + wave < p.kb_total;
+      if constexpr (IS_FP8) {
+        const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(tf[j]), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0,
+                                                                          0, 0, 0, 0);
+        const float sc = valid ? sav[j] * sbv[j] : 0.f;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[v] = fmaf(part[v], sc, acc[v]);
+      } else {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        const u32x4 tlo = valid ? tf[j].lo : z, thi = valid ? tf[j].hi : z;
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].lo.x, (int)wf[j].lo.y, (int)wf[j].lo.z, (int)wf[j].lo.w},
+                                                    v4i{(int)tlo.x, (int)tlo.y, (int)tlo.z, (int)tlo.w}, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].hi.x, (int)wf[j].hi.y, (int)wf[j].hi.z, (int)wf[j].hi.w},
+                                                    v4i{(int)thi.x, (int)thi.y, (int)thi.z, (int)thi.w}, acc, 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- add the W partial tiles in wave order
+  if (wave != 0) red[wave][lane] = acc;
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 1; w < W; ++w) {
+    const acc4 t = red[w][lane];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) acc[v] += t[v];
+  }
+  if (l16 >= p.M) return;
+  // lane holds channels n0 + 4 q .. + 3 for token l16
+  const int n = n0 + 4 * q;
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+  if constexpr (IS_FP8) {
+    float r4[4] = {acc[0], acc[1], acc[2], acc[3]};
+    fp8_channel_epilogue(p, n, r4);
+    store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r4, 4, vec_ok);
+  } else if (p.out_dtype == MI355_I32) {
+    int* o = reinterpret_cast<int*>(p.out) + (int64_t)l16 * p.ldo + n;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) o[v] = acc[v];
+  } else {
+    const float sa_m = p.sa[l16];
+    float r4[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      // separately rounded multiply and add: the contract is mul, mul, add, not a fused multiply-add
+      float t = mul_rn((float)acc[v], mul_rn(p.sb[n + v], sa_m));
+      if (p.bias) {
+        const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
+        t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+      }
+      r4[v] = t;
+    }
+    store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r4, 4, vec_ok);
+  }
+}
+
+template <bool IS_FP8, int W, int KBW>
+int launch_variant(const GemmParams& p, hipStream_t stream, const char* what) {
+  hipLaunchKernelGGL((decode_wavesplit_kernel<IS_FP8, W, KBW>), dim3((unsigned)(p.N / 16)), dim3(64 * W), 0, stream, p);
+  return check_launch(what);
+}
+
+template <bool IS_FP8>
+int launch_wavesplit(GemmParams& p, hipStream_t stream, const char* what) {
+  p.splits = 1;
+  p.tiles_m = 1;
+  p.tiles_n = p.N / 16;
+  const WavesplitShape s = wavesplit_shape(p.K);
+  return s.waves == 4 ? launch_variant<IS_FP8, 4, 4>(p, stream, what) : launch_variant<IS_FP8, 8, 4>(p, stream, what);
+}
+
+}  // namespace
+
+// Waves per workgroup and K blocks per wave and round.  Measured (us, M = 1; waves x blocks): K = 4096 -> N = 28672 INT8:
+// 8x4 24.5, 4x8 28.1, 4x4 30.6, 16x4 42.0; K = 7168 -> N = 36864 FP8: 8x4 49.2, 4x8 49.8, 4x4 51.2, 8x8 55.2, 16x4 56.3;
+// K = 14336 -> N = 4096 INT8: 4x4 15.5, 16x4 15.9, 8x4 16.3; K = 18432 -> N = 7168 FP8: 4x4 30.4, 4x8 30.9, 8x4 31.5, 16x4 36.4.
+// Eight waves of four blocks up to K = 8192 (one or two rounds); for longer K four waves, whose many short rounds overlap
+// across the workgroups that share a CU; four waves also where K has at most 16 blocks.
+WavesplitShape wavesplit_shape(int64_t K) {
+  const int64_t kb = (K + KSTEP - 1) / KSTEP;
+  return (kb > 16 && kb <= 64) ? WavesplitShape{8, 4} : WavesplitShape{4, 4};
+}
+
+bool wavesplit_supported(int64_t M, int64_t N, int64_t K) { return M >= 1 && M <= 16 && K % KSTEP == 0 && N % 16 == 0; }
+
+int launch_fp8_wavesplit(GemmParams& p, hipStream_t stream, const char* what) { return launch_wavesplit<true>(p, stream, what); }
+int launch_int8_wavesplit(GemmParams& p, hipStream_t stream, const char* what) { return launch_wavesplit<false>(p, stream, what); }
+
+}  // namespace mi355

@@ -406,10 +406,17 @@ static int launch_decode(GemmParams& p, int gpw, hipStream_t stream, const char*
       return check_launch(what);
     }
   }
-  if (p.splits > 1)
-    hipLaunchKernelGGL((decode_kernel<IS_FP8, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
-  else
+  if (p.splits > 1) {
+    if constexpr (IS_FP8) {
+      hipLaunchKernelGGL((decode_kernel<true, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+    } else {
+      // INT8 shapes with more than one K range (8 blocks) all go to the wave-split kernel: this variant is not built
+      set_error("%s: the INT8 streaming decode kernel has no K split", what);
+      return MI355_ERR_UNSUPPORTED;
+    }
+  } else {
     hipLaunchKernelGGL((decode_kernel<IS_FP8, false>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+  }
   return check_launch(what);
 }
 

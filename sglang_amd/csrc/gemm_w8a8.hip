@@ -401,8 +401,8 @@ int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* wha
 
 // Which kernel serves a problem, with which tiling.  One function decides for the launcher and for the plan query, so
 // what the query reports is what runs.
-enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_PINGPONG, RK_PIPELINED, RK_GENERIC };
-const char* const ROUTE_NAMES[] = {"decode", "dma3", "pingpong", "pipelined", "generic"};
+enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_PINGPONG, RK_PIPELINED, RK_GENERIC, RK_WAVESPLIT };
+const char* const ROUTE_NAMES[] = {"decode", "dma3", "pingpong", "pipelined", "generic", "decode_wavesplit"};
 
 struct Route {
   int kernel;
@@ -412,12 +412,32 @@ struct Route {
   bool aligned;
 };
 
+// Decode sizes: the kernel that splits K over the waves of a workgroup instead of over workgroups, where it was
+// measured faster than the streaming kernel (the numbers stand beside the thresholds in route_constants.h).
+bool wavesplit_preferred(bool is_fp8, int64_t M, int64_t N, int64_t K) {
+  if (!decode_supported(M, N, K)) return true;  // channels in whole 16s but not 128s: the streaming kernel cannot run
+  const RouteConstants& rc = route_constants();
+  if ((double)(K / KSTEP) < rc.wavesplit_min_kblocks) return false;
+  if (!is_fp8) return true;
+  if ((double)N * (double)K <= rc.wavesplit_small_weight_bytes) return N / 16 >= NUM_CUS || (double)M <= rc.wavesplit_small_weight_max_tokens;
+  return (double)M <= rc.wavesplit_large_weight_max_tokens;
+}
+
 // `aligned`: both operand base pointers and row strides are multiples of 16 bytes and K % 16 == 0.
-Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, bool aligned) {
+// `fused_quant`: the tokens arrive unquantized and the kernel is to quantize them itself, which only the streaming
+// decode kernel can.
+Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, bool aligned, bool fused_quant = false) {
   Route r{};
   r.aligned = aligned;
   const bool small_b = N * ldb < (1ll << 32);                 // kernels that address rows by 32-bit byte offsets
   const bool small_offsets = M * lda < (1ll << 32) && small_b;
+  if (!fused_quant && wavesplit_supported(M, N, K) && aligned && small_b && wavesplit_preferred(is_fp8, M, N, K)) {
+    const WavesplitShape ws = wavesplit_shape(K);
+    r.kernel = RK_WAVESPLIT, r.bm = 16, r.bn = 16, r.splits = 1;
+    r.kb_per_split = (int)((K + KSTEP - 1) / KSTEP);
+    r.groups_per_wg = ws.waves;  // waves that share a workgroup's K
+    return r;
+  }
   if (decode_supported(M, N, K) && aligned && small_b) {  // barrier-free weight streaming
     r.kernel = RK_DECODE, r.bm = 16, r.bn = 128;
     r.splits = decode_splits(M, N, K);
@@ -528,7 +548,7 @@ template <bool IS_FP8>
 int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipStream_t stream, const char* what) {
   p.kb_total = (p.K + KSTEP - 1) / KSTEP;
   const bool aligned = operands_aligned(p);
-  const Route r = choose_route(IS_FP8, p.M, p.N, p.K, p.lda, p.ldb, aligned);
+  const Route r = choose_route(IS_FP8, p.M, p.N, p.K, p.lda, p.ldb, aligned, p.x16 != nullptr);
   p.splits = r.splits;
   p.kb_per_split = r.kb_per_split;
   const size_t need = route_workspace_need(IS_FP8, r, p);
@@ -554,6 +574,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
     case RK_DECODE:
       rc = IS_FP8 ? launch_fp8_decode(p, r.groups_per_wg, stream, what) : launch_int8_decode(p, r.groups_per_wg, stream, what);
       break;
+    case RK_WAVESPLIT: return IS_FP8 ? launch_fp8_wavesplit(p, stream, what) : launch_int8_wavesplit(p, stream, what);
     case RK_DMA3:
       rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, r.bn, stream, what) : launch_int8_dma3(p, r.bm, r.bn, stream, what);
       break;
@@ -589,7 +610,8 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
     "dma3_latency_us[int8][128x256]", "dma3_latency_us[int8][64x256]", "dma3_latency_us[int8][128x128]", "dma3_latency_us[int8][64x128]",
     "dma3_latency_us[int8][unused]", "dma3_latency_us[int8][unused2]",
     "dma3_busy_chip_factor", "dma3_long_row_factor", "dma3_split_fixed_us", "dma3_split_per_split_us", "dma3_min_efficiency",
-    "dma3_small_tile_factor"};
+    "dma3_small_tile_factor", "wavesplit_min_kblocks", "wavesplit_small_weight_bytes", "wavesplit_small_weight_max_tokens",
+    "wavesplit_large_weight_max_tokens"};
 
 int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len, const char* what) {
   clear_error();
@@ -941,7 +963,7 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
   const size_t sa_bytes = align256((size_t)pitch * (size_t)(K / KSTEP) * 4u);
   // Decode sizes: the GEMM kernel quantizes the tokens of each K range itself (same arithmetic), no quantizer launch.
   if (x_dtype != MI355_F32 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && ldw % 16 == 0 &&
-      choose_route(true, M, N, K, K, ldw, true).kernel == RK_DECODE) {
+      choose_route(true, M, N, K, K, ldw, true, true).kernel == RK_DECODE) {
     GemmParams p;
     bool empty;
     // a / sa are not read by the kernel in this mode; they only have to satisfy the checks

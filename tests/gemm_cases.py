@@ -2,7 +2,8 @@
 parity tests, plus the full-size shapes of the benchmark configurations.
 
 A *variant* is one compiled code path: the kernel, its token-tile height, whether it writes split-K partial sums,
-for the decode kernel how many 128-channel groups a workgroup walks, for the large-M kernels whether K ends on a
+for the decode kernel how many 128-channel groups a workgroup walks, for the wave-split decode kernel how many waves
+share a workgroup's K and whether a wave's share takes several rounds, for the large-M kernels whether K ends on a
 128-byte block.  `variant_of` maps a plan (sglang_amd._lib.gemm_plan) to such a key.
 """
 
@@ -12,6 +13,10 @@ FP8_ROUTE_SHAPES = [
     # an uneven last workgroup (16640 = 130 groups), short last K ranges (4480 = 35 blocks, 2176 = 17 blocks)
     (1, 128, 128), (3, 256, 512), (1, 512, 7168), (16, 2048, 7168), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432),
     (7, 33280, 4096), (5, 66048, 512), (2, 133120, 384),
+    # wave-split decode kernel (few tokens or a small weight, K of at least 8 blocks; N % 16 == 0 is enough): 8 waves with one
+    # round (K = 4096) and two (K = 7168, 4480 = 35 blocks: a ragged second round), 4 waves with many rounds (K = 18432) and
+    # with one (N % 128 != 0 at short K), ragged N (576, 1088), every token count class
+    (1, 512, 4096), (4, 1536, 7168), (16, 7168, 2048), (2, 36864, 7168), (1, 512, 18432), (12, 48, 1152),
     # three-stage mid-M kernel: 64 / 128 token tiles x 256 / 192 / 128 channel tiles, whole-K and split, ragged M, K blocks per
     # range = 1, 2, 0 mod 3
     (48, 16384, 2048), (33, 16384, 2176), (40, 65536, 512), (200, 16384, 2048), (100, 32768, 640), (130, 8192, 7168),
@@ -25,7 +30,7 @@ FP8_ROUTE_SHAPES = [
     # (the pipelined kernel takes whole-K shapes only where N % 4 != 0 rules the mid-M kernel's split reduce out)
     (4096, 4352, 512), (4000, 4300, 400), (4096, 2178, 256), (4000, 2100, 272), (4096, 2176, 256),
     # generic kernel: every token-tile height, aligned and byte-granular loads, whole-K and split
-    (7, 1088, 512), (16, 576, 7168), (1, 1088, 3884), (17, 384, 2304), (20, 256, 264), (33, 512, 512), (64, 128, 3884),
+    (7, 1088, 512), (16, 576, 7168), (7, 1096, 512), (16, 584, 7168), (1, 1088, 3884), (17, 384, 2304), (20, 256, 264), (33, 512, 512), (64, 128, 3884),
     (50, 300, 520), (127, 128, 4096), (130, 640, 896), (1500, 640, 1000), (130, 200, 300), (2048, 4224, 264),
     # between 17 and 1024 tokens only K % 128 != 0 (or unaligned rows) leaves the mid-M kernel to the generic one
     (20, 256, 2064), (33, 256, 272), (100, 256, 400), (100, 640, 2064),
@@ -36,6 +41,8 @@ FP8_ROUTE_SHAPES = [
 FP8_REQUIRED_VARIANTS = {
     ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
     ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
+    ("decode_wavesplit", "w4", "one_round"), ("decode_wavesplit", "w4", "rounds"), ("decode_wavesplit", "w8", "one_round"),
+    ("decode_wavesplit", "w8", "rounds"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
     ("dma3", 64, "whole", "bn128"), ("dma3", 64, "split", "bn128"), ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"),
     ("dma3", 64, "whole", "bn192"), ("dma3", 64, "split", "bn192"), ("dma3", 128, "whole", "bn192"), ("dma3", 128, "split", "bn192"),
@@ -57,14 +64,16 @@ INT8_ROUTE_SHAPES = [
     (700, 6144, 14336), (100, 6144, 7168), (100, 28672, 512), (40, 6144, 14336), (20, 2048, 4096), (20, 4096, 1024),
     (50, 3000, 4224), (40, 8, 1024), (100, 16, 4096), (1000, 8, 128),
     (4096, 4096, 512), (4000, 4088, 1024),
-    (1, 16, 512), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
+    (1, 16, 512), (1, 24, 512), (3, 48, 1152), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
     # between 17 and 1024 tokens only K % 128 != 0 leaves the mid-M kernel to the generic one
     (20, 256, 2064), (33, 256, 272), (100, 256, 400), (100, 640, 2064),
 ]
 
+# (INT8 decode with a K split does not exist: from 8 K blocks on every INT8 decode shape takes the wave-split kernel)
 INT8_REQUIRED_VARIANTS = {
     ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
-    ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
+    ("decode_wavesplit", "w4", "one_round"), ("decode_wavesplit", "w4", "rounds"), ("decode_wavesplit", "w8", "one_round"),
+    ("decode_wavesplit", "w8", "rounds"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
     ("dma3", 64, "whole", "bn128"), ("dma3", 64, "split", "bn128"), ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"),
     ("pingpong", "kfull"),
@@ -88,6 +97,9 @@ def variant_of(plan: dict, K: int):
     if k == "decode":
         g = plan["groups_per_wg"]
         return (k, sp, f"gpw{g}" if g < 3 else "gpw3+")
+    if k == "decode_wavesplit":  # waves per workgroup; one round of K blocks or several
+        waves = plan["groups_per_wg"]
+        return (k, f"w{waves}", "rounds" if -(-K // 128) > 4 * waves else "one_round")
     if k == "dma3":
         return (k, plan["bm"], sp) if plan["bn"] == 256 else (k, plan["bm"], sp, f"bn{plan['bn']}")
     if k in ("pingpong", "pipelined"):

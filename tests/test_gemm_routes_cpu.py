@@ -92,7 +92,7 @@ def test_perturbed_plan_query():
 
     L = _lib.lib()
     n = L.mi355_route_constant_count()
-    assert n == 34 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
+    assert n == 38 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
     assert _lib.route_constants()["pp_fp8_us_per_kblock"] == 1.39
     buf = ctypes.create_string_buffer(256)
     assert L.mi355_gemm_plan_perturbed(1, 128, 7168, 18432, 1, n, 1.1, buf, len(buf)) == 1
@@ -114,8 +114,10 @@ def test_plan_query_rejects_bad_arguments():
     assert L.mi355_fp8_blockwise_mm_plan(16, 128, 128, 1, buf, len(buf)) == 1 and b"too small" in L.mi355_last_error()
     assert L.mi355_int8_scaled_mm_plan(0, 128, 128, 1, buf, len(buf)) == 1
     assert L.mi355_fp8_blockwise_mm_plan(16, 128, 128, 1, None, 0) == 1
+    p = _lib.gemm_plan("fp8", 8, 36864, 7168)
+    assert p["kernel"] == "decode" and p["splits"] == 7
     p = _lib.gemm_plan("fp8", 1, 36864, 7168)
-    assert p["kernel"] == "decode" and p["splits"] >= 1
+    assert p["kernel"] == "decode_wavesplit" and p["splits"] == 1 and p["bn"] == 16
 
 
 @pytest.mark.parametrize("kind,M,N,K", [("fp8", 16, 2048, 7168), ("fp8", 128, 36864, 7168), ("int8", 256, 4096, 14336)])

@@ -122,18 +122,21 @@ def test_fused_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (3, 16640, 4480), (8, 7168, 18432), (16, 512, 512), (5, 66048, 512), (9, 256, 128)])
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (8, 2048, 7168), (3, 16640, 4480), (8, 7168, 18432), (16, 512, 512), (5, 66048, 512),
+                                   (9, 256, 128)])
 def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype):
-    """At decode sizes the one-call linear has no quantizer launch: the GEMM kernel quantizes the tokens of each K range
-    in its prologue.  Same arithmetic on the same codes and scales as quantizer + GEMM in two steps, so the outputs must
-    be identical bit for bit (split and unsplit plans, several channel groups per workgroup, a short last K range, rows
-    past M); the two-step path is held to the oracle elsewhere, and once more here."""
+    """At decode sizes the one-call linear has no quantizer launch: the streaming decode kernel quantizes the tokens of
+    each K range in its prologue.  Same arithmetic on the same codes and scales as quantizer + GEMM in two steps, so where
+    the two-step GEMM takes the same kernel the outputs must be identical bit for bit (split and unsplit plans, several
+    channel groups per workgroup, a short last K range, rows past M).  Where the two-step GEMM takes the wave-split decode
+    kernel instead (M = 1 here) the sums are added in another order and both are held to the oracle."""
     from sglang_amd import _lib
     from sglang_amd.fp8_kernel import per_token_group_quant_fp8
     from sglang_amd.fp8_utils import fused_w8a8_block_fp8_linear as w8a8_block_fp8_linear
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
-    assert _lib.gemm_plan("fp8", M, N, K)["kernel"] == "decode"
+    kernel = _lib.gemm_plan("fp8", M, N, K)["kernel"]
+    assert kernel == ("decode_wavesplit" if M == 1 else "decode")
     x = make_activation(M, K, seed=M + N, dtype=dtype)
     x[0, :128] = 0  # a group of zeros: scale 1e-10 / 448, codes 0
     w_q, w_s = make_fp8_weight(N, K, seed=K)
@@ -141,10 +144,13 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
     fused = w8a8_block_fp8_linear(xg, wg, [128, 128], sg)
     q, s = per_token_group_quant_fp8(xg, 128, column_major_scales=True)
     two_step = fp8_blockwise_scaled_mm(q, wg.t(), s, sg.t(), dtype)
-    assert fused.dtype == dtype and torch.equal(fused.view(torch.int16), two_step.view(torch.int16))
+    assert fused.dtype == dtype
+    if kernel == "decode":
+        assert torch.equal(fused.view(torch.int16), two_step.view(torch.int16))
     xq, xs = oracle.group_quant(x, 128, mode="div")
     ref, mag = oracle.fp8_blockwise_mm(xq, w_q, xs, w_s, torch.float32, want_abs=True)
-    assert bool(((fused.float().cpu() - ref).abs() <= 1e-2 * ref.abs() + FP8_MAG_TOL * mag).all())
+    for out in (fused, two_step):
+        assert bool(((out.float().cpu() - ref).abs() <= 1e-2 * ref.abs() + FP8_MAG_TOL * mag).all())
 
 
 def test_block_fp8_linear_ragged_n_falls_back_to_the_triton_wrapper(gpu, oracle):
