@@ -253,5 +253,8 @@ WavesplitShape wavesplit_shape(int64_t K);
 bool wavesplit_supported(int64_t M, int64_t N, int64_t K);
 int launch_fp8_wavesplit(GemmParams& p, hipStream_t stream, const char* what);
 int launch_int8_wavesplit(GemmParams& p, hipStream_t stream, const char* what);
+// The FP8 kernel with packed power-of-two scales on both operands, applied by the MFMA (p.sa / p.sb point to the words,
+// p.sa_sk / p.sb_sn / p.sb_sk are word strides; see decode_wavesplit_kernel).
+int launch_fp8_wavesplit_ue8m0(GemmParams& p, hipStream_t stream, const char* what);
 
 }  // namespace mi355

@@ -28,8 +28,13 @@ __device__ __forceinline__ v8i as_v8i(const Frag& f) {
   return v8i{(int)f.lo.x, (int)f.lo.y, (int)f.lo.z, (int)f.lo.w, (int)f.hi.x, (int)f.hi.y, (int)f.hi.z, (int)f.hi.w};
 }
 
-template <bool IS_FP8, int W, int KBW>
+// UE8M0 (FP8 only): p.sa / p.sb point to 32-bit words of four exponent bytes (token words M-major: word (kb >> 2) * sa_sk + m;
+// weight words one row per weight row: (kb >> 2) * sb_sk + n * sb_sn, constant over a 128-row block) and the MFMA applies
+// them itself (v_mfma_scale_f32_16x16x128_f8f6f4: the weight row's byte with the A operand, the token's with the B
+// operand), accumulating in place: no scale arithmetic, no expansion of the exponents to fp32 in front of the GEMM.
+template <bool IS_FP8, int W, int KBW, bool UE8M0 = false>
 __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmParams p) {
+  static_assert(IS_FP8 || !UE8M0, "exponent scales belong to the FP8 path");
   using AccT = typename std::conditional<IS_FP8, float, int>::type;
   typedef AccT acc4 __attribute__((ext_vector_type(4)));
   __shared__ acc4 red[W][64];
@@ -42,7 +47,7 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
   const uint8_t* wrow = p.b + (int64_t)(n0 + l16) * p.ldb + q * 16;
   const uint8_t* trow = p.a + (int64_t)tok * p.lda + q * 16;
   const float* sa_row = IS_FP8 ? p.sa + (int64_t)tok * p.sa_sm : nullptr;
-  const float* sb_row = IS_FP8 ? p.sb + (int64_t)(n0 >> 7) * p.sb_sn : nullptr;  // wave-uniform
+  const float* sb_row = IS_FP8 ? p.sb + (int64_t)(UE8M0 ? n0 : (n0 >> 7)) * p.sb_sn : nullptr;  // wave-uniform
 
   acc4 acc = {0, 0, 0, 0};
   const int rounds = (p.kb_total + W * KBW - 1) / (W * KBW);
@@ -57,7 +62,10 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
       wf[j].hi = *reinterpret_cast<const u32x4*>(wrow + (int64_t)kc * KSTEP + 64);
       tf[j].lo = *reinterpret_cast<const u32x4*>(trow + (int64_t)kc * KSTEP);
       tf[j].hi = *reinterpret_cast<const u32x4*>(trow + (int64_t)kc * KSTEP + 64);
-      if constexpr (IS_FP8) {
+      if constexpr (UE8M0) {  // the words that hold block kc's bytes, kept as raw bits
+        sav[j] = sa_row[(int64_t)(kc >> 2) * p.sa_sk];
+        sbv[j] = sb_row[(int64_t)(kc >> 2) * p.sb_sk];
+      } else if constexpr (IS_FP8) {
         sav[j] = sa_row[(int64_t)kc * p.sa_sk];
         sbv[j] = sb_row[(int64_t)kc * p.sb_sk];
       }
@@ -67,8 +75,16 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < KBW; ++j) {
-      const bool valid = (r * KBW + j) * W + wave < p.kb_total;
-      if constexpr (IS_FP8) {
+      const int kb = (r * KBW + j) * W + wave;
+      const bool valid = kb < p.kb_total;
+      if constexpr (UE8M0) {
+        const int shift = 8 * (min(kb, p.kb_total - 1) & 3);
+        const int ea = (int)((__float_as_uint(sbv[j]) >> shift) & 0xffu), eb = (int)((__float_as_uint(sav[j]) >> shift) & 0xffu);
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        Frag t = tf[j];
+        if (!valid) t.lo = z, t.hi = z;  // a block past the end of K multiplies zeros
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(t), acc, 0, 0, 0, ea, 0, eb);
+      } else if constexpr (IS_FP8) {
         const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(tf[j]), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0,
                                                                           0, 0, 0, 0);
         const float sc = valid ? sav[j] * sbv[j] : 0.f;
@@ -124,9 +140,9 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
   }
 }
 
-template <bool IS_FP8, int W, int KBW>
+template <bool IS_FP8, int W, int KBW, bool UE8M0 = false>
 int launch_variant(const GemmParams& p, hipStream_t stream, const char* what) {
-  hipLaunchKernelGGL((decode_wavesplit_kernel<IS_FP8, W, KBW>), dim3((unsigned)(p.N / 16)), dim3(64 * W), 0, stream, p);
+  hipLaunchKernelGGL((decode_wavesplit_kernel<IS_FP8, W, KBW, UE8M0>), dim3((unsigned)(p.N / 16)), dim3(64 * W), 0, stream, p);
   return check_launch(what);
 }
 
@@ -155,5 +171,10 @@ bool wavesplit_supported(int64_t M, int64_t N, int64_t K) { return M >= 1 && M <
 
 int launch_fp8_wavesplit(GemmParams& p, hipStream_t stream, const char* what) { return launch_wavesplit<true>(p, stream, what); }
 int launch_int8_wavesplit(GemmParams& p, hipStream_t stream, const char* what) { return launch_wavesplit<false>(p, stream, what); }
+int launch_fp8_wavesplit_ue8m0(GemmParams& p, hipStream_t stream, const char* what) {
+  p.splits = 1, p.tiles_m = 1, p.tiles_n = p.N / 16;
+  const WavesplitShape s = wavesplit_shape(p.K);
+  return s.waves == 4 ? launch_variant<true, 4, 4, true>(p, stream, what) : launch_variant<true, 8, 4, true>(p, stream, what);
+}
 
 }  // namespace mi355

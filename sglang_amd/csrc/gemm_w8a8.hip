@@ -821,6 +821,10 @@ extern "C" int mi355_fp8_blockwise_mm_ue8m0(const void* a, const void* b, const 
     p.splits = 1, p.kb_per_split = p.kb_total;
     return launch_fp8_pp_ue8m0(p, st, what);
   }
+  if (r.kernel == RK_WAVESPLIT && K % KSTEP == 0) {
+    // decode sizes on the wave-split kernel: the same, one launch, no workspace
+    return launch_fp8_wavesplit_ue8m0(p, st, what);
+  }
   // every other shape: exponents to fp32 scales in the head of the workspace (tokens M-major, weights one row per
   // 128-channel block, read from the block's first channel), then the fp32-scale kernels
   const size_t head = ue8m0_unpacked_bytes(M, N, K);

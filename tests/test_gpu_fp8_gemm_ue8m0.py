@@ -5,8 +5,8 @@ python/sglang/srt/layers/quantization/fp8_kernel.py:1047-1065, fp8_utils.py:217-
 The oracle is the blockwise GEMM oracle fed with the decoded scales 2^(byte - 127).  Floating point:
 |out - ref| <= 1e-2 * |ref| + 1e-4 * mag, as for the fp32-scale GEMM (tests/test_gpu_fp8_gemm.py); with small-integer
 operands every product and partial sum is exact in fp32 and the result must match bit for bit, whichever kernel runs.
-Large shapes take the kernel whose MFMA applies the scales itself, the others the fp32-scale kernels behind an unpack
-step; both are covered, and so are K extents whose last exponent word is only partly used."""
+Large shapes and decode shapes on the wave-split kernel take kernels whose MFMA applies the scales itself, the others the
+fp32-scale kernels behind an unpack step; all are covered, and so are K extents whose last exponent word is only partly used."""
 import pytest
 import torch
 
@@ -18,8 +18,10 @@ FP8 = torch.float8_e4m3fn
 
 # (M, N, K): two-phase kernel with hardware scales (>= 256 tiles of 256 x 256): K of 4, 9 and 5 blocks; ragged M;
 # then decode, mid-M, generic routes through the unpack step
+# decode sizes on the wave-split kernel, which also lets the MFMA apply the scales (8 and 4 waves, a ragged last round and a
+# partly used last exponent word: K = 4480 is 35 blocks; N = 576 is not a multiple of 128)
 SHAPES = [(4096, 4352, 512), (4096, 4352, 1152), (4000, 4352, 640), (4, 512, 1024), (16, 2048, 7168), (200, 16384, 2048),
-          (50, 384, 512), (1500, 640, 1024)]
+          (50, 384, 512), (1500, 640, 1024), (2, 2048, 7168), (3, 1536, 4480), (1, 1024, 18432), (5, 576, 2048)]
 
 
 def _unpack_bytes(words, groups):
@@ -66,7 +68,7 @@ def test_ue8m0_gemm_against_oracle(gpu, oracle, M, N, K):
     check_fp8_gemm(out[rows.to(gpu)], ref, mag, f"M={M} N={N} K={K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 4352, 1152), (16, 2048, 1024), (200, 16384, 640)])
+@pytest.mark.parametrize("M,N,K", [(4096, 4352, 1152), (16, 2048, 1024), (200, 16384, 640), (2, 2048, 1152), (3, 144, 4480)])
 def test_ue8m0_gemm_exact_integers(gpu, oracle, M, N, K):
     """Operands in {-2..2}, exponents in a narrow band: every block product and every partial sum is an integer times a
     power of two well inside fp32, so any summation order gives the same bits."""
