@@ -265,6 +265,14 @@ int mi355_gemm_plan_perturbed(int is_fp8, int64_t M, int64_t N, int64_t K, int a
 int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream);
 
 /*
+ * The same with the row sums: x_sum[m] = T(sum_k f32(x[m,k])), accumulated in fp32 and rounded to the input's type T, which
+ * is also the type of x_sum [M].  Replaces per_token_quant_int8(cal_sum=True) (int8_kernel.py:52-54, :66-69; the INT8
+ * mixture-of-experts path uses the sums).  The reference's reduction order is whatever Triton's tl.sum emits, so the sum is
+ * defined up to fp32 reassociation; codes and scales are those of mi355_per_token_quant_int8, bit for bit.
+ */
+int mi355_per_token_quant_int8_sum(const void* x, int x_dtype, void* q, float* s, void* x_sum, int64_t M, int64_t K, void* stream);
+
+/*
  * Per-token FP8 activation quantization: s[m] = max |x[m,:]| / 448 (no floor), q = e4m3fn(clamp(x * (1 / s[m]))) rounded to
  * nearest even; a row of zeros gives s = 0 and zeros.
  * Replaces sgl_per_token_quant_fp8 (sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:162-227, arithmetic of its

@@ -182,6 +182,16 @@ def per_token_quant_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return q, s
 
 
+def per_token_row_sum(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Row sums of per_token_quant_int8(cal_sum=True) (python/sglang/srt/layers/quantization/int8_kernel.py:52-54): the
+    exact sum of the row (fp64), the sum of magnitudes, and the exact sum rounded to the input's type.
+    PARITY UNPINNED at bit level: the reference adds in fp32 in whatever order Triton's tl.sum emits, so a conforming
+    result lies within fp32 reassociation error of the exact sum before the final rounding; tests bound it by that."""
+    x = _cpu(x)
+    exact = x.double().sum(-1)
+    return exact, x.double().abs().sum(-1), exact.to(x.dtype)
+
+
 def per_token_quant_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """x [M,K] -> (e4m3fn [M,K], fp32 scales [M,1]); scale = max|x| / 448, zero rows give scale 0 and zeros."""
     x = _cpu(x)

@@ -43,6 +43,7 @@ EXPORTS = (
     "mi355_route_constant_value",
     "mi355_gemm_plan_perturbed",
     "mi355_per_token_quant_int8",
+    "mi355_per_token_quant_int8_sum",
     "mi355_per_token_quant_fp8",
     "mi355_row_group_quant_fp8",
     "mi355_per_tensor_quant_fp8",
@@ -119,6 +120,8 @@ def lib() -> ctypes.CDLL:
         fn.restype = i32
     L.mi355_per_token_quant_int8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
     L.mi355_per_token_quant_int8.restype = i32
+    L.mi355_per_token_quant_int8_sum.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
+    L.mi355_per_token_quant_int8_sum.restype = i32
     L.mi355_per_token_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
     L.mi355_per_token_quant_fp8.restype = i32
     L.mi355_row_group_quant_fp8.argtypes = [vp, i32, vp, vp, i64, i64, ctypes.c_float, i32, vp]

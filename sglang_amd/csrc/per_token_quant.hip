@@ -58,6 +58,25 @@ __device__ __forceinline__ float wave_allreduce_max(float v) {
   return r;
 }
 
+// Sum over the wave, the same value in every lane (butterfly over 16-lane rows, then the four rows in lane order).
+__device__ __forceinline__ float wave_allreduce_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));
+  float r = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  r += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  r += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return r;
+}
+
+// The row sum leaves in the input's type (int8_kernel.py:52-54: `x_sum.to(x_sum_ptr.dtype.element_ty)`).
+template <int DT>
+__device__ __forceinline__ void store_row_sum(void* x_sum, int64_t row, float v) {
+  if constexpr (DT == MI355_F32) reinterpret_cast<float*>(x_sum)[row] = v;
+  else reinterpret_cast<uint16_t*>(x_sum)[row] = (uint16_t)(DT == MI355_BF16 ? f32_to_bf16_bits(v) : f32_to_f16_bits(v));
+}
+
 // Scale of a row from its |x| maximum (written by the caller) and the factor the elements are multiplied with.
 template <bool FP8_OUT>
 __device__ __forceinline__ float row_scale(float amax, float& mul) {
@@ -103,8 +122,10 @@ __device__ __forceinline__ void emit_vector(const u32x4& raw, float mul, int8_t*
 }
 
 // One wave per row, the row in registers: NV vectors of eight two-byte elements per lane (K <= 512 * NV).
-template <int DT, bool FP8_OUT, int NV>
-__global__ __launch_bounds__(256) void per_token_quant_wave_kernel(const void* x, int8_t* q, float* s, int64_t M, int64_t K) {
+// SUM (INT8 only): also the fp32 sum of the row, rounded to the input's type (per_token_quant_int8(cal_sum=True)).
+template <int DT, bool FP8_OUT, int NV, bool SUM = false>
+__global__ __launch_bounds__(256) void per_token_quant_wave_kernel(const void* x, int8_t* q, float* s, int64_t M, int64_t K,
+                                                                   void* x_sum = nullptr) {
   static_assert(DT != MI355_F32, "two-byte inputs");
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -113,6 +134,7 @@ __global__ __launch_bounds__(256) void per_token_quant_wave_kernel(const void* x
   const u32x4* src = reinterpret_cast<const u32x4*>(x) + row * nvec;
   u32x4 keep[NV];
   float amax = FP8_OUT ? 0.f : 1e-10f;
+  [[maybe_unused]] float total = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = lane + 64 * i;
@@ -124,11 +146,19 @@ __global__ __launch_bounds__(256) void per_token_quant_wave_kernel(const void* x
     unpack16<DT>(keep[i], f);
 #pragma unroll
     for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(f[j]));
+    if constexpr (SUM) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) total += f[j];
+    }
   }
   amax = wave_allreduce_max(amax);
   float mul;
   const float scale = row_scale<FP8_OUT>(amax, mul);
   if (lane == 0) s[row] = scale;
+  if constexpr (SUM) {
+    total = wave_allreduce_sum(total);
+    if (lane == 0) store_row_sum<DT>(x_sum, row, total);
+  }
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int v = lane + 64 * i;
@@ -138,13 +168,16 @@ __global__ __launch_bounds__(256) void per_token_quant_wave_kernel(const void* x
 
 // ROW_GROUP (FP8 only): the row is one quantization group: absmax floored at eps; DIVIDE: elements are divided by the
 // scale instead of multiplied by its reciprocal.
-template <int DT, bool FP8_OUT, bool ROW_GROUP = false, bool DIVIDE = false>
-__global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int8_t* q, float* s, int64_t K, float eps) {
+template <int DT, bool FP8_OUT, bool ROW_GROUP = false, bool DIVIDE = false, bool SUM = false>
+__global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int8_t* q, float* s, int64_t K, float eps,
+                                                              void* x_sum = nullptr) {
   static_assert(FP8_OUT || !ROW_GROUP, "whole-row groups are built for FP8 codes");
   static_assert(ROW_GROUP || !DIVIDE, "division is a mode of the whole-row group");
   constexpr int VEC = (DT == MI355_F32) ? 4 : 8;
   constexpr int KEEP = 4;  // vectors per thread kept in registers
   __shared__ float wave_max[4];
+  __shared__ float wave_sum[4];
+  [[maybe_unused]] float total = 0.f;
   const int64_t row = blockIdx.x;
   const int64_t nvec = K / VEC;
   const u32x4* src = reinterpret_cast<const u32x4*>(x) + row * nvec;
@@ -158,16 +191,31 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int
     unpack16<DT>(keep[i], f);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) amax = fmaxf(amax, fabsf(f[j]));
+    if constexpr (SUM) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) total += f[j];
+    }
   }
   for (int64_t v = threadIdx.x + 256 * KEEP; v < nvec; v += 256) {
     float f[VEC];
     unpack16<DT>(src[v], f);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) amax = fmaxf(amax, fabsf(f[j]));
+    if constexpr (SUM) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) total += f[j];
+    }
   }
   amax = wave_allreduce_max(amax);
-  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = amax;
+  if constexpr (SUM) total = wave_allreduce_sum(total);
+  if ((threadIdx.x & 63) == 0) {
+    wave_max[threadIdx.x >> 6] = amax;
+    if constexpr (SUM) wave_sum[threadIdx.x >> 6] = total;
+  }
   __syncthreads();
+  if constexpr (SUM) {
+    if (threadIdx.x == 0) store_row_sum<DT>(x_sum, row, (wave_sum[0] + wave_sum[1]) + (wave_sum[2] + wave_sum[3]));
+  }
   amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
   float mul;
   float scale = row_scale<FP8_OUT>(amax, mul);
@@ -192,15 +240,15 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* x, int
 namespace mi355 {
 namespace {
 
-template <bool FP8_OUT, bool ROW_GROUP = false, bool DIVIDE = false>
+template <bool FP8_OUT, bool ROW_GROUP = false, bool DIVIDE = false, bool SUM = false>
 int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K, void* stream,
-                    float eps = 0.f) {
+                    float eps = 0.f, void* x_sum = nullptr) {
   clear_error();
   MI355_REQUIRE(M >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
   MI355_REQUIRE(x_dtype == MI355_F32 || x_dtype == MI355_F16 || x_dtype == MI355_BF16, MI355_ERR_INVALID_ARGUMENT,
                 "%s: input must be float32, float16 or bfloat16", what);
   if (M == 0 || K == 0) return MI355_OK;
-  MI355_REQUIRE(x && q && s, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  MI355_REQUIRE(x && q && s && (!SUM || x_sum), MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
   MI355_REQUIRE((K * (int64_t)dtype_size(x_dtype)) % 16 == 0, MI355_ERR_UNSUPPORTED,
                 "%s: a row must span a multiple of 16 input bytes", what);
   MI355_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)q % 8 == 0), MI355_ERR_INVALID_ARGUMENT,
@@ -212,7 +260,7 @@ int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float
     const dim3 grid((unsigned)((M + 3) / 4));
     const int nv = (int)((K / 8 + 63) / 64);
 #define MI355_WAVE_ROWS(DT, NV) \
-  hipLaunchKernelGGL((per_token_quant_wave_kernel<DT, FP8_OUT, NV>), grid, dim3(256), 0, st, x, qq, s, M, K)
+  hipLaunchKernelGGL((per_token_quant_wave_kernel<DT, FP8_OUT, NV, SUM>), grid, dim3(256), 0, st, x, qq, s, M, K, x_sum)
     if (x_dtype == MI355_BF16) {
       if (nv <= 4) MI355_WAVE_ROWS(MI355_BF16, 4);
       else if (nv <= 8) MI355_WAVE_ROWS(MI355_BF16, 8);
@@ -227,13 +275,13 @@ int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float
   }
   switch (x_dtype) {
     case MI355_F32:
-      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F32, FP8_OUT, ROW_GROUP, DIVIDE>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F32, FP8_OUT, ROW_GROUP, DIVIDE, SUM>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps, x_sum);
       break;
     case MI355_F16:
-      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F16, FP8_OUT, ROW_GROUP, DIVIDE>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_F16, FP8_OUT, ROW_GROUP, DIVIDE, SUM>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps, x_sum);
       break;
     default:
-      hipLaunchKernelGGL((per_token_quant_kernel<MI355_BF16, FP8_OUT, ROW_GROUP, DIVIDE>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps);
+      hipLaunchKernelGGL((per_token_quant_kernel<MI355_BF16, FP8_OUT, ROW_GROUP, DIVIDE, SUM>), dim3((unsigned)M), dim3(256), 0, st, x, qq, s, K, eps, x_sum);
   }
   return check_launch(what);
 }
@@ -244,6 +292,11 @@ int per_token_quant(const char* what, const void* x, int x_dtype, void* q, float
 extern "C" int mi355_per_token_quant_int8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K,
                                           void* stream) {
   return mi355::per_token_quant<false>("mi355_per_token_quant_int8", x, x_dtype, q, s, M, K, stream);
+}
+
+extern "C" int mi355_per_token_quant_int8_sum(const void* x, int x_dtype, void* q, float* s, void* x_sum, int64_t M, int64_t K,
+                                              void* stream) {
+  return mi355::per_token_quant<false, false, false, true>("mi355_per_token_quant_int8_sum", x, x_dtype, q, s, M, K, stream, 0.f, x_sum);
 }
 
 extern "C" int mi355_per_token_quant_fp8(const void* x, int x_dtype, void* q, float* s, int64_t M, int64_t K,

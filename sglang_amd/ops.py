@@ -552,10 +552,17 @@ def int8_mm_raw_accumulators(mat_a: torch.Tensor, mat_b: torch.Tensor) -> torch.
     return out
 
 
-def per_token_quant_int8(x2d: torch.Tensor, q: torch.Tensor, s: torch.Tensor) -> None:
+def per_token_quant_int8(x2d: torch.Tensor, q: torch.Tensor, s: torch.Tensor, x_sum: Optional[torch.Tensor] = None) -> None:
+    """Codes and scales of the rows of `x2d`; with `x_sum` ([M], the input's type) also the row sums."""
     M, K = x2d.shape
-    if M:
+    if not M:
+        return
+    if x_sum is None:
         check(lib().mi355_per_token_quant_int8(x2d.data_ptr(), _DT[x2d.dtype], q.data_ptr(), s.data_ptr(), M, K, _stream()))
+    else:
+        _require(x_sum.dtype == x2d.dtype and x_sum.numel() == M and x_sum.is_contiguous(), "x_sum must be [M] in the input's type")
+        check(lib().mi355_per_token_quant_int8_sum(x2d.data_ptr(), _DT[x2d.dtype], q.data_ptr(), s.data_ptr(), x_sum.data_ptr(), M, K,
+                                                   _stream()))
 
 
 # ---------------------------------------------------------------- registration

@@ -130,6 +130,29 @@ def test_per_token_quant_int8(gpu, oracle, dtype, M, K):
     assert torch.equal(q.cpu(), q_o)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K", [(1, 512), (7, 4096), (64, 14336), (33, 16384 + 512), (6, 2056)])
+def test_per_token_quant_int8_with_row_sums(gpu, oracle, dtype, M, K):
+    """per_token_quant_int8(cal_sum=True), int8_kernel.py:52-54, :66-69: codes and scales unchanged (bit for bit), plus the
+    row sums in the input's type.  The reference's fp32 reduction order is Triton's, not defined by the source, so the sum is
+    held to the exact (fp64) sum within fp32 reassociation error, K * 2^-24 * sum|x|, plus half a unit of the output type;
+    a row of small integers, where every partial sum is exact, must come back exactly."""
+    from sglang_amd.int8_kernel import per_token_quant_int8
+    from sglang_amd.workloads import make_activation
+
+    x = make_activation(M, K, seed=M + K, dtype=dtype)
+    x[0] = torch.randint(-3, 4, (K,), generator=torch.Generator().manual_seed(K)).to(dtype)
+    q, s, x_sum = per_token_quant_int8(x.view(1, M, K).to(gpu), cal_sum=True)
+    assert x_sum.dtype == dtype and tuple(x_sum.shape) == (1, M) and tuple(s.shape) == (1, M, 1) and q.dtype == torch.int8
+    q_o, s_o = oracle.per_token_quant_int8(x)
+    assert torch.equal(s.cpu().view(M, 1).view(torch.int32), s_o.view(torch.int32)) and torch.equal(q.cpu().view(M, K), q_o)
+    exact, mag, rounded = oracle.per_token_row_sum(x)
+    got = x_sum.cpu().view(M).double()
+    half_ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -24}[dtype]
+    assert bool(((got - exact).abs() <= half_ulp * 1.001 * exact.abs() + K * 2.0 ** -24 * mag + 1e-30).all())
+    assert got[0] == exact[0] == float(rounded[0])
+
+
 def test_int8_linear_end_to_end(gpu, oracle):
     """W8A8Int8LinearMethod.apply (python/sglang/srt/layers/quantization/w8a8_int8.py:387-417):
     per_token_quant_int8 then int8_scaled_mm, against the bf16 linear it approximates."""

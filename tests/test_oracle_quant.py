@@ -410,3 +410,19 @@ def test_block_dequant_against_torch(oracle, dtype):
     ref = (q.to(torch.float32) * s.repeat_interleave(128, 0).repeat_interleave(128, 1)[:n, :k]).to(dtype)
     assert torch.equal(out.view(torch.int16 if dtype != torch.float32 else torch.int32),
                        ref.view(torch.int16 if dtype != torch.float32 else torch.int32))
+
+
+def test_row_sum_known_answers(oracle):
+    """per_token_row_sum against sums that can be written down: small integers (exact in every type), a row whose terms
+    cancel to one survivor, and Python's exactly rounded fsum on random fp32 rows."""
+    import math
+
+    x = torch.tensor([[1.0, 2.0, 3.0, -4.0], [0.5, 0.25, -0.75, 100.0]], dtype=torch.bfloat16)
+    exact, mag, rounded = oracle.per_token_row_sum(x)
+    assert exact.tolist() == [2.0, 100.0] and mag.tolist() == [10.0, 101.5] and rounded.dtype == torch.bfloat16
+    assert rounded.tolist() == [2.0, 100.0]
+    y = torch.randn(3, 1000, generator=torch.Generator().manual_seed(0))
+    exact, mag, rounded = oracle.per_token_row_sum(y)
+    for r in range(3):
+        assert abs(float(exact[r]) - math.fsum(y[r].double().tolist())) <= 1e-12 * float(mag[r])
+        assert float(rounded[r]) == float(torch.tensor(math.fsum(y[r].double().tolist())).float())
