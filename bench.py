@@ -647,7 +647,7 @@ def bench_silu_quant(steps, warmup):
     return {
         "workload": f"silu_mul_quant M={T} H={H} g=128 bf16 [M,2H] -> e4m3fn [M,H], packed UE8M0 scales",
         "value": alg / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
-        "dtype": "f32 arithmetic, e4m3fn out", "kernel": "silu_mul_quant",
+        "dtype": "f32 arithmetic, e4m3fn out", "kernel": "silu_mul_quant", "traffic_key": "silu_mul_quant",
         "roofline": _roofline(0, alg, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
     }
 
@@ -698,7 +698,7 @@ def bench_row_quant(kind, steps, warmup):
     st = _stats(ms, b2b)
     return {
         "workload": name, "value": alg / (wall / steps) / 1e9, "unit": "GB/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
-        "dtype": "f32 arithmetic, 8-bit out", "kernel": kern, "roofline": _roofline(0, alg, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
+        "dtype": "f32 arithmetic, 8-bit out", "kernel": kern, "traffic_key": kind, "roofline": _roofline(0, alg, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
     }
 
 
@@ -731,6 +731,8 @@ def _measured_traffic():
 
 
 def _traffic_key(rec):
+    if "traffic_key" in rec:
+        return rec["traffic_key"]
     head = rec["workload"].split(" (")[0].split(",")[0]  # e.g. "fp8_gemm gate_up M=4096 K=7168 N=36864"
     parts = head.split()
     if parts[0] == "group":
@@ -746,6 +748,8 @@ def _short(rec):
            "bound": ro["bound"], "frac": ro["frac"]}
     if "kernel" in rec:
         row["kern"] = rec["kernel"]
+    if ro.get("traffic"):
+        row["traffic"] = ro["traffic"]
     if "operator_frac" in rec:
         row["operator_frac_same_call"] = rec["operator_frac"]
     if "streams" in rec:
