@@ -28,9 +28,9 @@ Infinity Cache.
 
 Per-launch durations are HIP events on the launch stream (torch's current stream, which is the stream
 handed to the C ABI).  `roofline.achieved` = algorithmic FLOPs (2*M*N*K) or bytes per launch / MEDIAN
-launch duration; `b2b_ms` is the average over the same launches queued back to back between one event
-pair (no per-launch event overhead; for kernels of tens of microseconds it also hides the tail of one
-launch behind the head of the next).  `cpu_baseline` times the CPU oracle on a bounded sample of the
+launch duration, the one basis of every `roofline.frac`; `kernel_ms.b2b` is the average over the same launches
+queued back to back between one event pair (no per-launch event overhead; for kernels of tens of microseconds it
+also hides the tail of one launch behind the head of the next) and `roofline.frac_b2b` the fraction on it.  `cpu_baseline` times the CPU oracle on a bounded sample of the
 same workload on this host's cores.
 """
 from __future__ import annotations
