@@ -234,6 +234,9 @@ int launch_int8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const ch
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases, direct-to-LDS loads,
 // 32x32x32 MFMA); gemm_int8_pp.hip.  Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
 int launch_int8_pp(GemmParams& p, hipStream_t stream, const char* what);
+// Mid-M INT8 GEMM (128 x 256 tile, the two-phase schedule over three LDS stages); gemm_int8_pp128.hip.  Same requirements;
+// optional split along K: the caller sets p.splits, p.kb_per_split and p.ws (int32 partials, ordered reduce afterwards).
+int launch_int8_pp128(GemmParams& p, hipStream_t stream, const char* what);
 
 // Small-M blockwise FP8 GEMM streaming the weight through wave-private LDS, no barriers; gemm_fp8_decode.hip.
 // decode_splits() is the split count it wants for a shape; the caller sets p.splits, p.kb_per_split and p.ws.

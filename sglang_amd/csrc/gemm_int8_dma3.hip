@@ -222,10 +222,12 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
 
 }  // namespace
 
-// Tiling and split are those of the FP8 mid-M kernel (dma3_plan): same tile shapes, same byte model.
+// Tiling and split are those of the FP8 mid-M kernel (dma3_plan): same tile shapes, same byte model.  The 128 x 256 tile is
+// not built here: the two-phase 128-token kernel (gemm_int8_pp128.hip) serves it.
 int launch_int8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what) {
   if (bn == 128) return bm == 64 ? launch_bm<64, 128>(p, stream, what) : launch_bm<128, 128>(p, stream, what);
-  return bm == 64 ? launch_bm<64, 256>(p, stream, what) : launch_bm<128, 256>(p, stream, what);
+  if (bm == 128) return launch_int8_pp128(p, stream, what);
+  return launch_bm<64, 256>(p, stream, what);
 }
 
 }  // namespace mi355

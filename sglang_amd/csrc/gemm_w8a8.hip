@@ -401,8 +401,8 @@ int launch_tile(GemmParams& p, bool aligned, hipStream_t stream, const char* wha
 
 // Which kernel serves a problem, with which tiling.  One function decides for the launcher and for the plan query, so
 // what the query reports is what runs.
-enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_PINGPONG, RK_PIPELINED, RK_GENERIC, RK_WAVESPLIT };
-const char* const ROUTE_NAMES[] = {"decode", "dma3", "pingpong", "pipelined", "generic", "decode_wavesplit"};
+enum RouteKernel { RK_DECODE = 0, RK_DMA3, RK_PINGPONG, RK_PIPELINED, RK_GENERIC, RK_WAVESPLIT, RK_PP128 };
+const char* const ROUTE_NAMES[] = {"decode", "dma3", "pingpong", "pipelined", "generic", "decode_wavesplit", "pingpong128"};
 
 struct Route {
   int kernel;
@@ -467,7 +467,9 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
       }
     }
     if (N % 4 == 0 || dp.efficiency >= route_constants().dma3_min_efficiency) {
-      r.kernel = RK_DMA3, r.bm = dp.bm, r.bn = dp.bn, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
+      // INT8: the 128 x 256 tile of this family is the two-phase 128-token kernel (gemm_int8_pp128.hip)
+      r.kernel = (!is_fp8 && dp.bm == 128 && dp.bn == 256) ? RK_PP128 : RK_DMA3;
+      r.bm = dp.bm, r.bn = dp.bn, r.splits = dp.splits, r.kb_per_split = dp.kb_per_split;
       return r;
     }
   }
@@ -575,6 +577,14 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
       rc = IS_FP8 ? launch_fp8_decode(p, r.groups_per_wg, stream, what) : launch_int8_decode(p, r.groups_per_wg, stream, what);
       break;
     case RK_WAVESPLIT: return IS_FP8 ? launch_fp8_wavesplit(p, stream, what) : launch_int8_wavesplit(p, stream, what);
+    case RK_PP128:
+      if constexpr (IS_FP8) {
+        set_error("%s: the 128-token two-phase kernel is built for INT8", what);
+        return MI355_ERR_UNSUPPORTED;
+      } else {
+        rc = launch_int8_pp128(p, stream, what);
+      }
+      break;
     case RK_DMA3:
       rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, r.bn, stream, what) : launch_int8_dma3(p, r.bm, r.bn, stream, what);
       break;

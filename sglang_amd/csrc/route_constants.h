@@ -22,8 +22,10 @@ struct RouteConstants {
   //      share of the chip's streaming rate.  Fitted to a sweep of 24 shapes x every (tile, split) (FP8) and to
   //      K = 4096 -> N = 4096 ... 28672, K = 14336 -> N = 4096 at 24 ... 1024 tokens (INT8).
   double dma3_hbm_bytes_per_us = 5.5e6;  // streaming rate of the 8-rows x 128-B access shape with two blocks in flight per CU
-  // order: 128x256, 64x256, 128x128, 64x128, 128x192, 64x192 (token x channel tile); [0] FP8, [1] INT8 (no 192-wide tiles)
-  double dma3_tile_us[2][6] = {{0.88, 0.58, 0.52, 0.40, 0.68, 0.50}, {1.14, 0.71, 0.64, 0.44, 0.0, 0.0}};
+  // order: 128x256, 64x256, 128x128, 64x128, 128x192, 64x192 (token x channel tile); [0] FP8, [1] INT8 (no 192-wide tiles).
+  // The INT8 128x256 entry is the two-phase 128-token kernel (gemm_int8_pp128.hip), 0.84 us; the lockstep kernel it
+  // replaced took 1.14 us (M=4096 K=4096 N=1536: 42.0 -> 30.8 us, M=1024 N=6144: 42.1 -> 30.6, M=256 N=28672: 55.8 -> 44.6).
+  double dma3_tile_us[2][6] = {{0.88, 0.58, 0.52, 0.40, 0.68, 0.50}, {0.84, 0.71, 0.64, 0.44, 0.0, 0.0}};
   double dma3_latency_us[2][6] = {{1.2, 1.0, 0.7, 0.51, 1.0, 0.75}, {0.96, 0.68, 0.59, 0.54, 0.0, 0.0}};
   double dma3_busy_chip_factor = 1.2;    // on the tile's own time in a round that keeps > 200 CUs multiplying: the clock drops
   double dma3_long_row_factor = 1.2;     // on the latency floor for weight rows longer than 8 KB (K = 18432 against K = 7168)

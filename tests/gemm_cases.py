@@ -62,6 +62,9 @@ INT8_ROUTE_SHAPES = [
     (100, 16384, 3584), (500, 4096, 14336),
     # the mid-M kernel's 128-channel tiles (and 128 x 256 with a K split): ragged M, a ragged last channel tile
     (700, 6144, 14336), (100, 6144, 7168), (100, 28672, 512), (40, 6144, 14336), (20, 2048, 4096), (20, 4096, 1024),
+    (33, 12288, 14336),  # 64 x 256 tiles with a K split
+    # the 128 x 256 tile is the two-phase 128-token kernel: whole K and split, ragged M (200, 300, 700), K steps 0, 1, 2 mod 3
+    (130, 8192, 1024), (250, 16384, 1152), (256, 28672, 4096),
     (50, 3000, 4224), (40, 8, 1024), (100, 16, 4096), (1000, 8, 128),
     (4096, 4096, 512), (4000, 4088, 1024),
     (1, 16, 512), (1, 24, 512), (3, 48, 1152), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
@@ -74,7 +77,7 @@ INT8_REQUIRED_VARIANTS = {
     ("decode", "whole", "gpw1"), ("decode", "whole", "gpw2"), ("decode", "whole", "gpw3+"),
     ("decode_wavesplit", "w4", "one_round"), ("decode_wavesplit", "w4", "rounds"), ("decode_wavesplit", "w8", "one_round"),
     ("decode_wavesplit", "w8", "rounds"),
-    ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
+    ("dma3", 64, "whole"), ("dma3", 64, "split"), ("pingpong128", "whole"), ("pingpong128", "split"),
     ("dma3", 64, "whole", "bn128"), ("dma3", 64, "split", "bn128"), ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"),
     ("pingpong", "kfull"),
     ("generic", 16, "aligned", "whole"), ("generic", 32, "aligned", "split"), ("generic", 64, "aligned", "whole"),
@@ -100,6 +103,8 @@ def variant_of(plan: dict, K: int):
     if k == "decode_wavesplit":  # waves per workgroup; one round of K blocks or several
         waves = plan["groups_per_wg"]
         return (k, f"w{waves}", "rounds" if -(-K // 128) > 4 * waves else "one_round")
+    if k == "pingpong128":
+        return (k, sp)
     if k == "dma3":
         return (k, plan["bm"], sp) if plan["bn"] == 256 else (k, plan["bm"], sp, f"bn{plan['bn']}")
     if k in ("pingpong", "pipelined"):

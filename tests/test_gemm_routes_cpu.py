@@ -46,7 +46,6 @@ RECORDED_BOUNDARIES = {
     ("fp8", (128, 7168, 18432)): {(128, 128, 4): 48.8, (64, 128, 2): 50.0, (128, 192, 6): 52.7},
     ("fp8", (4096, 1536, 7168)): {(128, 192, 1): 63.0, (128, 256, 1): 65.8},
     ("fp8", (4096, 576, 7168)): {(64, 192, 1): 45.7, (128, 128, 1): 47.0},
-    ("int8", (256, 28672, 4096)): {(128, 256, 1): 56.2, (128, 128, 1): 61.2},
     ("int8", (256, 4096, 14336)): {(128, 128, 4): 48.9, (64, 256, 4): 49.9, (128, 128, 3): 47.4},
 }
 BOUNDARY_COST = 1.10  # the slower side of a recorded boundary may cost at most this much more than the dispatcher's choice
