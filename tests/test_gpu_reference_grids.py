@@ -6,7 +6,9 @@ rtol 0.02 / atol 1 against scale-then-multiply in fp32; sgl-kernel/tests/test_in
 M x N x K x bias x out_dtype with int8(N(0, 5)) operands, N(0, 1) scales of either sign and a bias of N(0, 10).
 
 The same grids, operand distributions and (for FP8) the same criterion are used here; the comparison values are built
-with torch on the GPU, as the reference's tests build theirs.  FP8 is floating point, so the reference's tolerance
+with torch on the GPU, as the reference's tests build theirs, and - because that is one GPU library checking another - every
+FP8 case is also held to the CPU oracle on a sample of token rows over all channels, under the criterion of
+tests/fp8_tolerance.py.  FP8 is floating point, so the reference's tolerance
 applies; the INT8 result is held to the bits: exact integer accumulators (an fp64 matmul is exact at these sizes), then the
 epilogue f32(acc) * (sb[n] * sa[m]) + bias, each step rounded once.  Cases above 2^36 multiply-accumulates are left to
 the curated full-size tests (tests/test_gpu_fp8_gemm.py, tests/test_gpu_int8_gemm.py, tests/test_gpu_config_shapes.py).
@@ -32,13 +34,15 @@ def _m_major(t):
 
 @pytest.mark.parametrize("N", FP8_N)
 @pytest.mark.parametrize("K", FP8_K)
-def test_fp8_blockwise_scaled_mm_reference_grid(gpu, N, K):
+def test_fp8_blockwise_scaled_mm_reference_grid(gpu, oracle, N, K):
+    from fp8_tolerance import check_fp8_gemm
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
 
     g = torch.Generator(device=gpu).manual_seed(N * 31 + K)
     w = ((torch.rand(N, K, generator=g, device=gpu) - 0.5) * 2 * 448.0).clamp(-448, 448).to(FP8)
     sb = _m_major(torch.randn(K // 128, N // 128, generator=g, device=gpu) * 0.001)  # shaped like mat_b: [K / 128, N / 128]
     wb = w.float() * sb.t().repeat_interleave(128, 0).repeat_interleave(128, 1)
+    w_cpu = sw_cpu = None
     ran = 0
     for M in FP8_M:
         if M * N * K > MAX_MACS:
@@ -51,6 +55,13 @@ def test_fp8_blockwise_scaled_mm_reference_grid(gpu, N, K):
             out = fp8_blockwise_scaled_mm(a, w.t(), sa, sb, out_dtype)
             assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
             torch.testing.assert_close(out, want32.to(out_dtype), rtol=0.02, atol=1)
+        # the oracle on up to eight token rows (first, last, tile borders) over all channels; out is the fp16 result
+        rows = sorted({0, M - 1, M // 2, min(M - 1, 127), min(M - 1, 128), min(M - 1, 255), min(M - 1, 256), M // 3})
+        if w_cpu is None:
+            w_cpu, sw_cpu = w.cpu(), sb.t().contiguous().cpu()
+        idx = torch.tensor(rows, device=gpu)
+        ref, mag = oracle.fp8_blockwise_mm(a[idx].cpu().contiguous(), w_cpu, sa[idx].cpu().contiguous(), sw_cpu, torch.float32, want_abs=True)
+        check_fp8_gemm(out[idx], ref, mag, f"grid M={M} N={N} K={K}")
         ran += 1
     assert ran >= 5  # every (N, K) pair runs at least the five smallest token counts
 
@@ -153,7 +164,8 @@ def test_per_token_and_per_tensor_quant_fp8_reference_grid(gpu, oracle, tokens, 
 # and per-channel scales ~ N(0, 1e-3), bias ~ N(0, 1) in the output type; the reference's formula and its rtol 0.02 / atol 1.
 @pytest.mark.parametrize("N", [16, 128, 512, 1024, 4096])
 @pytest.mark.parametrize("K", [512, 1024, 4096, 8192, 16384])
-def test_fp8_scaled_mm_reference_grid(gpu, N, K):
+def test_fp8_scaled_mm_reference_grid(gpu, oracle, N, K):
+    from fp8_tolerance import check_fp8_gemm
     from sglang_amd.sgl_kernel import fp8_scaled_mm
 
     g = torch.Generator(device=gpu).manual_seed(N * 7 + K)
@@ -171,6 +183,11 @@ def test_fp8_scaled_mm_reference_grid(gpu, N, K):
                 out = fp8_scaled_mm(a, w.t(), sa, sb, out_dtype, b)
                 want = scaled.to(out_dtype) if b is None else scaled.to(out_dtype) + b.view(1, -1)
                 torch.testing.assert_close(out, want, rtol=0.02, atol=1)
+        # the last result (fp16, with bias) against the CPU oracle on a sample of token rows
+        rows = sorted({0, M - 1, M // 2, min(M - 1, 255), min(M - 1, 256), M // 3})
+        idx = torch.tensor(rows, device=gpu)
+        ref, mag = oracle.fp8_scaled_mm(a[idx].cpu().contiguous(), w.cpu(), sa[idx].cpu().contiguous(), sb.cpu(), torch.float32, None, want_abs=True)
+        check_fp8_gemm(out[idx], ref + bias.float().cpu()[None, :], mag, f"fp8_scaled_mm grid M={M} N={N} K={K}")
 
 
 # ---- python/sglang/test/test_block_fp8.py:326-398 (TestW8A8BlockFP8Matmul), both of its grids: the generic one with ragged
@@ -182,7 +199,8 @@ DSV3_NK = [(2112, 7168), (1536, 7168), (3072, 1536), (24576, 7168), (4096, 512),
            (7168, 2304), (7168, 512)]
 
 
-def _block_matmul_case(gpu, N, K, Ms, out_dtypes):
+def _block_matmul_case(gpu, oracle, N, K, Ms, out_dtypes):
+    from fp8_tolerance import check_fp8_gemm
     from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
 
     g = torch.Generator(device=gpu).manual_seed(N + K)
@@ -200,16 +218,21 @@ def _block_matmul_case(gpu, N, K, Ms, out_dtypes):
             ref = ref32.to(out_dtype).float()
             assert out.dtype == out_dtype and tuple(out.shape) == (M, N)
             assert float((out.float() - ref).abs().mean() / ref.abs().mean()) < 0.001, (M, N, K, out_dtype)
+        # the last result against the CPU oracle on a sample of token rows (ragged N and K included)
+        rows = sorted({0, M - 1, M // 2, min(M - 1, 255), min(M - 1, 256), M // 3})
+        idx = torch.tensor(rows, device=gpu)
+        want, mag = oracle.fp8_blockwise_mm(a[idx].cpu().contiguous(), w.cpu(), As[idx].cpu().contiguous(), Bs.cpu(), torch.float32, want_abs=True)
+        check_fp8_gemm(out[idx], want, mag, f"block matmul grid M={M} N={N} K={K}")
 
 
 @pytest.mark.parametrize("N,K", GENERIC_NK)
-def test_w8a8_block_fp8_matmul_generic_grid(gpu, N, K):
-    _block_matmul_case(gpu, N, K, [1, 7, 83, 512, 2048], [torch.float32, torch.half, torch.bfloat16])
+def test_w8a8_block_fp8_matmul_generic_grid(gpu, oracle, N, K):
+    _block_matmul_case(gpu, oracle, N, K, [1, 7, 83, 512, 2048], [torch.float32, torch.half, torch.bfloat16])
 
 
 @pytest.mark.parametrize("N,K", DSV3_NK)
-def test_w8a8_block_fp8_matmul_deepseek_grid(gpu, N, K):
-    _block_matmul_case(gpu, N, K, [64, 128, 512, 1024, 4096], [torch.bfloat16])
+def test_w8a8_block_fp8_matmul_deepseek_grid(gpu, oracle, N, K):
+    _block_matmul_case(gpu, oracle, N, K, [64, 128, 512, 1024, 4096], [torch.bfloat16])
 
 
 # ---- python/sglang/test/test_block_fp8.py:51-92 (TestPerTokenGroupQuantFP8) and :118-158 (TestStaticQuantFP8): inputs uniform
