@@ -17,6 +17,7 @@ FP8_ROUTE_SHAPES = [
     # round (K = 4096) and two (K = 7168, 4480 = 35 blocks: a ragged second round), 4 waves with many rounds (K = 18432) and
     # with one (N % 128 != 0 at short K), ragged N (576, 1088), every token count class
     (1, 512, 4096), (4, 1536, 7168), (16, 7168, 2048), (2, 36864, 7168), (1, 512, 18432), (12, 48, 1152),
+    (5, 48, 128), (16, 16, 256),  # a single K block (three of the four waves have nothing to add), a single workgroup
     # three-stage mid-M kernel: 64 / 128 token tiles x 256 / 192 / 128 channel tiles, whole-K and split, ragged M, K blocks per
     # range = 1, 2, 0 mod 3
     (48, 16384, 2048), (33, 16384, 2176), (40, 65536, 512), (200, 16384, 2048), (100, 32768, 640), (130, 8192, 7168),
@@ -67,7 +68,7 @@ INT8_ROUTE_SHAPES = [
     (130, 8192, 1024), (250, 16384, 1152), (256, 28672, 4096),
     (50, 3000, 4224), (40, 8, 1024), (100, 16, 4096), (1000, 8, 128),
     (4096, 4096, 512), (4000, 4088, 1024),
-    (1, 16, 512), (1, 24, 512), (3, 48, 1152), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
+    (1, 16, 512), (1, 24, 512), (3, 48, 1152), (5, 48, 128), (16, 16, 256), (17, 136, 1024), (64, 1024, 512), (100, 4096, 1024), (128, 16384, 512), (2048, 4224, 272),
     # between 17 and 1024 tokens only K % 128 != 0 leaves the mid-M kernel to the generic one
     (20, 256, 2064), (33, 256, 272), (100, 256, 400), (100, 640, 2064),
 ]
