@@ -20,7 +20,8 @@
 // kernels (chunks q and q + 4 per lane quarter: full-rate LDS reads).
 //
 // Split along K: every K range writes a partial tile to the caller's workspace and splitk_reduce_kernel adds them in a
-// fixed order (for INT8 the partials are int32 and the reduce kernel applies the epilogue).  INT8 uses two
+// fixed order.  (INT8 shapes with more than one K range all take the wave-split kernel of gemm_decode_wavesplit.hip, which
+// was measured faster for them at every decode size; the INT8 split variant of this kernel is therefore not built.)  INT8 uses two
 // v_mfma_i32_16x16x64_i8 per K block (chunk q of both operands, then chunk q + 4) and has no scales in the loop.
 // Requires K % 128 == 0, N % 128 == 0 and 16-byte aligned rows; other shapes take the generic kernel.
 #include "gemm_common.h"

@@ -1,4 +1,5 @@
-// Mid-M per-token x per-channel INT8 GEMM for gfx950: (64 or 128) x (256 or 128) macro tile, 8 waves, THREE LDS stages.
+// Mid-M per-token x per-channel INT8 GEMM for gfx950: 64 x 256, 128 x 128 or 64 x 128 macro tile, 8 waves, THREE LDS stages
+// (the 128 x 256 tile of this family is served by the two-phase kernel of gemm_int8_pp128.hip, which is a quarter faster).
 //
 // The loop structure is the one of gemm_fp8_dma3.hip: the direct-to-LDS loads of K step k+2 are issued while step k is
 // multiplied, the wait before the bare s_barrier that ends iteration k covers step k+1 only (s_waitcnt vmcnt(LOADS), the
