@@ -5,7 +5,12 @@ smoke check and the benchmark's CPU-baseline leg can compare the HIP kernels wit
 independent IEEE-fp32 restatement of the reference arithmetic.
 
 All tensors here are CPU ``torch`` tensors (torch is only the container: bf16/fp8 have
-no numpy dtype); every computation happens in the C library.
+no numpy dtype); every computation happens in the C library, except `per_token_row_sum`
+(an fp64 torch sum).
+
+Parity unpinned (see the functions' own notes and the header of qlinear_oracle.c): the order of
+the fp32 additions inside one 128-wide K block of the FP8 GEMM, the bits of exp inside the
+fused silu, and the fp32 reduction order of the row sums of per_token_quant_int8(cal_sum=True).
 """
 from __future__ import annotations
 
