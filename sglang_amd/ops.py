@@ -57,7 +57,8 @@ def _stream() -> int:
     """The current HIP stream; on a device's first use, the library's per-device set-up (it must not fall inside a graph
     capture, which the first launch of a process otherwise might)."""
     dev = torch.cuda.current_device()
-    if dev not in _ready_devices:
+    if dev not in _ready_devices and not torch.cuda.is_current_stream_capturing():
+        # (inside a capture the set-up is left alone: the two entry points that need it say so in their error)
         check(lib().mi355_qlinear_init())
         _ready_devices.add(dev)
     return torch.cuda.current_stream().cuda_stream
