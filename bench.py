@@ -348,7 +348,8 @@ def bench_fp8_ue8m0_gemm(name, M, K, N, steps, warmup):
     st = _stats(ms, b2b)
     flops, nbytes = gemm_flops(M, N, K), fp8_gemm_algorithmic_bytes(M, N, K)
     plan = _lib.gemm_plan("fp8", M, N, K)
-    kern = "pingpong (MFMA-applied scales)" if plan["kernel"] == "pingpong" else plan["kernel"] + " after unpack"
+    hw = plan["kernel"] in ("pingpong", "dma3", "decode_wavesplit") and K % 128 == 0  # kernels whose MFMA applies the exponents
+    kern = plan["kernel"] + (" (MFMA-applied scales)" if hw else " after unpack")
     return {
         "workload": f"fp8_gemm_ue8m0 {name} M={M} K={K} N={N} (e4m3fn x e4m3fn, packed UE8M0 scales on both sides, bf16 out)",
         "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,

@@ -39,6 +39,7 @@ struct GemmParams {
   int kb_total, kb_per_split, splits;
   int tiles_m, tiles_n;
   int out_dtype;
+  int ue8m0;  // FP8 only: sa / sb are packed exponent words and the route's kernel applies them in the MFMA (set by the UE8M0 entry point)
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -181,6 +182,9 @@ struct Dma3Plan {
 };
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8 = false);
 int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);  // bm: 64 or 128, bn: 128, 192 or 256, from dma3_plan()
+// The same for packed UE8M0 scales on both operands (p.sa / p.sb point to the words, p.sa_sk / p.sb_sn / p.sb_sk are word
+// strides; token words M-major with a pitch that is a multiple of four words), applied by the MFMA.
+int launch_fp8_dma3_ue8m0(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);
 
 // Grouped problems on the tile bodies of the dense kernels: token rows of all experts stacked in one matrix, one weight
 // matrix per expert.  `g` describes expert 0 (a, out, b, sb, and sa = the re-laid-out token scales: M-major, every

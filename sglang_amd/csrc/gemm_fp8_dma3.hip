@@ -65,7 +65,7 @@ struct Dma3State {
 // Load number i (< LOADS: tile rows; == LOADS: token scales) of K block kb, written as instructions.
 // The statements write m0; it cannot be listed as a clobber (the compiler reserves the register and rejects the entry), and
 // no compiler-managed use of m0 lies between them and the next statement that sets it.
-template <int BM, int BN>
+template <int BM, int BN, bool UE8M0 = false>
 __device__ __forceinline__ void issue_one(const Dma3State<BM, BN>& s, int i, uint8_t* stage, float* scale, int kb) {
   constexpr int LOADS = Dma3State<BM, BN>::LOADS;
   kb = min(kb, s.kb_last);
@@ -77,7 +77,9 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM, BN>& s, int i, uin
   } else {
     // the wave's BM / 8 token scales: BM / 32 lanes fetch 16 bytes each (a 4-byte-per-lane load in this stream costs far
     // more than its size: measured 1.5x on the whole large-M kernel).  exec is narrowed and restored inside the statement.
-    const float* sbase = s.sa_base + (int64_t)kb * s.sa_sk;  // wave-uniform
+    // fp32 scales: one row of floats per K block; packed exponents: one row of 32-bit words per four K blocks, fetched
+    // again for each of the four (the load count per K block stays constant)
+    const float* sbase = s.sa_base + (int64_t)(UE8M0 ? kb >> 2 : kb) * s.sa_sk;  // wave-uniform
     asm volatile("" : "+s"(sbase));
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(scale + s.wave * (BM / 8));
     uint64_t saved;
@@ -91,10 +93,12 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM, BN>& s, int i, uin
 }
 
 // One K block out of `cur`; the loads of block kb_next go out over the first LOADS + 1 steps into `nxt`.
-template <int BM, int BN>
+// UE8M0: the scale stage holds the tokens' packed exponent words and sbv the weight blocks' (as bits); the byte of block
+// `kb` goes to the MFMA, which applies both scales and accumulates in place: no promotion FMAs.
+template <int BM, int BN, bool UE8M0 = false>
 __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_t* cur, const float* sc_cur,
                                         const float (&sbv)[Dma3State<BM, BN>::SB], float (&acc)[BN / 64][BM / 32][4], uint8_t* nxt,
-                                        float* sc_nxt, int kb_next) {
+                                        float* sc_nxt, int kb_next, int kb = 0) {
   constexpr int MT = BM / 32, T_NT = BN / 64, LOADS = Dma3State<BM, BN>::LOADS;  // a wave owns BN / 4 channels = T_NT tiles of 16
   constexpr int SB = Dma3State<BM, BN>::SB, W_STRIDE = Dma3State<BM, BN>::W_STRIDE;
   static_assert(LOADS + 1 <= MT * T_NT, "one load per step");
@@ -107,18 +111,35 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
   tokb[0].lo = lds16(tk0, 0);
   tokb[0].hi = lds16(tk1, 0);
   const float* scp = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(sc_cur) + s.sc_off);
+  const int shift = (kb & 3) * 8;
+  int w_exp[SB];  // UE8M0: the weight blocks' exponent bytes of this K block, in byte 0
 #pragma unroll
-  for (int b = 0; b < SB; ++b) scb[0][b] = scp[0] * sbv[b];
+  for (int b = 0; b < SB; ++b) {
+    if constexpr (UE8M0) {
+      w_exp[b] = (int)(__float_as_uint(sbv[b]) >> shift);
+      scb[0][b] = __uint_as_float(__float_as_uint(scp[0]) >> shift);
+    } else {
+      w_exp[b] = 0;
+      scb[0][b] = scp[0] * sbv[b];
+    }
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   v4f part[2];
 #pragma unroll
   for (int t = 0; t < MT * T_NT; ++t) {
     const int j = t / T_NT, i = t % T_NT;
-    part[t & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w[i]), as_v8i(tokb[j & 1]),
-                                                                   v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+    if constexpr (UE8M0) {
+      float* a = acc[i][j];
+      const v4f r = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w[i]), as_v8i(tokb[j & 1]), v4f{a[0], a[1], a[2], a[3]}, 0, 0, 0,
+                                                                     w_exp[SB > 1 ? i : 0], 0, (int)__float_as_uint(scb[j & 1][0]));
+      a[0] = r[0], a[1] = r[1], a[2] = r[2], a[3] = r[3];
+    } else {
+      part[t & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w[i]), as_v8i(tokb[j & 1]),
+                                                                     v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+    }
     __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first; the rest of the step runs in its shadow
-    if (t > 0) {
+    if (!UE8M0 && t > 0) {
       const int pj = (t - 1) / T_NT, pi = (t - 1) % T_NT;
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[pi][pj][v] = fmaf(part[(t - 1) & 1][v], scb[pj & 1][SB > 1 ? pi : 0], acc[pi][pj][v]);
@@ -133,12 +154,15 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
     }
     if (i == 1 && j + 1 < MT) {
 #pragma unroll
-      for (int b = 0; b < SB; ++b) scb[(j + 1) & 1][b] = scp[(j + 1) * 16] * sbv[b];
+      for (int b = 0; b < SB; ++b) {
+        if constexpr (UE8M0) scb[(j + 1) & 1][b] = __uint_as_float(__float_as_uint(scp[(j + 1) * 16]) >> shift);
+        else scb[(j + 1) & 1][b] = scp[(j + 1) * 16] * sbv[b];
+      }
     }
-    if (t <= LOADS) issue_one<BM, BN>(s, t, nxt, sc_nxt, kb_next);
+    if (t <= LOADS) issue_one<BM, BN, UE8M0>(s, t, nxt, sc_nxt, kb_next);
     __builtin_amdgcn_sched_barrier(0);
   }
-  {
+  if constexpr (!UE8M0) {
     constexpr int t = MT * T_NT - 1;
     constexpr int pj = t / T_NT, pi = t % T_NT;
 #pragma unroll
@@ -157,7 +181,9 @@ __device__ __forceinline__ void wait_and_barrier() {
 }
 
 // One BM x 256 output tile at (m0, n0), K blocks of split `split`, by the whole workgroup.
-template <int BM, bool SPLIT, int BN = T_BN>
+// UE8M0: p.sa / p.sb point to packed exponent words (int32): token word (m, kw) at sa[kw * sa_sk + m], channel word (n, kw)
+// at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb; the MFMA applies them.
+template <int BM, bool SPLIT, int BN = T_BN, bool UE8M0 = false>
 __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, int split) {
   static_assert(BN == 128 || BN == 192 || BN == 256, "channel tile");
   constexpr int WM = BM / 2, MT = WM / 16, T_WN = BN / 4, T_NT = T_WN / 16, LOADS = Dma3State<BM, BN>::LOADS;
@@ -204,7 +230,7 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
 #pragma unroll
   for (int b = 0; b < SB; ++b) {
     const int first = INTERLEAVED ? n0 + 64 * b : n0 + wave_n * T_WN;  // first channel of the wave's tile(s) with this scale
-    s.sb_ptr[b] = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(first, p.N - 1) / 128) * p.sb_sn);
+    s.sb_ptr[b] = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(UE8M0 ? min(first, p.N - 1) : min(first, p.N - 1) / 128) * p.sb_sn);
   }
   s.sb_sk = p.sb_sk;
 
@@ -227,15 +253,15 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
 
   // ---- prologue: blocks 0 and 1 (clamped) into stages 0 and 1
 #pragma unroll
-  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN>(s, i, t_stage0, t_scale0, kb_begin);
+  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN, UE8M0>(s, i, t_stage0, t_scale0, kb_begin);
 #pragma unroll
-  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN>(s, i, t_stage1, t_scale1, kb_begin + 1);
+  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN, UE8M0>(s, i, t_stage1, t_scale1, kb_begin + 1);
   wait_and_barrier<LOADS + 1>();  // block 0 has landed everywhere
 
   // ---- three blocks per trip over the three stages; iteration k multiplies block k, requests block k + 2
   auto sb_of = [&](int kb, float (&v)[SB]) {
 #pragma unroll
-    for (int b = 0; b < SB; ++b) v[b] = s.sb_ptr[b][(int64_t)kb * s.sb_sk];
+    for (int b = 0; b < SB; ++b) v[b] = s.sb_ptr[b][(int64_t)(UE8M0 ? kb >> 2 : kb) * s.sb_sk];
   };
   int k = 0;
   for (; k + 2 < nkb; k += 3) {
@@ -243,22 +269,22 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
     sb_of(kb_begin + k, sb0);
     sb_of(kb_begin + k + 1, sb1);
     sb_of(kb_begin + k + 2, sb2);
-    k_block<BM, BN>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2);
+    k_block<BM, BN, UE8M0>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2, kb_begin + k);
     wait_and_barrier<LOADS + 1>();
-    k_block<BM, BN>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3);
+    k_block<BM, BN, UE8M0>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3, kb_begin + k + 1);
     wait_and_barrier<LOADS + 1>();
-    k_block<BM, BN>(s, t_stage2, t_scale2, sb2, acc, t_stage1, t_scale1, kb_begin + k + 4);
+    k_block<BM, BN, UE8M0>(s, t_stage2, t_scale2, sb2, acc, t_stage1, t_scale1, kb_begin + k + 4, kb_begin + k + 2);
     wait_and_barrier<LOADS + 1>();
   }
   if (k < nkb) {  // one or two blocks left, in stages 0 and 1
     float sb0[SB];
     sb_of(kb_begin + k, sb0);
-    k_block<BM, BN>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2);
+    k_block<BM, BN, UE8M0>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2, kb_begin + k);
     wait_and_barrier<LOADS + 1>();
     if (k + 1 < nkb) {
       float sb1[SB];
       sb_of(kb_begin + k + 1, sb1);
-      k_block<BM, BN>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3);
+      k_block<BM, BN, UE8M0>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3, kb_begin + k + 1);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
@@ -287,10 +313,10 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   }
 }
 
-template <int BM, bool SPLIT, int BN>
+template <int BM, bool SPLIT, int BN, bool UE8M0 = false>
 __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmParams p) {
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
-  dma3_tile<BM, SPLIT, BN>(p, tc.tile_m * BM, tc.tile_n * BN, tc.split);
+  dma3_tile<BM, SPLIT, BN, UE8M0>(p, tc.tile_m * BM, tc.tile_n * BN, tc.split);
 }
 
 // Grouped problems (see GroupedParams): the workgroup's token tile comes from the table the plan kernel wrote, the
@@ -303,15 +329,15 @@ __global__ __launch_bounds__(T_THREADS) void fp8_grouped_dma3_kernel(const Group
   dma3_tile<BM, false>(p, m0, tile_n * T_BN, 0);
 }
 
-template <int BM, int BN>
+template <int BM, int BN, bool UE8M0 = false>
 int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits));
   if (p.splits > 1)
-    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN>), grid, dim3(T_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
   else
-    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN>), grid, dim3(T_THREADS), 0, stream, p);
+    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
   return check_launch(what);
 }
 
@@ -418,6 +444,13 @@ int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const cha
   if (bn == 128) return bm == 64 ? launch_bm<64, 128>(p, stream, what) : launch_bm<128, 128>(p, stream, what);
   if (bn == 192) return bm == 64 ? launch_bm<64, 192>(p, stream, what) : launch_bm<128, 192>(p, stream, what);
   return bm == 64 ? launch_bm<64, 256>(p, stream, what) : launch_bm<128, 256>(p, stream, what);
+}
+
+// The same kernels for packed power-of-two (UE8M0) scales on both operands, applied by the MFMA (see dma3_tile).
+int launch_fp8_dma3_ue8m0(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what) {
+  if (bn == 128) return bm == 64 ? launch_bm<64, 128, true>(p, stream, what) : launch_bm<128, 128, true>(p, stream, what);
+  if (bn == 192) return bm == 64 ? launch_bm<64, 192, true>(p, stream, what) : launch_bm<128, 192, true>(p, stream, what);
+  return bm == 64 ? launch_bm<64, 256, true>(p, stream, what) : launch_bm<128, 256, true>(p, stream, what);
 }
 
 }  // namespace mi355

@@ -537,7 +537,7 @@ bool route_wants_m_major_scales(bool is_fp8, const Route& r) {
 // partial sums (after it).
 size_t route_workspace_need(bool is_fp8, const Route& r, const GemmParams& p) {
   size_t need = r.splits > 1 ? (size_t)r.splits * (size_t)p.M * (size_t)p.N * 4u : 0;
-  if (route_wants_m_major_scales(is_fp8, r) && !fp8_scales_conform(p)) need += scale_relayout_bytes(p.M, p.K);
+  if (!p.ue8m0 && route_wants_m_major_scales(is_fp8, r) && !fp8_scales_conform(p)) need += scale_relayout_bytes(p.M, p.K);
   return need;
 }
 
@@ -561,7 +561,7 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
                   "%s: workspace must be 16-byte aligned", what);
     p.ws = workspace;
   }
-  if (route_wants_m_major_scales(IS_FP8, r) && !fp8_scales_conform(p)) {
+  if (!p.ue8m0 && route_wants_m_major_scales(IS_FP8, r) && !fp8_scales_conform(p)) {
     float* dst = static_cast<float*>(workspace);
     const int64_t ld = (p.M + 3) & ~3;
     hipLaunchKernelGGL(relayout_scales_kernel, dim3((unsigned)((p.M + 31) / 32), (unsigned)((p.kb_total + 31) / 32)), dim3(256), 0,
@@ -586,7 +586,8 @@ int run_gemm(GemmParams& p, void* workspace, size_t workspace_bytes_given, hipSt
       }
       break;
     case RK_DMA3:
-      rc = IS_FP8 ? launch_fp8_dma3(p, r.bm, r.bn, stream, what) : launch_int8_dma3(p, r.bm, r.bn, stream, what);
+      if constexpr (IS_FP8) rc = p.ue8m0 ? launch_fp8_dma3_ue8m0(p, r.bm, r.bn, stream, what) : launch_fp8_dma3(p, r.bm, r.bn, stream, what);
+      else rc = launch_int8_dma3(p, r.bm, r.bn, stream, what);
       break;
     case RK_PINGPONG: return IS_FP8 ? launch_fp8_pp(p, stream, what) : launch_int8_pp(p, stream, what);
     case RK_PIPELINED: return launch_fp8_pipelined(p, stream, what);
@@ -834,6 +835,11 @@ extern "C" int mi355_fp8_blockwise_mm_ue8m0(const void* a, const void* b, const 
   if (r.kernel == RK_WAVESPLIT && K % KSTEP == 0) {
     // decode sizes on the wave-split kernel: the same, one launch, no workspace
     return launch_fp8_wavesplit_ue8m0(p, st, what);
+  }
+  if (r.kernel == RK_DMA3 && K % KSTEP == 0 && words_conform) {
+    // mid-M: the three-stage kernel with the exponents applied by the MFMA; the workspace only holds split-K partial sums
+    p.ue8m0 = 1;
+    return run_gemm<true>(p, workspace, workspace_bytes_given, st, what);
   }
   // every other shape: exponents to fp32 scales in the head of the workspace (tokens M-major, weights one row per
   // 128-channel block, read from the block's first channel), then the fp32-scale kernels

@@ -5,8 +5,8 @@ python/sglang/srt/layers/quantization/fp8_kernel.py:1047-1065, fp8_utils.py:217-
 The oracle is the blockwise GEMM oracle fed with the decoded scales 2^(byte - 127).  Floating point:
 |out - ref| <= 1e-2 * |ref| + 1e-4 * mag, as for the fp32-scale GEMM (tests/test_gpu_fp8_gemm.py); with small-integer
 operands every product and partial sum is exact in fp32 and the result must match bit for bit, whichever kernel runs.
-Large shapes and decode shapes on the wave-split kernel take kernels whose MFMA applies the scales itself, the others the
-fp32-scale kernels behind an unpack step; all are covered, and so are K extents whose last exponent word is only partly used."""
+Large shapes, mid-M shapes (every tile and split of the three-stage kernel) and decode shapes on the wave-split kernel
+take kernels whose MFMA applies the scales itself, the others the fp32-scale kernels behind an unpack step; all are covered, and so are K extents whose last exponent word is only partly used."""
 import pytest
 import torch
 
@@ -93,6 +93,63 @@ def test_ue8m0_gemm_exact_integers(gpu, oracle, M, N, K):
     sa_buf, sb_buf = pack(ea, M, 1).to(gpu), pack(eb, N, 128).to(gpu)
     sa_words, sb_words = sa_buf.t()[:M], sb_buf.t()[:N]
     out = ops.fp8_blockwise_mm_ue8m0(a.to(gpu), w.to(gpu), sa_words, sb_words, torch.bfloat16)
+    ref = oracle.fp8_blockwise_mm(a, w, torch.exp2(ea.float() - 127), torch.exp2(eb.float() - 127), torch.bfloat16)
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+# one shape per tile (64 / 128 tokens x 128 / 192 / 256 channels) and split of the mid-M kernel, which applies the exponents
+# in the MFMA too; 50 x 3000 has a ragged last channel tile, 33 x 16384 x 2176 a last exponent word with one byte used
+MID_M = [(48, 16384, 2048), (33, 16384, 2176), (40, 4096, 7168), (50, 3000, 4224), (24, 36864, 14336), (130, 3072, 7168), (40, 65536, 512),
+         (130, 4096, 7168), (100, 32768, 640), (65, 7168, 18432), (100, 36864, 640), (300, 3072, 14336), (100, 65536, 512),
+         (400, 4096, 16384)]
+
+
+def test_mid_m_shapes_reach_every_tile_and_split():
+    from sglang_amd import _lib
+
+    reached = set()
+    for M, N, K in MID_M:
+        p = _lib.gemm_plan("fp8", M, N, K)
+        assert p["kernel"] == "dma3", (M, N, K, p)
+        reached.add((p["bm"], p["bn"], p["splits"] > 1))
+    assert reached == {(bm, bn, sp) for bm in (64, 128) for bn in (128, 192, 256) for sp in (False, True)}
+
+
+@pytest.mark.parametrize("M,N,K", MID_M)
+def test_ue8m0_mid_m_kernel_against_oracle(gpu, oracle, M, N, K):
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul_deepgemm
+
+    x_q, sa_words, w2, sb_words = _operands(M, N, K, gpu, M + 7 * N + K)
+    out = w8a8_block_fp8_matmul_deepgemm(x_q, w2, sa_words, sb_words, [128, 128], torch.bfloat16)
+    rows = torch.arange(M) if M <= 64 else torch.cat([torch.tensor([0, 63, 64, min(127, M - 1), M - 1]),
+                                                       torch.randperm(M, generator=torch.Generator().manual_seed(M))[:27]])
+    ref, mag = _reference(oracle, x_q, sa_words, w2, sb_words, rows)
+    check_fp8_gemm(out[rows.to(gpu)], ref, mag, f"M={M} N={N} K={K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(130, 3072, 7168), (65, 7168, 18432), (100, 36864, 640)])
+def test_ue8m0_mid_m_exact_integers(gpu, oracle, M, N, K):
+    """Small-integer operands and exponents in a narrow band through the split and unsplit mid-M plans: exact in fp32, so the
+    MFMA-applied scales, the fp32 partial sums and their ordered reduce must reproduce the oracle's bits."""
+    from sglang_amd import ops
+
+    g = torch.Generator().manual_seed(K + M)
+    a = torch.randint(-2, 3, (M, K), generator=g).float().to(FP8)
+    w = torch.randint(-2, 3, (N, K), generator=g).float().to(FP8)
+    KB, KW = K // 128, (K // 128 + 3) // 4
+    ea = torch.randint(124, 129, (M, KB), generator=g, dtype=torch.uint8)
+    eb = torch.randint(124, 129, ((N + 127) // 128, KB), generator=g, dtype=torch.uint8)
+
+    def pack(e, rows_out, repeat):
+        full = torch.zeros(e.shape[0], KW * 4, dtype=torch.uint8)
+        full[:, :KB] = e
+        words = full.view(torch.int32).repeat_interleave(repeat, 0)[:rows_out]
+        buf = torch.zeros(KW, (rows_out + 3) // 4 * 4, dtype=torch.int32)
+        buf[:, :rows_out] = words.t()
+        return buf
+
+    sa_buf, sb_buf = pack(ea, M, 1).to(gpu), pack(eb, N, 128).to(gpu)
+    out = ops.fp8_blockwise_mm_ue8m0(a.to(gpu), w.to(gpu), sa_buf.t()[:M], sb_buf.t()[:N], torch.bfloat16)
     ref = oracle.fp8_blockwise_mm(a, w, torch.exp2(ea.float() - 127), torch.exp2(eb.float() - 127), torch.bfloat16)
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
 
