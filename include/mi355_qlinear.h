@@ -160,10 +160,11 @@ int mi355_fp8_blockwise_scaled_grouped_mm(const void* a, const void* b, const fl
  *             block is read, which one depends on the kernel
  *   bias      NULL or [N] in the output dtype, added in the epilogue
  * On gfx950 the matrix instruction applies such scales itself (v_mfma_scale_f32_16x16x128_f8f6f4), so for large M, for
- * the mid-M shapes on the three-stage kernel and for the decode sizes (M <= 16) that take the wave-split kernel the K
- * loop carries no scale arithmetic at all and nothing runs in front of the GEMM (K % 128 == 0 and, above decode sizes,
- * token words with a 16-byte aligned base and a pitch that is a multiple of four words); other shapes expand the
- * exponents to fp32 scales in the workspace and take the kernels of mi355_fp8_blockwise_mm.  Replaces w8a8_block_fp8_matmul_deepgemm / deep_gemm gemm_nt_f8f8bf16
+ * the mid-M shapes on the three-stage kernel and for the decode sizes (M <= 16, both decode kernels) the K loop carries
+ * no scale arithmetic at all and nothing runs in front of the GEMM (K % 128 == 0 and, above decode sizes, token words
+ * with a 16-byte aligned base and a pitch that is a multiple of four words); other shapes (ragged K, the generic and
+ * the two-stage kernels' shapes) expand the exponents to fp32 scales in the workspace and take the kernels of
+ * mi355_fp8_blockwise_mm.  Replaces w8a8_block_fp8_matmul_deepgemm / deep_gemm gemm_nt_f8f8bf16
  * (python/sglang/srt/layers/quantization/fp8_kernel.py:1047-1065; caller deepgemm_w8a8_block_fp8_linear_with_fallback,
  * fp8_utils.py:217-255), whose kernel lives in the DeepGEMM package, not in the reference tree.
  */

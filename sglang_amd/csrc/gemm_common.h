@@ -43,6 +43,15 @@ struct GemmParams {
 };
 
 // ---------------------------------------------------------------------------------------------
+// Puts a wave-uniform value into a vector register HERE.  The MFMA takes its scale operands from vector registers and reads
+// all 64 lanes whatever EXEC says; the compiler, which knows neither, may sink an MFMA whose result only a guarded store
+// uses into that store's divergent region together with the scalar-to-vector copy of its scale, and the copy then skips
+// the inactive lanes (rows of the operand that the active lanes' results still depend on).  Call it where every lane is active.
+__device__ __forceinline__ int in_vgpr(int x) {
+  asm volatile("" : "+v"(x));
+  return x;
+}
+
 __device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off, const float* r, int nvalid,
                                            bool vec_ok) {
   if (out_dtype == MI355_F32) {

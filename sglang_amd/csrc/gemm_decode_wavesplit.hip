@@ -79,7 +79,7 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
       const bool valid = kb < p.kb_total;
       if constexpr (UE8M0) {
         const int shift = 8 * (min(kb, p.kb_total - 1) & 3);
-        const int ea = (int)((__float_as_uint(sbv[j]) >> shift) & 0xffu), eb = (int)((__float_as_uint(sav[j]) >> shift) & 0xffu);
+        const int ea = in_vgpr((int)((__float_as_uint(sbv[j]) >> shift) & 0xffu)), eb = (int)((__float_as_uint(sav[j]) >> shift) & 0xffu);
         const u32x4 z = {0u, 0u, 0u, 0u};
         Frag t = tf[j];
         if (!valid) t.lo = z, t.hi = z;  // a block past the end of K multiplies zeros

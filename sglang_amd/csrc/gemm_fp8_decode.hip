@@ -23,6 +23,11 @@
 // fixed order.  (INT8 shapes with more than one K range all take the wave-split kernel of gemm_decode_wavesplit.hip, which
 // was measured faster for them at every decode size; the INT8 split variant of this kernel is therefore not built.)  INT8 uses two
 // v_mfma_i32_16x16x64_i8 per K block (chunk q of both operands, then chunk q + 4) and has no scales in the loop.
+// Packed UE8M0 scales on both operands (GemmParams.ue8m0): the token's exponent words of the range sit in registers, the
+// weight blocks' come by scalar loads, and v_mfma_scale_f32_16x16x128_f8f6f4 applies the byte of each and accumulates in
+// place, so the loop has no scale arithmetic.  The compiler sinks the last tile's MFMAs of a group into the group's guarded
+// stores (only lanes of valid tokens are active there, but an MFMA reads all 64): their scale operands are therefore put
+// into vector registers at the top of the group (in_vgpr).
 // Requires K % 128 == 0, N % 128 == 0 and 16-byte aligned rows; other shapes take the generic kernel.
 #include "gemm_common.h"
 
@@ -106,8 +111,11 @@ __device__ __forceinline__ void wait_ring() {
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-template <bool IS_FP8, typename AccT>
-__device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* stage, int d, float scale, AccT (&acc)[NT][4]) {
+// UE8M0 (FP8 only): `scale` and `w_scale` carry, as bits, the token's and the weight block's exponent byte of this K block in
+// byte 0; the MFMA applies both and accumulates in place.
+template <bool IS_FP8, bool UE8M0 = false, typename AccT>
+__device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* stage, int d, float scale, AccT (&acc)[NT][4],
+                                        float w_scale = 0.f) {
   const uint8_t* sl = stage + s.wave * SLICE;
   Frag t;
   t.lo = *reinterpret_cast<const u32x4*>(r_tok + d * TOK_BLOCK + s.tk_off[0]);
@@ -117,7 +125,12 @@ __device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* sta
     Frag w;
     w.lo = *reinterpret_cast<const u32x4*>(sl + s.rd_off[i][0]);
     w.hi = *reinterpret_cast<const u32x4*>(sl + s.rd_off[i][1]);
-    if constexpr (IS_FP8) {
+    if constexpr (UE8M0) {
+      const v4f r = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w), as_v8i(t), v4f{acc[i][0], acc[i][1], acc[i][2], acc[i][3]}, 0,
+                                                                     0, 0, (int)__float_as_uint(w_scale), 0, (int)__float_as_uint(scale));
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][v] = r[v];
+    } else if constexpr (IS_FP8) {
       const v4f part =
           __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(w), as_v8i(t), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
 #pragma unroll
@@ -205,9 +218,12 @@ __device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begi
 }
 
 // SPLIT: raw partial sums to the workspace (more than one K range).
-template <bool IS_FP8, bool SPLIT, bool QUANT = false>
+// UE8M0 (FP8 only): p.sa / p.sb point to packed exponent words (token word (m, kw) at sa[kw * sa_sk + m], channel word (n, kw)
+// at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb) and the MFMA applies them.
+template <bool IS_FP8, bool SPLIT, bool QUANT = false, bool UE8M0 = false>
 __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, int groups_per_wg, int wg_per_split) {
   static_assert(IS_FP8 || !QUANT, "the fused quantizer belongs to the FP8 path");
+  static_assert((IS_FP8 && !QUANT) || !UE8M0, "exponent scales come with already quantized FP8 tokens");
   using AccT = typename std::conditional<IS_FP8, float, int>::type;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -271,8 +287,13 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
     const float* sa_row = p.sa + (int64_t)min(l16, p.M - 1) * p.sa_sm;
 #pragma unroll
     for (int d = 0; d < KB_PER; ++d) {
-      const float v = sa_row[(int64_t)min(kb_begin + d, p.kb_total - 1) * p.sa_sk];
-      sa_r[d] = d < kb_valid ? v : 0.f;
+      const int kbc = min(kb_begin + d, p.kb_total - 1);
+      if constexpr (UE8M0) {  // the block's byte of the token's word, in byte 0 (blocks past K multiply zero tokens)
+        sa_r[d] = __uint_as_float(__float_as_uint(sa_row[(int64_t)(kbc >> 2) * p.sa_sk]) >> ((kbc & 3) * 8));
+      } else {
+        const float v = sa_row[(int64_t)kbc * p.sa_sk];
+        sa_r[d] = d < kb_valid ? v : 0.f;
+      }
     }
   } else {
 #pragma unroll
@@ -285,7 +306,15 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
   // has to wait for loads younger than the ring's
   float sb_cur[KB_PER], sb_nxt[KB_PER];
   auto load_sb = [&](int g, float (&dst)[KB_PER]) {
-    if constexpr (IS_FP8) {
+    if constexpr (UE8M0) {
+      // one word row per weight ROW (constant over the 128-channel group): the group's first row; scalar loads
+      const cfloat_ptr sb_row = (cfloat_ptr)(p.sb + (int64_t)(g_first + min(g, groups - 1)) * GROUP_N * p.sb_sn);
+#pragma unroll
+      for (int d = 0; d < KB_PER; ++d) {
+        const int kbc = kb_begin + min(d, kb_valid - 1);
+        dst[d] = __uint_as_float(__float_as_uint(sb_row[(int64_t)(kbc >> 2) * p.sb_sk]) >> ((kbc & 3) * 8));
+      }
+    } else if constexpr (IS_FP8) {
       // uniform addresses through a constant-address-space pointer: scalar loads, which do not count in vmcnt, so the
       // copy of these values at the end of a group never waits for the weight ring
       const cfloat_ptr sb_row =
@@ -301,9 +330,13 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
   for (int g = 0; g < groups; ++g) {
     const int nb = g_first + g;  // 128 channels = one weight scale block
     load_sb(g + 1, sb_nxt);
-    float sc[KB_PER];
+    float sc[KB_PER], wsc[KB_PER];  // fp32 scales: sc = token scale x block scale; UE8M0: the two exponent bytes apart
 #pragma unroll
-    for (int d = 0; d < KB_PER; ++d) sc[d] = sa_r[d] * sb_cur[d];
+    for (int d = 0; d < KB_PER; ++d) {
+      sc[d] = UE8M0 ? sa_r[d] : sa_r[d] * sb_cur[d];
+      // UE8M0: in a vector register before the group's guarded stores (the last MFMAs may be sunk into them)
+      wsc[d] = UE8M0 ? __uint_as_float((uint32_t)in_vgpr((int)__float_as_uint(sb_cur[d]))) : 0.f;
+    }
 #pragma unroll
     for (int d = 0; d < KB_PER; ++d) sb_cur[d] = sb_nxt[d];
     AccT acc[NT][4];
@@ -319,19 +352,19 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
       // that is due (the two requested after it may still be in flight), multiply it
       issue_weights<true>(s, r_stage3, f0 + d + 3);
       wait_ring<2>();
-      consume<IS_FP8>(s, r_stage0, d + 0, sc[d + 0], acc);
+      consume<IS_FP8, UE8M0>(s, r_stage0, d + 0, sc[d + 0], acc, wsc[d + 0]);
       __builtin_amdgcn_sched_barrier(0);
       issue_weights<true>(s, r_stage0, f0 + d + 4);
       wait_ring<2>();
-      consume<IS_FP8>(s, r_stage1, d + 1, sc[d + 1], acc);
+      consume<IS_FP8, UE8M0>(s, r_stage1, d + 1, sc[d + 1], acc, wsc[d + 1]);
       __builtin_amdgcn_sched_barrier(0);
       issue_weights<true>(s, r_stage1, f0 + d + 5);
       wait_ring<2>();
-      consume<IS_FP8>(s, r_stage2, d + 2, sc[d + 2], acc);
+      consume<IS_FP8, UE8M0>(s, r_stage2, d + 2, sc[d + 2], acc, wsc[d + 2]);
       __builtin_amdgcn_sched_barrier(0);
       issue_weights<true>(s, r_stage2, f0 + d + 6);
       wait_ring<2>();
-      consume<IS_FP8>(s, r_stage3, d + 3, sc[d + 3], acc);
+      consume<IS_FP8, UE8M0>(s, r_stage3, d + 3, sc[d + 3], acc, wsc[d + 3]);
       __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -421,7 +454,21 @@ static int launch_decode(GemmParams& p, int gpw, hipStream_t stream, const char*
   return check_launch(what);
 }
 
-int launch_fp8_decode(GemmParams& p, int gpw, hipStream_t stream, const char* what) { return launch_decode<true>(p, gpw, stream, what); }
+int launch_fp8_decode(GemmParams& p, int gpw, hipStream_t stream, const char* what) {
+  if (p.ue8m0) {  // packed exponent words on both operands, applied by the MFMA
+    const int groups_n = p.N / GROUP_N;
+    const int wg_per_split = (groups_n + gpw - 1) / gpw;
+    p.tiles_m = 1;
+    p.tiles_n = groups_n;
+    const dim3 grid((unsigned)(wg_per_split * p.splits));
+    if (p.splits > 1)
+      hipLaunchKernelGGL((decode_kernel<true, true, false, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+    else
+      hipLaunchKernelGGL((decode_kernel<true, false, false, true>), grid, dim3(64 * WAVES), 0, stream, p, gpw, wg_per_split);
+    return check_launch(what);
+  }
+  return launch_decode<true>(p, gpw, stream, what);
+}
 int launch_int8_decode(GemmParams& p, int gpw, hipStream_t stream, const char* what) { return launch_decode<false>(p, gpw, stream, what); }
 
 }  // namespace mi355

@@ -116,7 +116,7 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
 #pragma unroll
   for (int b = 0; b < SB; ++b) {
     if constexpr (UE8M0) {
-      w_exp[b] = (int)(__float_as_uint(sbv[b]) >> shift);
+      w_exp[b] = in_vgpr((int)(__float_as_uint(sbv[b]) >> shift));
       scb[0][b] = __uint_as_float(__float_as_uint(scp[0]) >> shift);
     } else {
       w_exp[b] = 0;

@@ -371,7 +371,7 @@ __device__ __forceinline__ void pp_tile(const GemmParams& p, const int m0, const
   auto k_block = [&](uint8_t* cur, uint8_t* nxt, int kb, float sbv) {
     const float* sc_cur = g_scale + (kb & 3) * G_BM;
     // the weight block's exponent byte, in byte 0 of a register (for SM_UE8M0 sbv carries the packed word as bits)
-    const int w_scale = UE8M0 ? (int)(__float_as_uint(sbv) >> ((kb & 3) * 8)) : 127;
+    const int w_scale = UE8M0 ? in_vgpr((int)(__float_as_uint(sbv) >> ((kb & 3) * 8))) : 127;
     if constexpr (!HW_SCALE) retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
     read_operands<0, SM>(s, cur, sc_cur, sbv, kb, w, tok, scb);
     if constexpr (!NOLOAD) issue_set_b<KFULL>(s, nxt, kb + 1);

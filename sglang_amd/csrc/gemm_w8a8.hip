@@ -836,8 +836,9 @@ extern "C" int mi355_fp8_blockwise_mm_ue8m0(const void* a, const void* b, const 
     // decode sizes on the wave-split kernel: the same, one launch, no workspace
     return launch_fp8_wavesplit_ue8m0(p, st, what);
   }
-  if (r.kernel == RK_DMA3 && K % KSTEP == 0 && words_conform) {
-    // mid-M: the three-stage kernel with the exponents applied by the MFMA; the workspace only holds split-K partial sums
+  if ((r.kernel == RK_DMA3 && K % KSTEP == 0 && words_conform) || r.kernel == RK_DECODE) {
+    // mid-M and streaming decode: the same kernels with the exponents applied by the MFMA; the workspace only holds
+    // split-K partial sums (the decode kernel reads the words with ordinary loads: any pitch will do)
     p.ue8m0 = 1;
     return run_gemm<true>(p, workspace, workspace_bytes_given, st, what);
   }

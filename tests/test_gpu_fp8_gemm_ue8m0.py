@@ -127,10 +127,34 @@ def test_ue8m0_mid_m_kernel_against_oracle(gpu, oracle, M, N, K):
     check_fp8_gemm(out[rows.to(gpu)], ref, mag, f"M={M} N={N} K={K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(130, 3072, 7168), (65, 7168, 18432), (100, 36864, 640)])
-def test_ue8m0_mid_m_exact_integers(gpu, oracle, M, N, K):
-    """Small-integer operands and exponents in a narrow band through the split and unsplit mid-M plans: exact in fp32, so the
-    MFMA-applied scales, the fp32 partial sums and their ordered reduce must reproduce the oracle's bits."""
+# the streaming decode kernel: one K range and several, the last range short (K blocks not a multiple of 8), one to four
+# bytes used in the last exponent word, token counts below and at the 16 rows of the MFMA tile (rows past M repeat the last token)
+DECODE = [(8, 256, 512), (4, 4352, 512), (3, 7168, 36864), (16, 7168, 36864), (5, 18432, 7168), (12, 18432, 7168), (9, 3072, 1536),
+          (6, 36864, 1280), (11, 16384, 2304), (15, 65536, 640), (16, 65536, 1152), (13, 7168, 18432), (8, 4352, 128)]
+
+
+def test_decode_shapes_reach_the_streaming_kernel():
+    from sglang_amd import _lib
+
+    plans = [_lib.gemm_plan("fp8", M, N, K) for M, N, K in DECODE]
+    assert all(p["kernel"] == "decode" for p in plans), plans
+    assert {p["splits"] > 1 for p in plans} == {False, True}
+
+
+@pytest.mark.parametrize("M,N,K", DECODE)
+def test_ue8m0_decode_kernel_against_oracle(gpu, oracle, M, N, K):
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul_deepgemm
+
+    x_q, sa_words, w2, sb_words = _operands(M, N, K, gpu, 3 * M + N + 5 * K)
+    out = w8a8_block_fp8_matmul_deepgemm(x_q, w2, sa_words, sb_words, [128, 128], torch.bfloat16)
+    ref, mag = _reference(oracle, x_q, sa_words, w2, sb_words)
+    check_fp8_gemm(out, ref, mag, f"M={M} N={N} K={K}")
+
+
+def _exact_integer_case(gpu, oracle, M, N, K):
+    """Small-integer operands and exponents drawn anew for every token, weight block and K block from a narrow band: exact in
+    fp32, so the MFMA-applied scales (each byte of each word in its place), the fp32 partial sums and their ordered reduce
+    must reproduce the oracle's bits."""
     from sglang_amd import ops
 
     g = torch.Generator().manual_seed(K + M)
@@ -152,6 +176,19 @@ def test_ue8m0_mid_m_exact_integers(gpu, oracle, M, N, K):
     out = ops.fp8_blockwise_mm_ue8m0(a.to(gpu), w.to(gpu), sa_buf.t()[:M], sb_buf.t()[:N], torch.bfloat16)
     ref = oracle.fp8_blockwise_mm(a, w, torch.exp2(ea.float() - 127), torch.exp2(eb.float() - 127), torch.bfloat16)
     assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("M,N,K", [(130, 3072, 7168), (65, 7168, 18432), (100, 36864, 640)])
+def test_ue8m0_mid_m_exact_integers(gpu, oracle, M, N, K):
+    _exact_integer_case(gpu, oracle, M, N, K)  # split and unsplit mid-M plans
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 4352, 512), (5, 18432, 7168), (16, 2048, 7168), (11, 16384, 2304), (3, 7168, 36864)])
+def test_ue8m0_decode_exact_integers(gpu, oracle, M, N, K):
+    from sglang_amd import _lib
+
+    assert _lib.gemm_plan("fp8", M, N, K)["kernel"] == "decode"
+    _exact_integer_case(gpu, oracle, M, N, K)
 
 
 @pytest.mark.parametrize("M", [8, 4096])
