@@ -4,8 +4,8 @@
 // The loop structure is the one of gemm_fp8_dma3.hip: the direct-to-LDS loads of K step k+2 are issued while step k is
 // multiplied, the wait before the bare s_barrier that ends iteration k covers step k+1 only (s_waitcnt vmcnt(LOADS), the
 // loads per wave and iteration being a constant), loads, wait and barrier are written as instructions.  The arithmetic
-// is the one of gemm_int8_pp.hip: v_mfma_i32_32x32x32_i8, four per 32 x 32 tile and 128-byte K step, exact int32
-// accumulation, fragments of 32 rows x 2 K halves read with the (row >> 1) & 7 swizzle.  A wave owns (BM / 2) x (BN / 4)
+// is the one of gemm_int8_pp.hip: v_mfma_i32_16x16x64_i8, two per 16 x 16 tile and 128-byte K step (chunk q of both
+// operands' rows, then chunk q + 4), exact int32 accumulation, (row & 7) chunk swizzle.  A wave owns (BM / 2) x (BN / 4)
 // outputs; the 128-channel tiles fill the chip for layers with few channels (K=4096 -> N=6144 at 256 tokens: 17 against 24 us).
 // Optional split along K: int32 partials to the workspace, the ordered reduce applies the epilogue.
 // Requires K % 128 == 0, 16-byte aligned rows, row offsets below 4 GiB.
@@ -13,8 +13,6 @@
 
 namespace mi355 {
 namespace {
-
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int U_THREADS = 512;
 
@@ -34,7 +32,7 @@ struct U8State {
   const uint8_t* b_base;
   uint32_t goff[LOADS];
   int wave, kb_last;
-  uint32_t tok_off[4], ch_off[4];  // per K sub-step: this lane's 16 bytes in the first token / channel tile
+  uint32_t tok_off[2], ch_off[2];  // per K half: this lane's 16 bytes in the first token / channel tile
 };
 
 // Writes m0, which cannot be listed as a clobber (reserved register); no compiler-managed use of m0 lies in the K loop.
@@ -49,27 +47,27 @@ __device__ __forceinline__ void issue_one(const U8State<BM, BN>& s, int i, uint8
 
 // One 128-byte K step out of `cur`; the loads of step kb_next go out in between, into `nxt`.
 template <int BM, int BN>
-__device__ __forceinline__ void k_step(const U8State<BM, BN>& s, const uint8_t* cur, v16i (&acc)[BN / 128][BM / 64], uint8_t* nxt,
+__device__ __forceinline__ void k_step(const U8State<BM, BN>& s, const uint8_t* cur, v4i (&acc)[BN / 64][BM / 32], uint8_t* nxt,
                                        int kb_next) {
-  constexpr int MT = BM / 64, U_NT = BN / 128, LOADS = U8State<BM, BN>::LOADS;  // a wave owns BN / 4 channels = U_NT tiles of 32
-  v4i w[U_NT][4], t[MT][4];
+  constexpr int MT = BM / 32, U_NT = BN / 64, LOADS = U8State<BM, BN>::LOADS;  // a wave owns BN / 4 channels = U_NT tiles of 16
+  v4i w[U_NT][2], t[MT][2];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int h = 0; h < 2; ++h) {
 #pragma unroll
-    for (int i = 0; i < U_NT; ++i) w[i][k] = lds16((lds_cptr)cur + s.ch_off[k], i * 4096);
+    for (int i = 0; i < U_NT; ++i) w[i][h] = lds16((lds_cptr)cur + s.ch_off[h], i * 2048);
 #pragma unroll
-    for (int j = 0; j < MT; ++j) t[j][k] = lds16((lds_cptr)cur + s.tok_off[k], j * 4096);
+    for (int j = 0; j < MT; ++j) t[j][h] = lds16((lds_cptr)cur + s.tok_off[h], j * 2048);
   }
   int issued = 0;
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int h = 0; h < 2; ++h) {
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
 #pragma unroll
       for (int i = 0; i < U_NT; ++i)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[i][k], t[j][k], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[i][h], t[j][h], acc[i][j], 0, 0, 0);
       if (issued < LOADS) issue_one<BM, BN>(s, issued++, nxt, kb_next);
-      if (issued < LOADS && MT == 1) issue_one<BM, BN>(s, issued++, nxt, kb_next);  // 4 groups only: two loads per group
+      if (issued < LOADS && MT == 2) issue_one<BM, BN>(s, issued++, nxt, kb_next);  // 4 groups only: two loads per group
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -87,12 +85,12 @@ __device__ __forceinline__ void wait_and_barrier() {
 template <int BM, bool SPLIT, int BN>
 __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmParams p) {
   static_assert(BN == 128 || BN == 256, "channel tile");
-  constexpr int WM = BM / 2, MT = WM / 32, U_WN = BN / 4, U_NT = U_WN / 32, LOADS = U8State<BM, BN>::LOADS;
+  constexpr int WM = BM / 2, MT = WM / 16, U_WN = BN / 4, U_NT = U_WN / 16, LOADS = U8State<BM, BN>::LOADS;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave >> 2, wave_n = wave & 3;
-  const int l32 = lane & 31, kh = lane >> 5;
+  const int l16 = lane & 15, q = lane >> 4;
 
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
   const int m0 = tc.tile_m * BM, n0 = tc.tile_n * BN;
@@ -111,11 +109,10 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
   s.a_base = p.a;
   s.b_base = p.b;
   {
-    // lane l lands in row l / 8, physical chunk l % 8 of the 8 rows one load fills; rows start at multiples of 8, so
-    // (row >> 1) & 7 == (4 * wave + (l >> 4)) & 7 for every load of this wave
+    // lane l lands in row l / 8, physical chunk l % 8 of the 8 rows one load fills (rows start at multiples of 8); it
+    // fetches the logical chunk that belongs there under the (row & 7) swizzle
     const int lrow = lane >> 3;
-    const int key = (4 * wave + (lane >> 4)) & 7;
-    const int chunk_byte = ((lane & 7) ^ key) * 16;
+    const int chunk_byte = ((lane & 7) ^ lrow) * 16;
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int row = i * 64 + wave * 8 + lrow;
@@ -124,21 +121,19 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
       else
         s.goff[i] = (uint32_t)((int64_t)min(n0 + row - BM, p.N - 1) * p.ldb + chunk_byte);
     }
-    const int trow = wave_m * WM + l32, crow = BM + wave_n * U_WN + l32;
+    const int trow = wave_m * WM + l16, crow = BM + wave_n * U_WN + l16;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {  // K sub-step k takes the 16-byte chunk 2k + kh of the row
-      s.tok_off[k] = trow * KSTEP + (((2 * k + kh) ^ ((trow >> 1) & 7)) << 4);
-      s.ch_off[k] = crow * KSTEP + (((2 * k + kh) ^ ((crow >> 1) & 7)) << 4);
+    for (int h = 0; h < 2; ++h) {  // K half h takes the 16-byte chunk q + 4h of the row
+      s.tok_off[h] = trow * KSTEP + (((q + 4 * h) ^ (trow & 7)) << 4);
+      s.ch_off[h] = crow * KSTEP + (((q + 4 * h) ^ (crow & 7)) << 4);
     }
   }
 
-  v16i acc[U_NT][MT];
+  v4i acc[U_NT][MT];
 #pragma unroll
   for (int i = 0; i < U_NT; ++i)
 #pragma unroll
-    for (int j = 0; j < MT; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    for (int j = 0; j < MT; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
 #pragma unroll
   for (int i = 0; i < LOADS; ++i) issue_one<BM, BN>(s, i, u_stage0, kb_begin);
@@ -162,12 +157,12 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
 
-  // ---- epilogue: lane holds, for token m, channels n0 + 32 i + 8 g + 4 kh + (0..3), g = 0..3
+  // ---- epilogue: lane holds, for token m = 16 j + l16 of the wave's rows, channels 16 i + 4 q + (0..3) of its columns
   const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
   const bool raw = p.out_dtype == MI355_I32;
 #pragma unroll
   for (int j = 0; j < MT; ++j) {
-    const int m = m0 + wave_m * WM + j * 32 + l32;
+    const int m = m0 + wave_m * WM + j * 16 + l16;
     if (m >= p.M) continue;
     float sa_m = 1.f;
     if constexpr (!SPLIT) {
@@ -175,27 +170,26 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
     }
 #pragma unroll
     for (int i = 0; i < U_NT; ++i) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wave_n * U_WN + i * 32 + 8 * g + 4 * kh;
+      {
+        const int n = n0 + wave_n * U_WN + i * 16 + 4 * q;
         if (n >= p.N) continue;
         const int nvalid = min(4, p.N - n);
         if constexpr (SPLIT) {
           int* wsp = reinterpret_cast<int*>(p.ws) + ((int64_t)tc.split * p.M + m) * p.N + n;
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            if (v < nvalid) wsp[v] = acc[i][j][4 * g + v];
+            if (v < nvalid) wsp[v] = acc[i][j][v];
         } else if (raw) {
           int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            if (v < nvalid) o[v] = acc[i][j][4 * g + v];
+            if (v < nvalid) o[v] = acc[i][j][v];
         } else {
           float r[4];
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             const int nn = min(n + v, p.N - 1);
-            float t = mul_rn((float)acc[i][j][4 * g + v], mul_rn(p.sb[nn], sa_m));
+            float t = mul_rn((float)acc[i][j][v], mul_rn(p.sb[nn], sa_m));
             if (p.bias) {
               const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[nn];
               t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));

@@ -4,8 +4,8 @@
 // (the matrix pipe waits), then all of them multiply (LDS waits); a 128 x 256 tile takes 1.14 us per 128-byte K step where
 // the 256 x 256 two-phase kernel (gemm_int8_pp.hip) spends 0.73 us on the same amount of work.  This kernel gives the short
 // tile the two-phase schedule: waves 0..3 own token rows 0..63, waves 4..7 rows 64..127, each wave 64 channels
-// (2 x 2 tiles of 32 x 32); a group alternates a memory phase (the sixteen ds_read_b128 of its next K step, then its six
-// direct-to-LDS loads of the K step after next) with a compute phase (sixteen v_mfma_i32_32x32x32_i8 and nothing else),
+// (4 x 4 tiles of 16 x 16); a group alternates a memory phase (the sixteen ds_read_b128 of its next K step, then its six
+// direct-to-LDS loads of the K step after next) with a compute phase (32 v_mfma_i32_16x16x64_i8 and nothing else),
 // one workgroup barrier per phase, group 1 one phase behind - so while one group multiplies the other reads.
 // A K step is 2 phases (~0.7 us), too short for loads that come from HBM to land within one step, hence three stages of
 // 48 KB: the loads of step b + 2 go out in the memory phase of step b into the stage step b - 1 was read from (both groups
@@ -18,11 +18,9 @@
 namespace mi355 {
 namespace {
 
-typedef int v16i __attribute__((ext_vector_type(16)));
-
 constexpr int J_THREADS = 512;
 constexpr int J_BM = 128, J_BN = 256, J_WM = 64, J_WN = 64;
-constexpr int J_MT = J_WM / 32, J_NT = J_WN / 32;  // 2 token tiles x 2 channel tiles of 32 x 32 per wave
+constexpr int J_MT = J_WM / 16, J_NT = J_WN / 16;  // 4 token tiles x 4 channel tiles of 16 x 16 per wave
 constexpr int J_ROWS = J_BM + J_BN;
 constexpr int J_LOADS = J_ROWS / 64;  // 6 direct-to-LDS loads per wave and K step: 2 of token rows, 4 of channel rows
 constexpr int J_STAGE = J_ROWS * KSTEP;
@@ -47,7 +45,7 @@ struct JState {
   const uint8_t* b_base;
   uint32_t goff[J_LOADS];  // loads 0..1 token rows, 2..5 channel rows
   int wave, kb_last;
-  uint32_t tok_off[4], ch_off[4];  // per K sub-step: this lane's 16 bytes in the first token / channel tile
+  uint32_t tok_off[2], ch_off[2];  // per K half: this lane's 16 bytes in the first token / channel tile
 };
 
 // Direct-to-LDS load number i of K step kb (clamped to the last step): tile rows i * 64 + 8 * wave .. + 7 into `stage`.
@@ -81,24 +79,24 @@ __device__ __forceinline__ void memory_end() {
 }
 
 // Memory phase, operand part: the wave's weight and token fragments of the K step in `cur`.
-__device__ __forceinline__ void read_operands(const JState& s, const uint8_t* cur, v4i (&w)[J_NT][4], v4i (&t)[J_MT][4]) {
+__device__ __forceinline__ void read_operands(const JState& s, const uint8_t* cur, v4i (&w)[J_NT][2], v4i (&t)[J_MT][2]) {
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int h = 0; h < 2; ++h) {
 #pragma unroll
-    for (int i = 0; i < J_NT; ++i) w[i][k] = lds16((lds_cptr)cur + s.ch_off[k], i * 4096);
+    for (int i = 0; i < J_NT; ++i) w[i][h] = lds16((lds_cptr)cur + s.ch_off[h], i * 2048);
 #pragma unroll
-    for (int j = 0; j < J_MT; ++j) t[j][k] = lds16((lds_cptr)cur + s.tok_off[k], j * 4096);
+    for (int j = 0; j < J_MT; ++j) t[j][h] = lds16((lds_cptr)cur + s.tok_off[h], j * 2048);
   }
 }
 
-// Compute phase: 16 MFMAs; a tile's accumulator comes round every fourth one.
-__device__ __forceinline__ void compute(const v4i (&w)[J_NT][4], const v4i (&t)[J_MT][4], v16i (&acc)[J_NT][J_MT]) {
+// Compute phase: 32 MFMAs; a tile's accumulator comes round every sixteenth one.
+__device__ __forceinline__ void compute(const v4i (&w)[J_NT][2], const v4i (&t)[J_MT][2], v4i (&acc)[J_NT][J_MT]) {
 #pragma unroll
-  for (int k = 0; k < 4; ++k)
+  for (int h = 0; h < 2; ++h)
 #pragma unroll
     for (int j = 0; j < J_MT; ++j)
 #pragma unroll
-      for (int i = 0; i < J_NT; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[i][k], t[j][k], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < J_NT; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[i][h], t[j][h], acc[i][j], 0, 0, 0);
 }
 
 // 128-row output tile through LDS (rows of 512 bytes, chunks swizzled as out_tile_put4 writes them): every wave stores 16
@@ -122,7 +120,7 @@ __global__ __launch_bounds__(J_THREADS) void int8_gemm_pp128_kernel(const GemmPa
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave >> 2;  // 0: starts computing first; 1: one phase behind.  Also the wave's token half of the tile.
   const int wave_n = wave & 3;
-  const int l32 = lane & 31, kh = lane >> 5;
+  const int l16 = lane & 15, q = lane >> 4;
 
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
   const int m0 = tc.tile_m * J_BM, n0 = tc.tile_n * J_BN;
@@ -136,11 +134,10 @@ __global__ __launch_bounds__(J_THREADS) void int8_gemm_pp128_kernel(const GemmPa
   s.a_base = p.a;
   s.b_base = p.b;
   {
-    // lane l lands in row l / 8, physical chunk l % 8 of the 8 rows one load fills; rows start at multiples of 8, so
-    // (row >> 1) & 7 == (4 * wave + (l >> 4)) & 7 for every load of this wave
+    // lane l lands in row l / 8, physical chunk l % 8 of the 8 rows one load fills (rows start at multiples of 8); it
+    // fetches the logical chunk that belongs there under the (row & 7) swizzle
     const int lrow = lane >> 3;
-    const int key = (4 * wave + (lane >> 4)) & 7;
-    const int chunk_byte = ((lane & 7) ^ key) * 16;
+    const int chunk_byte = ((lane & 7) ^ lrow) * 16;
 #pragma unroll
     for (int i = 0; i < J_LOADS; ++i) {
       const int row = i * 64 + wave * 8 + lrow;
@@ -149,23 +146,21 @@ __global__ __launch_bounds__(J_THREADS) void int8_gemm_pp128_kernel(const GemmPa
       else
         s.goff[i] = (uint32_t)((int64_t)min(n0 + row - J_BM, p.N - 1) * p.ldb + chunk_byte);
     }
-    const int trow = grp * J_WM + l32, crow = J_BM + wave_n * J_WN + l32;
+    const int trow = grp * J_WM + l16, crow = J_BM + wave_n * J_WN + l16;
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {  // K sub-step k takes the 16-byte chunk 2k + kh of the row
-      s.tok_off[k] = trow * KSTEP + (((2 * k + kh) ^ ((trow >> 1) & 7)) << 4);
-      s.ch_off[k] = crow * KSTEP + (((2 * k + kh) ^ ((crow >> 1) & 7)) << 4);
+    for (int h = 0; h < 2; ++h) {  // K half h takes the 16-byte chunk q + 4h of the row
+      s.tok_off[h] = trow * KSTEP + (((q + 4 * h) ^ (trow & 7)) << 4);
+      s.ch_off[h] = crow * KSTEP + (((q + 4 * h) ^ (crow & 7)) << 4);
     }
   }
 
-  v16i acc[J_NT][J_MT];
+  v4i acc[J_NT][J_MT];
 #pragma unroll
   for (int i = 0; i < J_NT; ++i)
 #pragma unroll
-    for (int j = 0; j < J_MT; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    for (int j = 0; j < J_MT; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-  v4i w[J_NT][4], t[J_MT][4];
+  v4i w[J_NT][2], t[J_MT][2];
 
   // ---- prologue: steps 0 and 1
   issue_step(s, j_stage0, kb_begin);
@@ -196,23 +191,22 @@ __global__ __launch_bounds__(J_THREADS) void int8_gemm_pp128_kernel(const GemmPa
   // the last requests refetch the last step into rows nobody reads any more: they must not outlive the workgroup's LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-  // ---- epilogue: lane holds, for token m, channels n0 + 32 i + 8 g + 4 kh + (0..3), g = 0..3
+  // ---- epilogue: lane holds, for token m = 16 j + l16 of the wave's rows, channels 16 i + 4 q + (0..3) of its columns
   if constexpr (SPLIT) {
 #pragma unroll
     for (int j = 0; j < J_MT; ++j) {
-      const int m = m0 + grp * J_WM + j * 32 + l32;
+      const int m = m0 + grp * J_WM + j * 16 + l16;
       if (m >= p.M) continue;
 #pragma unroll
       for (int i = 0; i < J_NT; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int n = n0 + wave_n * J_WN + i * 32 + 8 * g + 4 * kh;
+        {
+          const int n = n0 + wave_n * J_WN + i * 16 + 4 * q;
           if (n >= p.N) continue;
           const int nvalid = min(4, p.N - n);
           int* wsp = reinterpret_cast<int*>(p.ws) + ((int64_t)tc.split * p.M + m) * p.N + n;
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            if (v < nvalid) wsp[v] = acc[i][j][4 * g + v];
+            if (v < nvalid) wsp[v] = acc[i][j][v];
         }
     }
     return;
@@ -225,12 +219,11 @@ __global__ __launch_bounds__(J_THREADS) void int8_gemm_pp128_kernel(const GemmPa
     asm volatile("s_barrier" ::: "memory");  // every wave's stray loads have landed: the stages are free
     float sa_j[J_MT];
 #pragma unroll
-    for (int j = 0; j < J_MT; ++j) sa_j[j] = p.sa[min(m0 + grp * J_WM + j * 32 + l32, p.M - 1)];
+    for (int j = 0; j < J_MT; ++j) sa_j[j] = p.sa[min(m0 + grp * J_WM + j * 16 + l16, p.M - 1)];
 #pragma unroll
     for (int i = 0; i < J_NT; ++i) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int col = wave_n * J_WN + i * 32 + 8 * g + 4 * kh;
+      {
+        const int col = wave_n * J_WN + i * 16 + 4 * q;
         const v4f sbv = *reinterpret_cast<const v4f*>(p.sb + n0 + col);
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
         if (p.bias) {
@@ -244,11 +237,11 @@ __global__ __launch_bounds__(J_THREADS) void int8_gemm_pp128_kernel(const GemmPa
           float r[4];
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
-            float x = mul_rn((float)acc[i][j][4 * g + v], mul_rn(sbv[v], sa_j[j]));
+            float x = mul_rn((float)acc[i][j][v], mul_rn(sbv[v], sa_j[j]));
             if (p.bias) x = add_rn(x, bv[v]);
             r[v] = x;
           }
-          out_tile_put4(j_stages, grp * J_WM + j * 32 + l32, col, p.out_dtype, r);
+          out_tile_put4(j_stages, grp * J_WM + j * 16 + l16, col, p.out_dtype, r);
         }
       }
     }
@@ -258,27 +251,26 @@ __global__ __launch_bounds__(J_THREADS) void int8_gemm_pp128_kernel(const GemmPa
   }
 #pragma unroll
   for (int j = 0; j < J_MT; ++j) {
-    const int m = m0 + grp * J_WM + j * 32 + l32;
+    const int m = m0 + grp * J_WM + j * 16 + l16;
     if (m >= p.M) continue;
     const float sa_m = raw ? 1.f : p.sa[m];
 #pragma unroll
     for (int i = 0; i < J_NT; ++i) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wave_n * J_WN + i * 32 + 8 * g + 4 * kh;
+      {
+        const int n = n0 + wave_n * J_WN + i * 16 + 4 * q;
         if (n >= p.N) continue;
         const int nvalid = min(4, p.N - n);
         if (raw) {
           int* o = reinterpret_cast<int*>(p.out) + (int64_t)m * p.ldo + n;
 #pragma unroll
           for (int v = 0; v < 4; ++v)
-            if (v < nvalid) o[v] = acc[i][j][4 * g + v];
+            if (v < nvalid) o[v] = acc[i][j][v];
         } else {
           float r[4];
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             const int nn = min(n + v, p.N - 1);
-            float x = mul_rn((float)acc[i][j][4 * g + v], mul_rn(p.sb[nn], sa_m));
+            float x = mul_rn((float)acc[i][j][v], mul_rn(p.sb[nn], sa_m));
             if (p.bias) {
               const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[nn];
               x = add_rn(x, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
