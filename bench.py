@@ -473,12 +473,22 @@ def bench_mfma_stream(steps, warmup):
     stream = torch.cuda.current_stream().cuda_stream
     iters = 2000
     flops = 256.0 * 8 * iters * 16 * 2 * 16 * 16 * 128
+    # INT8 operands as bench_int8_gemm has them: per-token quantized N(0,1) activations, per-channel quantized N(0, 0.02) weights
+    xi = torch.randn(n // 4096, 4096, generator=gen, device=dev)
+    a_i8 = torch.round(xi * (127.0 / xi.abs().amax(dim=1, keepdim=True))).to(torch.int8)
+    wi = torch.randn(n // 4096, 4096, generator=gen, device=dev) * 0.02
+    w_i8 = torch.round(wi * (127.0 / wi.abs().amax(dim=1, keepdim=True))).to(torch.int8)
+    out_i = torch.empty(256 * 512, dtype=torch.int32, device=dev)
     rows = []
-    for data, (pa, pb) in (("benchmark operand values", (a_real, w_q)), ("zeros", (zeros, zeros))):
+    for data, (pa, pb), (qa, qb) in (("benchmark operand values", (a_real, w_q), (a_i8, w_i8)), ("zeros", (zeros, zeros), (zeros, zeros))):
         for mode, name in ((0, "C=0 + 4 promotion FMAs per MFMA (fp32-scale kernel)"), (1, "accumulate in place (UE8M0 kernel)"),
-                           (2, "MFMA only")):
-            def step(i, mode=mode, pa=pa, pb=pb):
-                _lib.check(L.mi355_probe_fp8_mfma_stream(mode, 256, iters, pa.data_ptr(), pb.data_ptr(), out.data_ptr(), stream))
+                           (2, "MFMA only"), (3, "MFMA only, 32x32x64 instead of 16x16x128 (not used)"),
+                           (10, "int8 16x16x64 in place (INT8 kernels)"), (11, "int8 32x32x32 in place (not used)")):
+            def step(i, mode=mode, pa=pa, pb=pb, qa=qa, qb=qb):
+                if mode >= 10:
+                    _lib.check(L.mi355_probe_int8_mfma_stream(mode - 10, 256, iters, qa.data_ptr(), qb.data_ptr(), out_i.data_ptr(), stream))
+                else:
+                    _lib.check(L.mi355_probe_fp8_mfma_stream(mode, 256, iters, pa.data_ptr(), pb.data_ptr(), out.data_ptr(), stream))
 
             wall, ms, b2b = _time_launches(step, 1, max(10, steps // 2), 3)
             st = _stats(ms, b2b)

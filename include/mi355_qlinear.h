@@ -209,11 +209,19 @@ int mi355_fp8_blockwise_mm_kloop_ceiling(const void* a, const void* b, const flo
  * Measurement aid, not an operator (no counterpart in the reference): the fp8 matrix-instruction stream of the large-M
  * kernels with every operand in registers (no LDS, no global loads, no barriers), `workgroups` workgroups of 8 waves,
  * `iters` rounds of 16 instructions of 2 * 16 * 16 * 128 FLOP per wave.  mode 0: C = 0 and four promotion FMAs per result
- * (the fp32-scale kernel's compute phase); 1: accumulating in place (the UE8M0 kernel's); 2: C = 0, no vector arithmetic.
+ * (the fp32-scale kernel's compute phase); 1: accumulating in place (the UE8M0 kernel's); 2: C = 0, no vector arithmetic;
+ * 3: as 2 with v_mfma_f32_32x32x64_f8f6f4 (8 instructions of twice the FLOP), the instruction shape the kernels do not use.
  * a, b: 8 * 4 * 64 * 32 = 65536 bytes of e4m3fn operand values each (the timing depends on them through the chip's power
  * management); out: workgroups * 512 floats.  bench.py --workload mfma_stream reports the rates.
  */
 int mi355_probe_fp8_mfma_stream(int mode, int workgroups, int iters, const void* a, const void* b, void* out, void* stream);
+
+/*
+ * The same for the INT8 kernels (measurement aid, no counterpart in the reference): the same number of operations per
+ * round and wave, accumulating in place.  mode 0: 32 v_mfma_i32_16x16x64_i8 (the instruction the INT8 kernels use);
+ * 1: 16 v_mfma_i32_32x32x32_i8.  a, b: 65536 bytes of int8 operand values each; out: workgroups * 512 int32.
+ */
+int mi355_probe_int8_mfma_stream(int mode, int workgroups, int iters, const void* a, const void* b, void* out, void* stream);
 
 /*
  * Per-token x per-channel INT8 GEMM:  acc = sum_k a[m,k] * b[n,k] exactly in int32;

@@ -29,6 +29,7 @@ EXPORTS = (
     "mi355_fp8_blockwise_mm_noalloc",
     "mi355_fp8_blockwise_mm_kloop_ceiling",
     "mi355_probe_fp8_mfma_stream",
+    "mi355_probe_int8_mfma_stream",
     "mi355_fp8_blockwise_mm_ue8m0_workspace_bytes",
     "mi355_fp8_blockwise_mm_ue8m0",
     "mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes",
@@ -105,6 +106,8 @@ def lib() -> ctypes.CDLL:
     L.mi355_fp8_blockwise_mm_kloop_ceiling.restype = i32
     L.mi355_probe_fp8_mfma_stream.argtypes = [i32, i32, i32, vp, vp, vp, vp]
     L.mi355_probe_fp8_mfma_stream.restype = i32
+    L.mi355_probe_int8_mfma_stream.argtypes = [i32, i32, i32, vp, vp, vp, vp]
+    L.mi355_probe_int8_mfma_stream.restype = i32
     L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes.argtypes = [i64, i64, i64, i64]
     L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes.restype = sz
     L.mi355_fp8_blockwise_scaled_grouped_mm_plan.argtypes = [i64, i64, i64, i64, ctypes.c_char_p, sz]

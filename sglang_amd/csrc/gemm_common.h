@@ -245,7 +245,7 @@ int launch_fp8_grouped_pp(GroupedParams& gp, hipStream_t stream, const char* wha
 int launch_int8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);  // gemm_int8_dma3.hip: same tiling, int8 MFMA, int32 partials
 
 // Large-M INT8 GEMM (256 x 256 tile, 8 waves in two groups that alternate compute and memory phases, direct-to-LDS loads,
-// 32x32x32 MFMA); gemm_int8_pp.hip.  Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
+// 16x16x64 MFMA); gemm_int8_pp.hip.  Needs 16-byte aligned rows, K % 128 == 0 and row offsets below 4 GiB.
 int launch_int8_pp(GemmParams& p, hipStream_t stream, const char* what);
 // Mid-M INT8 GEMM (128 x 256 tile, the two-phase schedule over three LDS stages); gemm_int8_pp128.hip.  Same requirements;
 // optional split along K: the caller sets p.splits, p.kb_per_split and p.ws (int32 partials, ordered reduce afterwards).

@@ -79,7 +79,7 @@ def test_int8_scaled_mm(gpu, oracle, M, N, K, with_bias, out_dtype):
 
 @pytest.mark.parametrize("M,N,K", [(4096, 4096, 512), (4000, 4088, 1024), (2048, 8192, 256)])
 def test_large_m_kernel(gpu, oracle, M, N, K):
-    """The 256x256 direct-to-LDS kernel (32x32x32 MFMA): raw accumulators and epilogue on a sample of rows that includes
+    """The 256x256 direct-to-LDS kernel (16x16x64 MFMA): raw accumulators and epilogue on a sample of rows that includes
     tile borders and the ragged last tile, all columns."""
     from sglang_amd import ops
     from sglang_amd.sgl_kernel import int8_scaled_mm
