@@ -5,14 +5,16 @@
 // (K = 7168 -> N = 2048: 14 MB) then makes ~100 workgroups, half the CUs stay empty, and a second launch adds the K
 // ranges.  Both cost more than the traffic itself: 6.1 us + 2.8 us for a weight that leaves HBM in 2 us.  Here a workgroup
 // owns 16 channels - one MFMA tile for the <= 16 tokens - over ALL of K; its W waves take K blocks w, w + W, w + 2 W, ...
-// so that neighbouring waves read neighbouring 128-byte pieces of the same weight rows.  A wave requests every block of
-// its share at once, straight into registers in MFMA operand layout (two 16-byte pieces per lane and block for the
-// weight, two for the tokens, which come from L2 after the first workgroups touched them), multiplies them as they
-// arrive, and the W partial tiles are added through LDS in wave order by wave 0, which applies the epilogue and stores.
-// No workspace, no second launch, N / 16 workgroups, and the whole weight is requested within the first microsecond.
+// so that neighbouring waves read neighbouring 128-byte pieces of the same weight rows.  A wave requests its blocks
+// straight into registers in MFMA operand layout (two 16-byte pieces per lane and block for the weight, two for the
+// tokens, which come from L2 after the first workgroups touched them), multiplies them as they arrive, and the W partial
+// tiles are added through LDS in wave order by wave 0, which applies the epilogue and stores.
+// No workspace, no second launch, N / 16 workgroups.
 //
-// A wave's share is KBW blocks per round (all requested before the first is used); longer K takes several rounds, whose
-// start-up gaps the other workgroups on the CU fill (~80 registers: six waves per SIMD).
+// A wave keeps a ring of KBW register slots: a slot is multiplied and requested again at once for the block KBW further
+// on, so KBW - 1 blocks stay in flight for as long as K lasts (requesting KBW blocks together and waiting for all of
+// them left nothing in flight between such rounds: K = 18432 -> N = 7168 at M = 1 30.4 -> 27.2 us, INT8 K = 14336 -> N = 4096
+// 15.6 -> 14.5 us; shapes of one or two turns are unchanged).  ~80-90 registers: five waves per SIMD.
 // Blocks past the end of K are fetched from the last valid block and multiply a zero scale (FP8) or zeroed tokens (INT8).
 // Requires K % 128 == 0, N % 16 == 0, 16-byte aligned rows.  FP8 sums differ from the streaming kernel's in the order of
 // the additions only (per wave in K order, then over waves); INT8 results are exact either way.
@@ -20,6 +22,8 @@
 
 namespace mi355 {
 namespace {
+
+typedef const __attribute__((address_space(4))) float* cfloat_ptr;
 
 struct Frag {
   u32x4 lo, hi;
@@ -47,59 +51,108 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
   const uint8_t* wrow = p.b + (int64_t)(n0 + l16) * p.ldb + q * 16;
   const uint8_t* trow = p.a + (int64_t)tok * p.lda + q * 16;
   const float* sa_row = IS_FP8 ? p.sa + (int64_t)tok * p.sa_sm : nullptr;
-  const float* sb_row = IS_FP8 ? p.sb + (int64_t)(UE8M0 ? n0 : (n0 >> 7)) * p.sb_sn : nullptr;  // wave-uniform
+  // wave-uniform, read through the constant address space: scalar loads, which the vector-memory counter does not see
+  const cfloat_ptr sb_row = (cfloat_ptr)(IS_FP8 ? p.sb + (int64_t)(UE8M0 ? n0 : (n0 >> 7)) * p.sb_sn : nullptr);
 
   acc4 acc = {0, 0, 0, 0};
-  const int rounds = (p.kb_total + W * KBW - 1) / (W * KBW);
-  for (int r = 0; r < rounds; ++r) {
-    Frag wf[KBW], tf[KBW];
-    float sav[KBW], sbv[KBW];
-#pragma unroll
-    for (int j = 0; j < KBW; ++j) {
-      const int kb = (r * KBW + j) * W + wave;  // wave-uniform
-      const int kc = min(kb, p.kb_total - 1);
-      wf[j].lo = *reinterpret_cast<const u32x4*>(wrow + (int64_t)kc * KSTEP);
-      wf[j].hi = *reinterpret_cast<const u32x4*>(wrow + (int64_t)kc * KSTEP + 64);
-      tf[j].lo = *reinterpret_cast<const u32x4*>(trow + (int64_t)kc * KSTEP);
-      tf[j].hi = *reinterpret_cast<const u32x4*>(trow + (int64_t)kc * KSTEP + 64);
-      if constexpr (UE8M0) {  // the words that hold block kc's bytes, kept as raw bits
-        sav[j] = sa_row[(int64_t)(kc >> 2) * p.sa_sk];
-        sbv[j] = sb_row[(int64_t)(kc >> 2) * p.sb_sk];
-      } else if constexpr (IS_FP8) {
-        sav[j] = sa_row[(int64_t)kc * p.sa_sk];
-        sbv[j] = sb_row[(int64_t)kc * p.sb_sk];
-      }
+  // A ring of KBW register slots: the wave's i-th block is K block i * W + wave; slot j is multiplied and at once requested
+  // again for the block KBW further on, so KBW - 1 blocks are always in flight (rounds of KBW blocks that are requested
+  // together and awaited together leave the wave with nothing in flight between rounds).  Blocks past the end of K (the padding of the
+  // last turn) clamp to the last one and contribute zero.
+  // The loads and their waits are written as instructions: left to the compiler, the wait at the loop's back edge becomes
+  // "everything but the newest block" and the ring runs empty once per turn.  A slot's registers are outputs of its request
+  // and in-out operands of its wait, so no compiler-generated instruction touches them in between; vector loads complete in
+  // order, so "at most (KBW - 1) blocks' loads outstanding" means the oldest slot has landed.
+  constexpr int LOADS = IS_FP8 ? 5 : 4;  // per block: two weight and two token fragments' halves, the token scale (word)
+  Frag wf[KBW], tf[KBW];
+  float sav[KBW], sbv[KBW];
+  auto request = [&](int j, int i) {
+    const int kc = min(i * W + wave, p.kb_total - 1);  // wave-uniform
+    const uint8_t* wp = wrow + (int64_t)kc * KSTEP;
+    const uint8_t* tp = trow + (int64_t)kc * KSTEP;
+    asm volatile(
+        "global_load_dwordx4 %0, %4, off\n\tglobal_load_dwordx4 %1, %4, off offset:64\n\t"
+        "global_load_dwordx4 %2, %5, off\n\tglobal_load_dwordx4 %3, %5, off offset:64"
+        : "=&v"(wf[j].lo), "=&v"(wf[j].hi), "=&v"(tf[j].lo), "=&v"(tf[j].hi)
+        : "v"(wp), "v"(tp)
+        : "memory");
+    if constexpr (IS_FP8) {
+      // fp32 scales: block kc's; packed exponents: the word that holds block kc's byte, kept as raw bits
+      const float* sp = sa_row + (int64_t)(UE8M0 ? (kc >> 2) : kc) * p.sa_sk;
+      asm volatile("global_load_dword %0, %1, off" : "=&v"(sav[j]) : "v"(sp) : "memory");
+      sbv[j] = sb_row[(int64_t)(UE8M0 ? (kc >> 2) : kc) * p.sb_sk];  // wave-uniform: a scalar load, not counted in vmcnt
     }
-    // every request of the round is out before the first result is used: without this fence the scheduler pairs each
-    // block's loads with its MFMA to save registers, and the wave waits out one memory latency per block
-    __builtin_amdgcn_sched_barrier(0);
+  };
+  // waits until at most `behind` blocks requested after slot j's are still outstanding: slot j has landed
+  auto await = [&](int j, int behind) {  // `behind` is a constant at every call; the switch folds away
+#define MI355_WS_AWAIT(NBLK)                                                                                                     \
+  if constexpr (IS_FP8)                                                                                                          \
+    asm volatile("s_waitcnt vmcnt(%5)" : "+v"(wf[j].lo), "+v"(wf[j].hi), "+v"(tf[j].lo), "+v"(tf[j].hi), "+v"(sav[j]) : "n"((NBLK)*LOADS)); \
+  else                                                                                                                           \
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(wf[j].lo), "+v"(wf[j].hi), "+v"(tf[j].lo), "+v"(tf[j].hi) : "n"((NBLK)*LOADS))
+    switch (behind) {
+      case 3: MI355_WS_AWAIT(3); break;
+      case 2: MI355_WS_AWAIT(2); break;
+      case 1: MI355_WS_AWAIT(1); break;
+      default: MI355_WS_AWAIT(0); break;
+    }
+#undef MI355_WS_AWAIT
+  };
+  auto multiply = [&](int j, int i) {
+    const int kb = i * W + wave;
+    const bool valid = kb < p.kb_total;
+    if constexpr (UE8M0) {
+      const int shift = 8 * (min(kb, p.kb_total - 1) & 3);
+      const int ea = in_vgpr((int)((__float_as_uint(sbv[j]) >> shift) & 0xffu)), eb = (int)((__float_as_uint(sav[j]) >> shift) & 0xffu);
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      Frag t = tf[j];
+      if (!valid) t.lo = z, t.hi = z;  // a block past the end of K multiplies zeros
+      acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(t), acc, 0, 0, 0, ea, 0, eb);
+    } else if constexpr (IS_FP8) {
+      const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(tf[j]), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0,
+                                                                        0, 0, 0, 0);
+      const float sc = valid ? sav[j] * sbv[j] : 0.f;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[v] = fmaf(part[v], sc, acc[v]);
+    } else {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      const u32x4 tlo = valid ? tf[j].lo : z, thi = valid ? tf[j].hi : z;
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].lo.x, (int)wf[j].lo.y, (int)wf[j].lo.z, (int)wf[j].lo.w},
+                                                  v4i{(int)tlo.x, (int)tlo.y, (int)tlo.z, (int)tlo.w}, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].hi.x, (int)wf[j].hi.y, (int)wf[j].hi.z, (int)wf[j].hi.w},
+                                                  v4i{(int)thi.x, (int)thi.y, (int)thi.z, (int)thi.w}, acc, 0, 0, 0);
+    }
+  };
+  const int blocks = (p.kb_total + W * KBW - 1) / (W * KBW) * KBW;  // per wave, padded to whole turns of the ring
+#pragma unroll
+  for (int j = 0; j < KBW; ++j) request(j, j);
+  // the fences keep the order "await and multiply slot j, request it again"
+  int i0 = 0;
+  for (; i0 + KBW < blocks; i0 += KBW) {
 #pragma unroll
     for (int j = 0; j < KBW; ++j) {
-      const int kb = (r * KBW + j) * W + wave;
-      const bool valid = kb < p.kb_total;
-      if constexpr (UE8M0) {
-        const int shift = 8 * (min(kb, p.kb_total - 1) & 3);
-        const int ea = in_vgpr((int)((__float_as_uint(sbv[j]) >> shift) & 0xffu)), eb = (int)((__float_as_uint(sav[j]) >> shift) & 0xffu);
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        Frag t = tf[j];
-        if (!valid) t.lo = z, t.hi = z;  // a block past the end of K multiplies zeros
-        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(t), acc, 0, 0, 0, ea, 0, eb);
-      } else if constexpr (IS_FP8) {
-        const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(tf[j]), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0,
-                                                                          0, 0, 0, 0);
-        const float sc = valid ? sav[j] * sbv[j] : 0.f;
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[v] = fmaf(part[v], sc, acc[v]);
-      } else {
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        const u32x4 tlo = valid ? tf[j].lo : z, thi = valid ? tf[j].hi : z;
-        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].lo.x, (int)wf[j].lo.y, (int)wf[j].lo.z, (int)wf[j].lo.w},
-                                                    v4i{(int)tlo.x, (int)tlo.y, (int)tlo.z, (int)tlo.w}, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].hi.x, (int)wf[j].hi.y, (int)wf[j].hi.z, (int)wf[j].hi.w},
-                                                    v4i{(int)thi.x, (int)thi.y, (int)thi.z, (int)thi.w}, acc, 0, 0, 0);
-      }
+      __builtin_amdgcn_sched_barrier(0);
+      await(j, KBW - 1);
+      multiply(j, i0 + j);
+      __builtin_amdgcn_sched_barrier(0);
+      request(j, i0 + j + KBW);
     }
   }
+  // last turn: nothing is requested any more, so slot j has KBW - 1 - j blocks behind it
+  static_assert(KBW == 4, "the last turn is written out for four slots");
+  __builtin_amdgcn_sched_barrier(0);
+  await(0, 3);
+  multiply(0, i0);
+  __builtin_amdgcn_sched_barrier(0);
+  await(1, 2);
+  multiply(1, i0 + 1);
+  __builtin_amdgcn_sched_barrier(0);
+  await(2, 1);
+  multiply(2, i0 + 2);
+  __builtin_amdgcn_sched_barrier(0);
+  await(3, 0);
+  multiply(3, i0 + 3);
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- add the W partial tiles in wave order
   if (wave != 0) red[wave][lane] = acc;
@@ -157,11 +210,11 @@ int launch_wavesplit(GemmParams& p, hipStream_t stream, const char* what) {
 
 }  // namespace
 
-// Waves per workgroup and K blocks per wave and round.  Measured (us, M = 1; waves x blocks): K = 4096 -> N = 28672 INT8:
-// 8x4 24.5, 4x8 28.1, 4x4 30.6, 16x4 42.0; K = 7168 -> N = 36864 FP8: 8x4 49.2, 4x8 49.8, 4x4 51.2, 8x8 55.2, 16x4 56.3;
-// K = 14336 -> N = 4096 INT8: 4x4 15.5, 16x4 15.9, 8x4 16.3; K = 18432 -> N = 7168 FP8: 4x4 30.4, 4x8 30.9, 8x4 31.5, 16x4 36.4.
-// Eight waves of four blocks up to K = 8192 (one or two rounds); for longer K four waves, whose many short rounds overlap
-// across the workgroups that share a CU; four waves also where K has at most 16 blocks.
+// Waves per workgroup (the ring has four slots).  Measured (us, M = 1; 4 / 8 waves): K = 4096 -> N = 28672 INT8 27.3 / 24.8,
+// K = 4096 -> N = 6144 INT8 10.7 / 10.3, K = 7168 -> N = 36864 FP8 48.9 / 48.2, K = 14336 -> N = 4096 INT8 14.5 / 15.7,
+// K = 18432 -> N = 7168 FP8 27.2 / 29.8, K = 2048 -> N = 7168 FP8 7.0 / 9.2, K = 1536 -> N = 24576 FP8 11.5 / 18.1; sixteen
+// waves were slower everywhere.  Eight waves up to K = 8192 (one or two turns of the ring); four for longer K and where K
+// has at most 16 blocks.
 WavesplitShape wavesplit_shape(int64_t K) {
   const int64_t kb = (K + KSTEP - 1) / KSTEP;
   return (kb > 16 && kb <= 64) ? WavesplitShape{8, 4} : WavesplitShape{4, 4};

@@ -36,17 +36,18 @@ struct RouteConstants {
   double dma3_small_tile_factor = 0.65;  // the byte-model score of 64-token tiles above 128 tokens
   // ---- decode sizes (M <= 16): the kernel that splits K over the waves of a workgroup (gemm_decode_wavesplit.hip) against
   //      the streaming kernel with its reduce launch (gemm_fp8_decode.hip).  Median launch, us, wave-split / streaming:
-  //      FP8  M=1: 7168->2048 9.2/10.8, 7168->36864 49.2/52.1, 18432->7168 30.4/30.6;  M=4: 7168->1536 9.8/11.0, 1536->24576
-  //      12.2/13.4, 512->32768 14.6/8.9;  M=8: 7168->36864 64.1/57.3, 18432->7168 33.6/31.9;  M=16: 2048->7168 8.7/11.3,
-  //      4096->4096 9.0/11.4, 7168->2048 11.6/10.5 (128 workgroups: half the CUs), 7168->36864 81/60.
-  //      INT8 M=1: 4096->6144 10.0/11.4, 4096->28672 24.5/30.9, 14336->4096 15.5/18.4;  M=16: 4096->6144 12.4/12.1,
-  //      4096->28672 32.7/35.1, 14336->4096 18.7/19.7.
+  //      FP8  7168->36864: M=1 48.1/52.1, 2 50.3/53.0, 3 51.8/53.9, 4 54.3/54.3, 8 62.7/56.9, 16 74.2/59.8;
+  //      18432->7168: M=1 27.2/30.6, 2 28.0/31.3, 4 30.1/31.5, 8 33.5/32.1, 16 38.4/33.3;  7168->2048: M=2 9.3/10.9, 4 9.6/11.1,
+  //      8 10.4/11.1, 16 11.7/10.9 (128 workgroups: half the CUs);  7168->4096: M=2 9.5/12.1, 16 11.6/12.6;  2048->7168: M=2
+  //      8.7/11.0, 16 9.0/11.2;  M=4: 7168->1536 9.8/11.0, 1536->24576 12.2/13.4, 512->32768 14.6/8.9.
+  //      INT8 M=1: 4096->6144 10.2/11.4, 4096->28672 24.7/30.9, 14336->4096 14.5/18.4;  M=16: 4096->6144 12.4/12.1,
+  //      4096->28672 33.0/35.1, 14336->4096 18.2/19.7.
   //      Every token row costs the wave-split kernel a pass over K from L2 per workgroup, so it wins for few tokens or small
   //      weights; the INT8 streaming kernel is slower than the FP8 one, so there it wins at every decode size.
   double wavesplit_min_kblocks = 8.0;              // shorter K: one block per wave, the streaming kernel's wide tiles win
   double wavesplit_small_weight_bytes = 32e6;      // FP8: up to here the second launch it saves outweighs the token traffic ...
-  double wavesplit_small_weight_max_tokens = 4.0;  // ... for this many tokens, or for any M <= 16 once N / 16 fills the CUs
-  double wavesplit_large_weight_max_tokens = 2.0;  // FP8, larger weights: the token traffic decides
+  double wavesplit_small_weight_max_tokens = 8.0;  // ... for this many tokens, or for any M <= 16 once N / 16 fills the CUs
+  double wavesplit_large_weight_max_tokens = 4.0;  // FP8, larger weights: the token traffic decides
 };
 constexpr int ROUTE_CONSTANT_COUNT = sizeof(RouteConstants) / sizeof(double);
 static_assert(sizeof(RouteConstants) == ROUTE_CONSTANT_COUNT * sizeof(double), "the table is read as an array of doubles");
