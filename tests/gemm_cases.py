@@ -3,7 +3,7 @@ parity tests, plus the full-size shapes of the benchmark configurations.
 
 A *variant* is one compiled code path: the kernel, its token-tile height, whether it writes split-K partial sums,
 for the decode kernel how many 128-channel groups a workgroup walks, for the wave-split decode kernel how many waves
-share a workgroup's K and whether a wave's share takes several rounds, for the large-M kernels whether K ends on a
+share a workgroup's K and whether a wave's share takes one turn of its four-slot register ring ("one_round") or several, for the large-M kernels whether K ends on a
 128-byte block.  `variant_of` maps a plan (sglang_amd._lib.gemm_plan) to such a key.
 """
 
@@ -101,7 +101,7 @@ def variant_of(plan: dict, K: int):
     if k == "decode":
         g = plan["groups_per_wg"]
         return (k, sp, f"gpw{g}" if g < 3 else "gpw3+")
-    if k == "decode_wavesplit":  # waves per workgroup; one round of K blocks or several
+    if k == "decode_wavesplit":  # waves per workgroup; one turn of the wave's four-slot ring or several
         waves = plan["groups_per_wg"]
         return (k, f"w{waves}", "rounds" if -(-K // 128) > 4 * waves else "one_round")
     if k == "pingpong128":
