@@ -348,7 +348,8 @@ def bench_fp8_ue8m0_gemm(name, M, K, N, steps, warmup):
     st = _stats(ms, b2b)
     flops, nbytes = gemm_flops(M, N, K), fp8_gemm_algorithmic_bytes(M, N, K)
     plan = _lib.gemm_plan("fp8", M, N, K)
-    hw = plan["kernel"] in ("pingpong", "dma3", "decode_wavesplit") and K % 128 == 0  # kernels whose MFMA applies the exponents
+    # kernels whose MFMA applies the exponents
+    hw = plan["kernel"] in ("pingpong", "dma3", "decode", "decode_wavesplit") and K % 128 == 0
     kern = plan["kernel"] + (" (MFMA-applied scales)" if hw else " after unpack")
     return {
         "workload": f"fp8_gemm_ue8m0 {name} M={M} K={K} N={N} (e4m3fn x e4m3fn, packed UE8M0 scales on both sides, bf16 out)",
@@ -856,6 +857,10 @@ def main():
             also.append(bench_fp8_ceiling(4096, K, N, S, W))
             also.append(bench_mfma_stream(S, W))
             also.append(bench_fp8_ue8m0_gemm("gate_up", 4096, K, N, S, W))
+            # the same operator at decode and mid-M sizes: wave-split, streaming decode and three-stage kernels, each
+            # with the scales applied by the MFMA
+            for M in (1, 8, 128):
+                also.append(bench_fp8_ue8m0_gemm("gate_up", M, K, N, S, W))
             also.append(bench_silu_quant(S, W))
             # expert GEMMs of DeepSeek-R1 (shapes of the reference's grouped-GEMM benchmark): prefill TP=8, prefill EP=16, decode EP=8
             for E, rows, Kg, Ng in ((256, 128, 7168, 512), (16, 512, 7168, 4096), (32, 4, 7168, 4096)):
