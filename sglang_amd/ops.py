@@ -10,6 +10,7 @@ stream to ``libmi355_qlinear.so``.
 """
 from __future__ import annotations
 
+import functools
 from typing import Optional
 
 import torch
@@ -61,7 +62,19 @@ def _stream() -> int:
         # (inside a capture the set-up is left alone: the two entry points that need it say so in their error)
         check(lib().mi355_qlinear_init())
         _ready_devices.add(dev)
+    if _raw_stream is not None:  # the handle itself, without building a torch.cuda.Stream object around it (~3 us a call)
+        return _raw_stream(dev)
     return torch.cuda.current_stream().cuda_stream
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+@functools.lru_cache(maxsize=8192)
+def _workspace_bytes(query: str, *dims: int) -> int:
+    """Workspace size of an entry point for a shape (the `<entry>_workspace_bytes` query): a pure function of the shape,
+    asked once per shape."""
+    return int(getattr(lib(), query)(*dims))
 
 
 def _require(cond: bool, msg: str) -> None:
@@ -217,7 +230,7 @@ def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
 
 def _launch_fp8_mm(a, b_ptr, ldb, sa, sb_ptr, sb_sn, sb_sk, out, M, N, K):
     L = lib()
-    ws_bytes = L.mi355_fp8_blockwise_mm_workspace_bytes(M, N, K)
+    ws_bytes = _workspace_bytes("mi355_fp8_blockwise_mm_workspace_bytes", int(M), int(N), int(K))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     check(
         L.mi355_fp8_blockwise_mm(
@@ -342,7 +355,7 @@ def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[to
     if M == 0:
         return out
     L = lib()
-    ws_bytes = L.mi355_fp8_scaled_mm_workspace_bytes(M, N, K)
+    ws_bytes = _workspace_bytes("mi355_fp8_scaled_mm_workspace_bytes", int(M), int(N), int(K))
     ws = _workspace(ws_bytes, mat_a.device)
     check(L.mi355_fp8_scaled_mm(mat_a.data_ptr(), mat_b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(),
                                 bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype], M, N, K,
@@ -373,7 +386,7 @@ def block_fp8_linear(x2d: torch.Tensor, weight: torch.Tensor, weight_scale: torc
     if M == 0:
         return out
     L = lib()
-    ws_bytes = L.mi355_fp8_block_linear_workspace_bytes(M, N, K)
+    ws_bytes = _workspace_bytes("mi355_fp8_block_linear_workspace_bytes", int(M), int(N), int(K))
     ws = _workspace(ws_bytes, x2d.device)
     check(L.mi355_fp8_block_linear(x2d.data_ptr(), _DT[x2d.dtype], weight.data_ptr(), weight_scale.data_ptr(),
                                    weight_scale.stride(0), weight_scale.stride(1),
@@ -408,7 +421,7 @@ def fp8_blockwise_mm_ue8m0(a: torch.Tensor, b: torch.Tensor, a_words: torch.Tens
     if M == 0 or N == 0:
         return out
     L = lib()
-    ws_bytes = L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(M, N, K)
+    ws_bytes = _workspace_bytes("mi355_fp8_blockwise_mm_ue8m0_workspace_bytes", int(M), int(N), int(K))
     ws = _workspace(ws_bytes, a.device)
     check(L.mi355_fp8_blockwise_mm_ue8m0(
         a.data_ptr(), b.data_ptr(), a_words.data_ptr(), b_words.data_ptr(), bias.data_ptr() if bias is not None else None,
@@ -453,7 +466,7 @@ def _grouped_mm(op, output, a, b, scales_a, scales_b, problem_sizes, expert_offs
     if total_m == 0 or N == 0 or E == 0:
         return
     L = lib()
-    need = L.mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes(E, total_m, N, K)
+    need = _workspace_bytes("mi355_fp8_blockwise_scaled_grouped_mm_workspace_bytes", int(E), int(total_m), int(N), int(K))
     ws = workspace
     if not (ws.is_cuda and ws.is_contiguous() and ws.numel() * ws.element_size() >= need and ws.data_ptr() % 256 == 0):
         ws = _workspace(need, a.device)
@@ -531,7 +544,7 @@ def _launch_int8_mm(mat_a, mat_b, scales_a, scales_b, bias, out):
     M, K = mat_a.shape
     N = mat_b.size(1)
     L = lib()
-    ws_bytes = L.mi355_int8_scaled_mm_workspace_bytes(M, N, K)
+    ws_bytes = _workspace_bytes("mi355_int8_scaled_mm_workspace_bytes", int(M), int(N), int(K))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=mat_a.device) if ws_bytes else None
     check(
         L.mi355_int8_scaled_mm(

@@ -122,7 +122,7 @@ def test_fused_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (8, 2048, 7168), (3, 16640, 4480), (8, 7168, 18432), (16, 512, 512), (5, 66048, 512),
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (12, 2048, 7168), (6, 16640, 4480), (8, 7168, 18432), (16, 512, 512), (5, 66048, 512),
                                    (9, 256, 128)])
 def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype):
     """At decode sizes the one-call linear has no quantizer launch: the streaming decode kernel quantizes the tokens of
