@@ -6,8 +6,8 @@ state at replay time (the reference runs these operators inside its decode graph
 python/sglang/srt/model_executor/cuda_graph_runner.py:452-540).  Every replay is compared with the eager result of the
 same inputs (bit for bit: same kernels, deterministic reduce order) and the first one with the CPU oracle.  Replays are
 separated by eager work and synchronizations, and the graph holds no memset node of its own (split-K partial sums need no
-clearing).  Shapes cover a split-K decode plan (workspace from torch inside the capture), a mid-M plan with re-laid-out
-token scales, and an unsplit plan.
+clearing).  Shapes cover the wave-split decode plan, a split-K decode plan (workspace from torch inside the capture), a mid-M
+plan with re-laid-out token scales, and an unsplit plan.
 """
 import pytest
 import torch
@@ -32,7 +32,7 @@ def _linear_chain(x, w_q, w_s, wi_q, wi_s):
     return x_q, x_s, y, y2, z
 
 
-@pytest.mark.parametrize("M", [4, 48, 300])
+@pytest.mark.parametrize("M", [4, 12, 48, 300])  # wave-split decode, split-K streaming decode, mid-M, unsplit
 def test_capture_and_replay_matches_eager(gpu, oracle, M):
     from sglang_amd import _lib
 
@@ -72,6 +72,49 @@ def test_capture_and_replay_matches_eager(gpu, oracle, M):
             assert torch.equal(got[0].cpu().view(torch.uint8), q_o.view(torch.uint8)) and torch.equal(got[1].cpu(), s_o)
             ref, mag = oracle.fp8_blockwise_mm(q_o, w_q.cpu(), s_o, w_s.cpu(), torch.float32, want_abs=True)
             check_fp8_gemm(got[2], ref, mag, f"replay {i}")
+
+
+@pytest.mark.parametrize("M", [2, 12, 48])  # wave-split decode, split-K streaming decode, mid-M: each with MFMA-applied scales
+def test_packed_scale_linear_replays(gpu, M):
+    """Quantizer with packed UE8M0 scales -> GEMM that takes the packed words on both operands, captured and replayed with
+    new inputs; every replay equals the eager result of the same input bit for bit."""
+    from sglang_amd import _lib
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul_deepgemm
+    from sglang_amd.fp8_utils import requant_weight_ue8m0
+
+    K, N = 2048, 1024
+    print(f"case M={M}: {_lib.gemm_plan('fp8', M, N, K)}", flush=True)
+    w_q, w_s = make_fp8_weight(N, K, seed=21)
+    w2, sw = requant_weight_ue8m0(w_q.to(gpu), w_s.to(gpu), [128, 128])
+
+    def chain(x):
+        x_q, x_s = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True,
+                                                    enable_v2=True)
+        return x_q, x_s, w8a8_block_fp8_matmul_deepgemm(x_q, w2, x_s, sw, [128, 128], torch.bfloat16)
+
+    inputs = [make_activation(M, K, seed=200 + i) for i in range(3)]
+    static_x = inputs[0].to(gpu).clone()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(2):
+            chain(static_x)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            static_out = chain(static_x)
+    torch.cuda.synchronize()
+    for i, x in enumerate(inputs[1:] + inputs[:1]):
+        static_x.copy_(x.to(gpu))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in static_out]
+        want = chain(x.to(gpu))
+        torch.cuda.synchronize()
+        assert torch.equal(got[0].view(torch.uint8), want[0].view(torch.uint8)), i
+        assert torch.equal(got[1], want[1]), i
+        assert torch.equal(got[2].view(torch.int16), want[2].view(torch.int16)), i
+        assert bool(torch.isfinite(got[2]).all())
 
 
 def test_grouped_gemm_replays_with_new_routing(gpu, oracle):
