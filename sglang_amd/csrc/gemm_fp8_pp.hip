@@ -183,7 +183,7 @@ __device__ __forceinline__ void read_operands(const PpState& s, const uint8_t* c
     if constexpr (SM == SM_UE8M0)
       scb[jj] = __uint_as_float(__float_as_uint(scp[(HALF * G_HT + jj) * 16]) >> ((kb & 3) * 8));
     else if constexpr (SM == SM_EPILOGUE)
-      scb[jj] = __uint_as_float(127u);
+      scb[jj] = __int_as_float(in_vgpr(127));  // (a constant, too, is put into its register where every lane is active)
     else
       scb[jj] = scp[(HALF * G_HT + jj) * 16] * sbv;
   }
@@ -371,7 +371,7 @@ __device__ __forceinline__ void pp_tile(const GemmParams& p, const int m0, const
   auto k_block = [&](uint8_t* cur, uint8_t* nxt, int kb, float sbv) {
     const float* sc_cur = g_scale + (kb & 3) * G_BM;
     // the weight block's exponent byte, in byte 0 of a register (for SM_UE8M0 sbv carries the packed word as bits)
-    const int w_scale = UE8M0 ? in_vgpr((int)(__float_as_uint(sbv) >> ((kb & 3) * 8))) : 127;
+    const int w_scale = HW_SCALE ? in_vgpr(UE8M0 ? (int)(__float_as_uint(sbv) >> ((kb & 3) * 8)) : 127) : 127;
     if constexpr (!HW_SCALE) retire<1>(pd, acc);  // last tile of the previous block (adds zero the first time)
     read_operands<0, SM>(s, cur, sc_cur, sbv, kb, w, tok, scb);
     if constexpr (!NOLOAD) issue_set_b<KFULL>(s, nxt, kb + 1);

@@ -21,7 +21,8 @@ FP8 = torch.float8_e4m3fn
 # decode sizes on the wave-split kernel, which also lets the MFMA apply the scales (8 and 4 waves, a ragged last round and a
 # partly used last exponent word: K = 4480 is 35 blocks; N = 576 is not a multiple of 128)
 SHAPES = [(4096, 4352, 512), (4096, 4352, 1152), (4000, 4352, 640), (4, 512, 1024), (16, 2048, 7168), (200, 16384, 2048),
-          (50, 384, 512), (1500, 640, 1024), (2, 2048, 7168), (3, 1536, 4480), (1, 1024, 18432), (5, 576, 2048)]
+          (50, 384, 512), (1500, 640, 1024), (2, 2048, 7168), (3, 1536, 4480), (1, 1024, 18432), (5, 576, 2048),
+          (3990, 4224, 640)]  # two-phase kernel: a last token tile with 6 of 16 rows and half a last channel tile (guarded stores)
 
 
 def _unpack_bytes(words, groups):
