@@ -550,11 +550,12 @@ def bench_fp8_linear(M, K, N, steps, warmup, two_step):
     wall, ms, b2b = _time_launches(step, nbuf, steps, warmup)
     st = _stats(ms, b2b)
     flops, nbytes = gemm_flops(M, N, K), fp8_gemm_algorithmic_bytes(M, N, K) + M * K
-    plan = _lib.gemm_plan("fp8", M, N, K)
+    plan = _lib.gemm_plan("fp8", M, N, K) if two_step else _lib.block_linear_plan(M, N, K)
+    label = ("quantizer + " if two_step or plan["quantizer"] == "launch" else "") + plan["kernel"] + ("" if two_step or plan["quantizer"] == "launch" else " (quantizer in its prologue)")
     return {
         "workload": f"fp8_linear{'_two_step' if two_step else ''} M={M} K={K} N={N} (bf16 in, 1x128 quantization, blockwise GEMM, bf16 out)",
         "value": flops / (wall / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall / steps * 1e3, "kernel_ms": st,
-        "dtype": "fp8(e4m3fn) MFMA, f32 accumulate", "kernel": ("quantizer + " if two_step or plan["kernel"] != "decode" else "") + plan["kernel"],
+        "dtype": "fp8(e4m3fn) MFMA, f32 accumulate", "kernel": label,
         "roofline": _roofline(flops, nbytes, st, FP8_PEAK_TFLOPS, "TFLOP/s"),
     }
 

@@ -38,6 +38,7 @@ EXPORTS = (
     "mi355_int8_scaled_mm_workspace_bytes",
     "mi355_int8_scaled_mm",
     "mi355_fp8_blockwise_mm_plan",
+    "mi355_fp8_block_linear_plan",
     "mi355_int8_scaled_mm_plan",
     "mi355_route_constant_count",
     "mi355_route_constant_name",
@@ -121,6 +122,8 @@ def lib() -> ctypes.CDLL:
     for fn in (L.mi355_fp8_blockwise_mm_plan, L.mi355_int8_scaled_mm_plan):
         fn.argtypes = [i64, i64, i64, i32, ctypes.c_char_p, sz]
         fn.restype = i32
+    L.mi355_fp8_block_linear_plan.argtypes = [i64, i64, i64, ctypes.c_char_p, sz]
+    L.mi355_fp8_block_linear_plan.restype = i32
     L.mi355_per_token_quant_int8.argtypes = [vp, i32, vp, vp, i64, i64, vp]
     L.mi355_per_token_quant_int8.restype = i32
     L.mi355_per_token_quant_int8_sum.argtypes = [vp, i32, vp, vp, vp, i64, i64, vp]
@@ -169,6 +172,18 @@ def gemm_plan(kind: str, M: int, N: int, K: int, aligned: bool = True) -> dict:
     for item in buf.value.decode().split():
         k, v = item.split("=")
         out[k] = v if k == "kernel" else int(v)
+    return out
+
+
+def block_linear_plan(M: int, N: int, K: int) -> dict:
+    """Plan of the one-call block-FP8 linear: `gemm_plan`'s keys plus "quantizer": "fused" (the GEMM kernel quantizes the
+    tokens in its prologue) or "launch" (a quantizer launch in front of the GEMM)."""
+    buf = ctypes.create_string_buffer(256)
+    check(lib().mi355_fp8_block_linear_plan(M, N, K, buf, len(buf)))
+    out = {}
+    for item in buf.value.decode().split():
+        k, v = item.split("=")
+        out[k] = v if k in ("kernel", "quantizer") else int(v)
     return out
 
 

@@ -266,6 +266,7 @@ struct WavesplitShape {
   int waves, blocks_per_round;
 };
 WavesplitShape wavesplit_shape(int64_t K);
+bool wavesplit_two_tiles(bool is_fp8, int64_t M, int64_t N, int64_t K);  // 32 channels per workgroup instead of 16
 bool wavesplit_supported(int64_t M, int64_t N, int64_t K);
 int launch_fp8_wavesplit(GemmParams& p, hipStream_t stream, const char* what);
 int launch_int8_wavesplit(GemmParams& p, hipStream_t stream, const char* what);

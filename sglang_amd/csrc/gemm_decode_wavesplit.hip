@@ -9,12 +9,13 @@
 // straight into registers in MFMA operand layout (two 16-byte pieces per lane and block for the weight, two for the
 // tokens, which come from L2 after the first workgroups touched them), multiplies them as they arrive, and the W partial
 // tiles are added through LDS in wave order by wave 0, which applies the epilogue and stores.
-// No workspace, no second launch, N / 16 workgroups.
+// No workspace, no second launch, N / 16 workgroups - or N / 32 with two channel tiles each (FP8, where wavesplit_two_tiles
+// says so): a block's token fragment then serves both tiles, which halves what the tokens add to a workgroup's L2 traffic.
 //
 // A wave keeps a ring of KBW register slots: a slot is multiplied and requested again at once for the block KBW further
 // on, so KBW - 1 blocks stay in flight for as long as K lasts (requesting KBW blocks together and waiting for all of
 // them left nothing in flight between such rounds: K = 18432 -> N = 7168 at M = 1 30.4 -> 27.2 us, INT8 K = 14336 -> N = 4096
-// 15.6 -> 14.5 us; shapes of one or two turns are unchanged).  ~80-90 registers: five waves per SIMD.
+// 15.6 -> 14.5 us; shapes of one or two turns are unchanged).  ~80-90 registers: five waves per SIMD (two tiles: 118-128, four waves).
 // Blocks past the end of K are fetched from the last valid block and multiply a zero scale (FP8) or zeroed tokens (INT8).
 // Requires K % 128 == 0, N % 16 == 0, 16-byte aligned rows.  FP8 sums differ from the streaming kernel's in the order of
 // the additions only (per wave in K order, then over waves); INT8 results are exact either way.
@@ -36,16 +37,19 @@ __device__ __forceinline__ v8i as_v8i(const Frag& f) {
 // weight words one row per weight row: (kb >> 2) * sb_sk + n * sb_sn, constant over a 128-row block) and the MFMA applies
 // them itself (v_mfma_scale_f32_16x16x128_f8f6f4: the weight row's byte with the A operand, the token's with the B
 // operand), accumulating in place: no scale arithmetic, no expansion of the exponents to fp32 in front of the GEMM.
-template <bool IS_FP8, int W, int KBW, bool UE8M0 = false>
-__global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmParams p) {
+// CT: MFMA channel tiles per workgroup (16 or 32 channels).  With two, a block's token fragment is fetched once for both:
+// the tokens' share of what a workgroup pulls from L2 halves, which matters from about five tokens on.
+template <bool IS_FP8, int W, int KBW, bool UE8M0 = false, int CT = 1>
+__global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(CT == 2 ? 4 : 5))) void decode_wavesplit_kernel(const GemmParams p) {
   static_assert(IS_FP8 || !UE8M0, "exponent scales belong to the FP8 path");
+  static_assert(CT == 1 || CT == 2, "one or two channel tiles");
   using AccT = typename std::conditional<IS_FP8, float, int>::type;
   typedef AccT acc4 __attribute__((ext_vector_type(4)));
-  __shared__ acc4 red[W][64];
+  __shared__ acc4 red[W][CT][64];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l16 = lane & 15, q = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * (16 * CT);  // (a multiple of 32 for CT = 2: both tiles lie in one 128-channel scale block)
   const int tok = min(l16, p.M - 1);  // lanes past M repeat the last token; their results are never stored
   // operand layout of the 16 x 16 x 128 MFMA: lane (row l16, quarter q) holds bytes [16 q, +16) and [64 + 16 q, +16) of the row's block
   const uint8_t* wrow = p.b + (int64_t)(n0 + l16) * p.ldb + q * 16;
@@ -54,7 +58,9 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
   // wave-uniform, read through the constant address space: scalar loads, which the vector-memory counter does not see
   const cfloat_ptr sb_row = (cfloat_ptr)(IS_FP8 ? p.sb + (int64_t)(UE8M0 ? n0 : (n0 >> 7)) * p.sb_sn : nullptr);
 
-  acc4 acc = {0, 0, 0, 0};
+  acc4 acc[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) acc[c] = acc4{0, 0, 0, 0};
   // A ring of KBW register slots: the wave's i-th block is K block i * W + wave; slot j is multiplied and at once requested
   // again for the block KBW further on, so KBW - 1 blocks are always in flight (rounds of KBW blocks that are requested
   // together and awaited together leave the wave with nothing in flight between rounds).  Blocks past the end of K (the padding of the
@@ -63,8 +69,8 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
   // "everything but the newest block" and the ring runs empty once per turn.  A slot's registers are outputs of its request
   // and in-out operands of its wait, so no compiler-generated instruction touches them in between; vector loads complete in
   // order, so "at most (KBW - 1) blocks' loads outstanding" means the oldest slot has landed.
-  constexpr int LOADS = IS_FP8 ? 5 : 4;  // per block: two weight and two token fragments' halves, the token scale (word)
-  Frag wf[KBW], tf[KBW];
+  constexpr int LOADS = 2 * CT + 2 + (IS_FP8 ? 1 : 0);  // per block: the halves of the weight and token fragments, the token scale (word)
+  Frag wf[KBW][CT], tf[KBW];
   float sav[KBW], sbv[KBW];
   auto request = [&](int j, int i) {
     const int kc = min(i * W + wave, p.kb_total - 1);  // wave-uniform
@@ -73,9 +79,16 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
     asm volatile(
         "global_load_dwordx4 %0, %4, off\n\tglobal_load_dwordx4 %1, %4, off offset:64\n\t"
         "global_load_dwordx4 %2, %5, off\n\tglobal_load_dwordx4 %3, %5, off offset:64"
-        : "=&v"(wf[j].lo), "=&v"(wf[j].hi), "=&v"(tf[j].lo), "=&v"(tf[j].hi)
+        : "=&v"(wf[j][0].lo), "=&v"(wf[j][0].hi), "=&v"(tf[j].lo), "=&v"(tf[j].hi)
         : "v"(wp), "v"(tp)
         : "memory");
+    if constexpr (CT == 2) {
+      const uint8_t* wp1 = wp + 16 * p.ldb;  // the same block of the next sixteen weight rows
+      asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:64"
+                   : "=&v"(wf[j][1].lo), "=&v"(wf[j][1].hi)
+                   : "v"(wp1)
+                   : "memory");
+    }
     if constexpr (IS_FP8) {
       // fp32 scales: block kc's; packed exponents: the word that holds block kc's byte, kept as raw bits
       const float* sp = sa_row + (int64_t)(UE8M0 ? (kc >> 2) : kc) * p.sa_sk;
@@ -86,10 +99,14 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
   // waits until at most `behind` blocks requested after slot j's are still outstanding: slot j has landed
   auto await = [&](int j, int behind) {  // `behind` is a constant at every call; the switch folds away
 #define MI355_WS_AWAIT(NBLK)                                                                                                     \
-  if constexpr (IS_FP8)                                                                                                          \
-    asm volatile("s_waitcnt vmcnt(%5)" : "+v"(wf[j].lo), "+v"(wf[j].hi), "+v"(tf[j].lo), "+v"(tf[j].hi), "+v"(sav[j]) : "n"((NBLK)*LOADS)); \
+  if constexpr (IS_FP8 && CT == 2)                                                                                               \
+    asm volatile("s_waitcnt vmcnt(%7)" : "+v"(wf[j][0].lo), "+v"(wf[j][0].hi), "+v"(wf[j][1].lo), "+v"(wf[j][1].hi), "+v"(tf[j].lo), "+v"(tf[j].hi), "+v"(sav[j]) : "n"((NBLK)*LOADS)); \
+  else if constexpr (IS_FP8)                                                                                                     \
+    asm volatile("s_waitcnt vmcnt(%5)" : "+v"(wf[j][0].lo), "+v"(wf[j][0].hi), "+v"(tf[j].lo), "+v"(tf[j].hi), "+v"(sav[j]) : "n"((NBLK)*LOADS)); \
+  else if constexpr (CT == 2)                                                                                                    \
+    asm volatile("s_waitcnt vmcnt(%6)" : "+v"(wf[j][0].lo), "+v"(wf[j][0].hi), "+v"(wf[j][1].lo), "+v"(wf[j][1].hi), "+v"(tf[j].lo), "+v"(tf[j].hi) : "n"((NBLK)*LOADS)); \
   else                                                                                                                           \
-    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(wf[j].lo), "+v"(wf[j].hi), "+v"(tf[j].lo), "+v"(tf[j].hi) : "n"((NBLK)*LOADS))
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(wf[j][0].lo), "+v"(wf[j][0].hi), "+v"(tf[j].lo), "+v"(tf[j].hi) : "n"((NBLK)*LOADS))
     switch (behind) {
       case 3: MI355_WS_AWAIT(3); break;
       case 2: MI355_WS_AWAIT(2); break;
@@ -107,20 +124,29 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
       const u32x4 z = {0u, 0u, 0u, 0u};
       Frag t = tf[j];
       if (!valid) t.lo = z, t.hi = z;  // a block past the end of K multiplies zeros
-      acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(t), acc, 0, 0, 0, ea, 0, eb);
+#pragma unroll
+      for (int c = 0; c < CT; ++c)
+        acc[c] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j][c]), as_v8i(t), acc[c], 0, 0, 0, ea, 0, eb);
     } else if constexpr (IS_FP8) {
-      const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j]), as_v8i(tf[j]), v4f{0.f, 0.f, 0.f, 0.f}, 0, 0,
-                                                                        0, 0, 0, 0);
       const float sc = valid ? sav[j] * sbv[j] : 0.f;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[v] = fmaf(part[v], sc, acc[v]);
+      for (int c = 0; c < CT; ++c) {
+        const v4f part = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(as_v8i(wf[j][c]), as_v8i(tf[j]), v4f{0.f, 0.f, 0.f, 0.f}, 0,
+                                                                          0, 0, 0, 0, 0);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[c][v] = fmaf(part[v], sc, acc[c][v]);
+      }
     } else {
       const u32x4 z = {0u, 0u, 0u, 0u};
       const u32x4 tlo = valid ? tf[j].lo : z, thi = valid ? tf[j].hi : z;
-      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].lo.x, (int)wf[j].lo.y, (int)wf[j].lo.z, (int)wf[j].lo.w},
-                                                  v4i{(int)tlo.x, (int)tlo.y, (int)tlo.z, (int)tlo.w}, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)wf[j].hi.x, (int)wf[j].hi.y, (int)wf[j].hi.z, (int)wf[j].hi.w},
-                                                  v4i{(int)thi.x, (int)thi.y, (int)thi.z, (int)thi.w}, acc, 0, 0, 0);
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        const Frag& f = wf[j][c];
+        acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)f.lo.x, (int)f.lo.y, (int)f.lo.z, (int)f.lo.w},
+                                                       v4i{(int)tlo.x, (int)tlo.y, (int)tlo.z, (int)tlo.w}, acc[c], 0, 0, 0);
+        acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(v4i{(int)f.hi.x, (int)f.hi.y, (int)f.hi.z, (int)f.hi.w},
+                                                       v4i{(int)thi.x, (int)thi.y, (int)thi.z, (int)thi.w}, acc[c], 0, 0, 0);
+      }
     }
   };
   const int blocks = (p.kb_total + W * KBW - 1) / (W * KBW) * KBW;  // per wave, padded to whole turns of the ring
@@ -155,57 +181,68 @@ __global__ __launch_bounds__(64 * W) void decode_wavesplit_kernel(const GemmPara
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- add the W partial tiles in wave order
-  if (wave != 0) red[wave][lane] = acc;
+  if (wave != 0) {
+#pragma unroll
+    for (int c = 0; c < CT; ++c) red[wave][c][lane] = acc[c];
+  }
   __syncthreads();
   if (wave != 0) return;
 #pragma unroll
   for (int w = 1; w < W; ++w) {
-    const acc4 t = red[w][lane];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) acc[v] += t[v];
+    for (int c = 0; c < CT; ++c) {
+      const acc4 t = red[w][c][lane];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[c][v] += t[v];
+    }
   }
   if (l16 >= p.M) return;
-  // lane holds channels n0 + 4 q .. + 3 for token l16
-  const int n = n0 + 4 * q;
   const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-  if constexpr (IS_FP8) {
-    float r4[4] = {acc[0], acc[1], acc[2], acc[3]};
-    fp8_channel_epilogue(p, n, r4);
-    store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r4, 4, vec_ok);
-  } else if (p.out_dtype == MI355_I32) {
-    int* o = reinterpret_cast<int*>(p.out) + (int64_t)l16 * p.ldo + n;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) o[v] = acc[v];
-  } else {
-    const float sa_m = p.sa[l16];
-    float r4[4];
+  for (int c = 0; c < CT; ++c) {
+    // lane holds channels n .. n + 3 for token l16
+    const int n = n0 + 16 * c + 4 * q;
+    if constexpr (IS_FP8) {
+      float r4[4] = {acc[c][0], acc[c][1], acc[c][2], acc[c][3]};
+      fp8_channel_epilogue(p, n, r4);
+      store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r4, 4, vec_ok);
+    } else if (p.out_dtype == MI355_I32) {
+      int* o = reinterpret_cast<int*>(p.out) + (int64_t)l16 * p.ldo + n;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      // separately rounded multiply and add: the contract is mul, mul, add, not a fused multiply-add
-      float t = mul_rn((float)acc[v], mul_rn(p.sb[n + v], sa_m));
-      if (p.bias) {
-        const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
-        t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+      for (int v = 0; v < 4; ++v) o[v] = acc[c][v];
+    } else {
+      const float sa_m = p.sa[l16];
+      float r4[4];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        // separately rounded multiply and add: the contract is mul, mul, add, not a fused multiply-add
+        float t = mul_rn((float)acc[c][v], mul_rn(p.sb[n + v], sa_m));
+        if (p.bias) {
+          const uint32_t hb = reinterpret_cast<const uint16_t*>(p.bias)[n + v];
+          t = add_rn(t, (p.out_dtype == MI355_BF16) ? bf16_bits_to_f32(hb) : f16_bits_to_f32(hb));
+        }
+        r4[v] = t;
       }
-      r4[v] = t;
+      store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r4, 4, vec_ok);
     }
-    store_out4(p.out, p.out_dtype, (int64_t)l16 * p.ldo + n, r4, 4, vec_ok);
   }
 }
 
-template <bool IS_FP8, int W, int KBW, bool UE8M0 = false>
+template <bool IS_FP8, int W, int KBW, bool UE8M0 = false, int CT = 1>
 int launch_variant(const GemmParams& p, hipStream_t stream, const char* what) {
-  hipLaunchKernelGGL((decode_wavesplit_kernel<IS_FP8, W, KBW, UE8M0>), dim3((unsigned)(p.N / 16)), dim3(64 * W), 0, stream, p);
+  hipLaunchKernelGGL((decode_wavesplit_kernel<IS_FP8, W, KBW, UE8M0, CT>), dim3((unsigned)(p.N / (16 * CT))), dim3(64 * W), 0, stream, p);
   return check_launch(what);
 }
 
-template <bool IS_FP8>
+template <bool IS_FP8, bool UE8M0 = false>
 int launch_wavesplit(GemmParams& p, hipStream_t stream, const char* what) {
   p.splits = 1;
   p.tiles_m = 1;
   p.tiles_n = p.N / 16;
   const WavesplitShape s = wavesplit_shape(p.K);
-  return s.waves == 4 ? launch_variant<IS_FP8, 4, 4>(p, stream, what) : launch_variant<IS_FP8, 8, 4>(p, stream, what);
+  if (wavesplit_two_tiles(IS_FP8, p.M, p.N, p.K))
+    return s.waves == 4 ? launch_variant<IS_FP8, 4, 4, UE8M0, 2>(p, stream, what) : launch_variant<IS_FP8, 8, 4, UE8M0, 2>(p, stream, what);
+  return s.waves == 4 ? launch_variant<IS_FP8, 4, 4, UE8M0>(p, stream, what) : launch_variant<IS_FP8, 8, 4, UE8M0>(p, stream, what);
 }
 
 }  // namespace
@@ -220,14 +257,19 @@ WavesplitShape wavesplit_shape(int64_t K) {
   return (kb > 16 && kb <= 64) ? WavesplitShape{8, 4} : WavesplitShape{4, 4};
 }
 
+// Two channel tiles per workgroup (32 channels, FP8): where the tokens' share of the L2 traffic outweighs the halved number of
+// workgroups (the measurements stand beside the thresholds in route_constants.h).
+bool wavesplit_two_tiles(bool is_fp8, int64_t M, int64_t N, int64_t K) {
+  if (!is_fp8 || N % 32 != 0) return false;
+  const RouteConstants& rc = route_constants();
+  if ((double)(N / 32) < rc.wavesplit_two_tile_min_workgroups) return false;
+  return (double)M >= rc.wavesplit_two_tile_min_tokens || (double)((K + KSTEP - 1) / KSTEP) > rc.wavesplit_two_tile_long_k_blocks;
+}
+
 bool wavesplit_supported(int64_t M, int64_t N, int64_t K) { return M >= 1 && M <= 16 && K % KSTEP == 0 && N % 16 == 0; }
 
 int launch_fp8_wavesplit(GemmParams& p, hipStream_t stream, const char* what) { return launch_wavesplit<true>(p, stream, what); }
 int launch_int8_wavesplit(GemmParams& p, hipStream_t stream, const char* what) { return launch_wavesplit<false>(p, stream, what); }
-int launch_fp8_wavesplit_ue8m0(GemmParams& p, hipStream_t stream, const char* what) {
-  p.splits = 1, p.tiles_m = 1, p.tiles_n = p.N / 16;
-  const WavesplitShape s = wavesplit_shape(p.K);
-  return s.waves == 4 ? launch_variant<true, 4, 4, true>(p, stream, what) : launch_variant<true, 8, 4, true>(p, stream, what);
-}
+int launch_fp8_wavesplit_ue8m0(GemmParams& p, hipStream_t stream, const char* what) { return launch_wavesplit<true, true>(p, stream, what); }
 
 }  // namespace mi355

@@ -47,7 +47,9 @@ __shared__ __attribute__((aligned(1024))) uint8_t r_stage1[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_stage2[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_stage3[WAVES * SLICE];
 __shared__ __attribute__((aligned(1024))) uint8_t r_tok[KB_PER * TOK_BLOCK];
-__shared__ float r_sa[KB_PER * 16];  // token scales of the range when the kernel quantizes the tokens itself
+// The five arrays are exactly half of a CU's 160 KB, so two workgroups share a CU.  When the kernel quantizes the tokens itself,
+// the token scales of the range (KB_PER x 16 floats) pass through the head of every wave's slice of stage 3, which the ring
+// fills last: a wave reads its copy back before it requests its first block into that stage.
 
 // 16 zero bytes in global memory: the source of token chunks that lie past the end of K (short last range), so that
 // whatever weight block is refetched there multiplies zeros.  Not const: it must share the operands' address space.
@@ -213,7 +215,7 @@ __device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begi
     const bool valid = kb_begin + d < p.kb_total;  // blocks past the end of K: zero tokens, zero scale
     *reinterpret_cast<u32x2*>(tok + d * TOK_BLOCK + m * KSTEP + (((gl >> 1) ^ (m & 7)) << 4) + (gl & 1) * 8) =
         valid ? u32x2{(uint32_t)c0, (uint32_t)c1} : u32x2{0u, 0u};
-    if (gl == 0) sa_lds[d * 16 + m] = valid ? sc : 0.f;
+    if (gl < WAVES) sa_lds[gl * (SLICE / 4) + d * 16 + m] = valid ? sc : 0.f;  // one copy per wave slice (all 16 lanes hold sc)
   }
 }
 
@@ -265,7 +267,7 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
   issue_weights<false>(s, r_stage1, 1);
   issue_weights<false>(s, r_stage2, 2);
   if constexpr (QUANT) {
-    quantize_tokens<KB_PER>(p, kb_begin, raw_tok, r_tok, r_sa);
+    quantize_tokens<KB_PER>(p, kb_begin, raw_tok, r_tok, reinterpret_cast<float*>(r_stage3));
   } else {
 #pragma unroll
     for (int e = 0; e < 2 * KB_PER / WAVES; ++e) {  // 16 instructions of 8 rows x 128 B, 4 per wave
@@ -282,7 +284,8 @@ __global__ __launch_bounds__(64 * WAVES) void decode_kernel(const GemmParams p, 
   if constexpr (QUANT) {
     __syncthreads();  // codes and scales of the range are in LDS
 #pragma unroll
-    for (int d = 0; d < KB_PER; ++d) sa_r[d] = r_sa[d * 16 + l16];
+    for (int d = 0; d < KB_PER; ++d) sa_r[d] = reinterpret_cast<const float*>(r_stage3 + wave * SLICE)[d * 16 + l16];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read back before this wave's first request into stage 3
   } else if constexpr (IS_FP8) {
     const float* sa_row = p.sa + (int64_t)min(l16, p.M - 1) * p.sa_sm;
 #pragma unroll

@@ -420,7 +420,8 @@ bool wavesplit_preferred(bool is_fp8, int64_t M, int64_t N, int64_t K) {
   if ((double)(K / KSTEP) < rc.wavesplit_min_kblocks) return false;
   if (!is_fp8) return true;
   if ((double)N * (double)K <= rc.wavesplit_small_weight_bytes) return N / 16 >= NUM_CUS || (double)M <= rc.wavesplit_small_weight_max_tokens;
-  return (double)M <= rc.wavesplit_large_weight_max_tokens;
+  if (!wavesplit_two_tiles(true, M, N, K)) return (double)M <= rc.wavesplit_large_weight_max_tokens;
+  return (double)M <= ((double)(K / KSTEP) > rc.wavesplit_two_tile_long_k_blocks ? rc.wavesplit_long_k_max_tokens : rc.wavesplit_two_tile_max_tokens);
 }
 
 // `aligned`: both operand base pointers and row strides are multiples of 16 bytes and K % 16 == 0.
@@ -433,7 +434,7 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   const bool small_offsets = M * lda < (1ll << 32) && small_b;
   if (!fused_quant && wavesplit_supported(M, N, K) && aligned && small_b && wavesplit_preferred(is_fp8, M, N, K)) {
     const WavesplitShape ws = wavesplit_shape(K);
-    r.kernel = RK_WAVESPLIT, r.bm = 16, r.bn = 16, r.splits = 1;
+    r.kernel = RK_WAVESPLIT, r.bm = 16, r.bn = wavesplit_two_tiles(is_fp8, M, N, K) ? 32 : 16, r.splits = 1;
     r.kb_per_split = (int)((K + KSTEP - 1) / KSTEP);
     r.groups_per_wg = ws.waves;  // waves that share a workgroup's K
     return r;
@@ -622,7 +623,9 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
     "dma3_latency_us[int8][unused]", "dma3_latency_us[int8][unused2]",
     "dma3_busy_chip_factor", "dma3_long_row_factor", "dma3_split_fixed_us", "dma3_split_per_split_us", "dma3_min_efficiency",
     "dma3_small_tile_factor", "wavesplit_min_kblocks", "wavesplit_small_weight_bytes", "wavesplit_small_weight_max_tokens",
-    "wavesplit_large_weight_max_tokens"};
+    "wavesplit_large_weight_max_tokens", "wavesplit_two_tile_min_workgroups", "wavesplit_two_tile_min_tokens",
+    "wavesplit_two_tile_long_k_blocks", "wavesplit_two_tile_max_tokens", "wavesplit_long_k_max_tokens",
+    "fused_quant_long_k_blocks", "fused_quant_short_k_blocks", "fused_quant_short_k_max_tokens"};
 
 int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len, const char* what) {
   clear_error();
@@ -950,6 +953,17 @@ extern "C" int mi355_fp8_scaled_mm(const void* a, const void* b, const float* sa
 
 namespace {
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+// One-call linear where the streaming decode kernel can quantize the tokens itself: is that faster than a quantizer launch
+// plus the kernel the GEMM alone would take?  Always where that kernel is the streaming one (a launch saved, nothing else
+// changes); against the wave-split kernel by measurement.
+bool fused_quant_preferred(int64_t M, int64_t N, int64_t K, int64_t ldw) {
+  if (choose_route(true, M, N, K, K, ldw, true).kernel != RK_WAVESPLIT) return true;
+  const RouteConstants& rc = route_constants();
+  const double kb = (double)(K / KSTEP);
+  if (kb > rc.fused_quant_long_k_blocks) return false;
+  return !(kb <= rc.fused_quant_short_k_blocks && (double)M > rc.fused_quant_short_k_max_tokens);
+}
 }  // namespace
 
 extern "C" size_t mi355_fp8_block_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
@@ -982,9 +996,10 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
   float* sa = reinterpret_cast<float*>(q + q_bytes);
   const int64_t pitch = (M + 3) & ~3ll;
   const size_t sa_bytes = align256((size_t)pitch * (size_t)(K / KSTEP) * 4u);
-  // Decode sizes: the GEMM kernel quantizes the tokens of each K range itself (same arithmetic), no quantizer launch.
-  if (x_dtype != MI355_F32 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && ldw % 16 == 0 &&
-      choose_route(true, M, N, K, K, ldw, true, true).kernel == RK_DECODE) {
+  // Decode sizes: the GEMM kernel quantizes the tokens of each K range itself (same arithmetic), no quantizer launch -
+  // except where a quantizer launch in front of the wave-split kernel is measured faster (route_constants.h).
+  const bool ptr_ok = x_dtype != MI355_F32 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && ldw % 16 == 0;
+  if (ptr_ok && choose_route(true, M, N, K, K, ldw, true, true).kernel == RK_DECODE && fused_quant_preferred(M, N, K, ldw)) {
     GemmParams p;
     bool empty;
     // a / sa are not read by the kernel in this mode; they only have to satisfy the checks
@@ -1004,6 +1019,21 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
   if (rc != MI355_OK || empty) return rc;
   p.bias = bias;
   return run_gemm<true>(p, q + q_bytes + sa_bytes, workspace_bytes_given - q_bytes - sa_bytes, static_cast<hipStream_t>(stream), what);
+}
+
+extern "C" int mi355_fp8_block_linear_plan(int64_t M, int64_t N, int64_t K, char* buf, size_t buf_len) {
+  const char* what = "mi355_fp8_block_linear_plan";
+  clear_error();
+  MI355_REQUIRE(buf != nullptr && buf_len > 0, MI355_ERR_INVALID_ARGUMENT, "%s: no buffer", what);
+  MI355_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && K % KSTEP == 0,
+                MI355_ERR_INVALID_ARGUMENT, "%s: shape out of range (K must be a multiple of 128)", what);
+  const bool fused = choose_route(true, M, N, K, K, K, true, true).kernel == RK_DECODE && fused_quant_preferred(M, N, K, K);
+  const Route r = choose_route(true, M, N, K, K, K, true, fused);
+  const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d quantizer=%s",
+                         ROUTE_NAMES[r.kernel], r.bm, r.bn, r.splits, r.kb_per_split, r.groups_per_wg, (int)r.aligned,
+                         fused ? "fused" : "launch");
+  MI355_REQUIRE(n > 0 && (size_t)n < buf_len, MI355_ERR_INVALID_ARGUMENT, "%s: buffer of %zu bytes is too small", what, buf_len);
+  return MI355_OK;
 }
 
 extern "C" size_t mi355_int8_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) {

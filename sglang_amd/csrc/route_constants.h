@@ -47,7 +47,27 @@ struct RouteConstants {
   double wavesplit_min_kblocks = 8.0;              // shorter K: one block per wave, the streaming kernel's wide tiles win
   double wavesplit_small_weight_bytes = 32e6;      // FP8: up to here the second launch it saves outweighs the token traffic ...
   double wavesplit_small_weight_max_tokens = 8.0;  // ... for this many tokens, or for any M <= 16 once N / 16 fills the CUs
-  double wavesplit_large_weight_max_tokens = 4.0;  // FP8, larger weights: the token traffic decides
+  double wavesplit_large_weight_max_tokens = 4.0;  // FP8, larger weights, one channel tile per workgroup: the token traffic decides
+  // ---- two channel tiles (32 channels) per workgroup: a block's token fragment serves both, so the tokens' share of the
+  //      L2 traffic halves, at half the workgroups.  FP8, median launch, us, one tile / two tiles / streaming kernel:
+  //      7168->36864: M=1 48.0/50.2/51.5, 2 49.8/50.8/53.0, 3 52.0/51.4/54.0, 4 54.3/52.2/54.4, 8 62.6/54.3/57.1, 12 69.7/57.8/58.1,
+  //      16 74.0/61.5/60.3;  18432->7168: M=1 27.2/25.9/30.5, 4 29.8/26.2/31.5, 8 33.2/27.3/32.1, 16 38.3/30.0/33.4;  1536->24576:
+  //      M=1 11.3/11.0, 8 13.2/11.8/13.6;  7168->8192: M=1 14.5/14.7, 3 15.0/14.8, 8 17.0/15.2/17.7;  4096->14336: M=1 15.6/15.2,
+  //      8 17.6/16.0/19.6;  7168->4096 (128 workgroups of two tiles): M=4 9.8/13.3, 16 11.7/15.3;  7168->2048: 9.8/13.3.
+  //      INT8 stays on one tile: 4096->28672 M=4 25.4/29.1, 8 27.4/29.6, 16 32.8/31.0; 14336->4096 M=4 14.8/21.3; 4096->6144 10.7/10.4.
+  double wavesplit_two_tile_min_workgroups = 200.0;  // N / 32 from here on
+  double wavesplit_two_tile_min_tokens = 3.0;        // ... and from this many tokens on,
+  double wavesplit_two_tile_long_k_blocks = 64.0;    // ... or at any token count once K has more blocks than this (four-wave workgroups)
+  double wavesplit_two_tile_max_tokens = 12.0;       // FP8, larger weights, two tiles: up to here against the streaming kernel,
+  double wavesplit_long_k_max_tokens = 16.0;         // ... and up to here beyond wavesplit_two_tile_long_k_blocks
+  // ---- one-call linear at decode sizes: the streaming kernel with the quantizer in its prologue (one launch) against a
+  //      quantizer launch + the wave-split kernel, where that is the GEMM's plan.  FP8, median call, us, fused / two launches:
+  //      7168->36864: M=1 52.0/52.3, 4 54.6/56.2, 8 58.3/58.6;  18432->7168: M=1 30.8/30.1, 4 32.1/30.4, 8 33.6/31.6, 16 36.6/34.8;
+  //      1536->24576: M=1 13.5/15.5, 4 14.0/15.7, 8 15.1/16.3;  7168->4096: M=1 11.9/13.7, 8 13.5/14.5, 16 16.0/15.9;
+  //      7168->2048: M=1 10.3/13.2, 8 12.2/14.5;  2048->7168: M=1 10.5/11.5, 4 10.9/11.9, 8 12.2/12.0, 16 14.4/11.8.
+  double fused_quant_long_k_blocks = 64.0;       // beyond this many K blocks the two launches win
+  double fused_quant_short_k_blocks = 16.0;      // up to this many K blocks they win too,
+  double fused_quant_short_k_max_tokens = 8.0;   // ... above this many tokens
 };
 constexpr int ROUTE_CONSTANT_COUNT = sizeof(RouteConstants) / sizeof(double);
 static_assert(sizeof(RouteConstants) == ROUTE_CONSTANT_COUNT * sizeof(double), "the table is read as an array of doubles");

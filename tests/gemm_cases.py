@@ -3,7 +3,8 @@ parity tests, plus the full-size shapes of the benchmark configurations.
 
 A *variant* is one compiled code path: the kernel, its token-tile height, whether it writes split-K partial sums,
 for the decode kernel how many 128-channel groups a workgroup walks, for the wave-split decode kernel how many waves
-share a workgroup's K and whether a wave's share takes one turn of its four-slot register ring ("one_round") or several, for the large-M kernels whether K ends on a
+share a workgroup's K, whether a wave's share takes one turn of its four-slot register ring ("one_round") or several and
+whether the workgroup owns one 16-channel tile or two, for the large-M kernels whether K ends on a
 128-byte block.  `variant_of` maps a plan (sglang_amd._lib.gemm_plan) to such a key.
 """
 
@@ -11,12 +12,16 @@ share a workgroup's K and whether a wave's share takes one turn of its four-slot
 FP8_ROUTE_SHAPES = [
     # decode kernel (M <= 16, K % 128 == 0, N % 128 == 0): whole-K and split, 1 / 2 / 3+ channel groups per workgroup,
     # an uneven last workgroup (16640 = 130 groups), short last K ranges (4480 = 35 blocks, 2176 = 17 blocks)
-    (1, 128, 128), (3, 256, 512), (1, 512, 7168), (16, 2048, 7168), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432),
-    (7, 33280, 4096), (5, 66048, 512), (2, 133120, 384),
+    (1, 128, 128), (3, 256, 512), (16, 2048, 7168), (13, 18432, 7168), (13, 36864, 7168), (16, 16640, 4480), (15, 33280, 2176),
+    (5, 66048, 512), (2, 133120, 384),
     # wave-split decode kernel (few tokens or a small weight, K of at least 8 blocks; N % 16 == 0 is enough): 8 waves with one
     # round (K = 4096) and two (K = 7168, 4480 = 35 blocks: a ragged second round), 4 waves with many rounds (K = 18432) and
     # with one (N % 128 != 0 at short K), ragged N (576, 1088), every token count class
-    (1, 512, 4096), (4, 1536, 7168), (16, 7168, 2048), (2, 36864, 7168), (1, 512, 18432), (12, 48, 1152),
+    (1, 512, 4096), (4, 1536, 7168), (2, 7168, 2048), (2, 36864, 7168), (1, 512, 18432), (12, 48, 1152), (1, 512, 7168), (1, 16640, 4480),
+    # ... and two channel tiles per workgroup (N / 32 >= 200 and three tokens or more, or K beyond 64 blocks): both wave counts,
+    # one round and several, an uneven split of the K blocks over the waves (2176 = 17 blocks), N % 32 == 0 but N % 128 != 0
+    (16, 7168, 2048), (9, 33280, 2176), (7, 33280, 4096), (12, 36864, 7168), (6, 16640, 4480), (1, 7168, 18432), (16, 7168, 18432),
+    (5, 6432, 1280),
     (5, 48, 128), (16, 16, 256),  # a single K block (three of the four waves have nothing to add), a single workgroup
     # three-stage mid-M kernel: 64 / 128 token tiles x 256 / 192 / 128 channel tiles, whole-K and split, ragged M, K blocks per
     # range = 1, 2, 0 mod 3
@@ -44,6 +49,8 @@ FP8_REQUIRED_VARIANTS = {
     ("decode", "split", "gpw1"), ("decode", "split", "gpw2"), ("decode", "split", "gpw3+"),
     ("decode_wavesplit", "w4", "one_round"), ("decode_wavesplit", "w4", "rounds"), ("decode_wavesplit", "w8", "one_round"),
     ("decode_wavesplit", "w8", "rounds"),
+    ("decode_wavesplit", "w4", "one_round", "two_tiles"), ("decode_wavesplit", "w4", "rounds", "two_tiles"),
+    ("decode_wavesplit", "w8", "one_round", "two_tiles"), ("decode_wavesplit", "w8", "rounds", "two_tiles"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
     ("dma3", 64, "whole", "bn128"), ("dma3", 64, "split", "bn128"), ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"),
     ("dma3", 64, "whole", "bn192"), ("dma3", 64, "split", "bn192"), ("dma3", 128, "whole", "bn192"), ("dma3", 128, "split", "bn192"),
@@ -103,7 +110,8 @@ def variant_of(plan: dict, K: int):
         return (k, sp, f"gpw{g}" if g < 3 else "gpw3+")
     if k == "decode_wavesplit":  # waves per workgroup; one turn of the wave's four-slot ring or several
         waves = plan["groups_per_wg"]
-        return (k, f"w{waves}", "rounds" if -(-K // 128) > 4 * waves else "one_round")
+        key = (k, f"w{waves}", "rounds" if -(-K // 128) > 4 * waves else "one_round")
+        return key + ("two_tiles",) if plan["bn"] == 32 else key  # 32 channels per workgroup (FP8) or 16
     if k == "pingpong128":
         return (k, sp)
     if k == "dma3":

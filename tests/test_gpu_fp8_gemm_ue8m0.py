@@ -19,9 +19,11 @@ FP8 = torch.float8_e4m3fn
 # (M, N, K): two-phase kernel with hardware scales (>= 256 tiles of 256 x 256): K of 4, 9 and 5 blocks; ragged M;
 # then decode, mid-M, generic routes through the unpack step
 # decode sizes on the wave-split kernel, which also lets the MFMA apply the scales (8 and 4 waves, a ragged last round and a
-# partly used last exponent word: K = 4480 is 35 blocks; N = 576 is not a multiple of 128)
+# partly used last exponent word: K = 4480 is 35 blocks; N = 576 is not a multiple of 128), then the same kernel with two
+# channel tiles per workgroup (8 waves with one round and two, 4 waves with one round and many)
 SHAPES = [(4096, 4352, 512), (4096, 4352, 1152), (4000, 4352, 640), (4, 512, 1024), (16, 2048, 7168), (200, 16384, 2048),
           (50, 384, 512), (1500, 640, 1024), (2, 2048, 7168), (3, 1536, 4480), (1, 1024, 18432), (5, 576, 2048),
+          (7, 6432, 4096), (12, 18432, 7168), (6, 16640, 4480), (5, 36864, 1280), (1, 7168, 18432), (16, 7168, 36864),
           (3990, 4224, 640)]  # two-phase kernel: a last token tile with 6 of 16 rows and half a last channel tile (guarded stores)
 
 
@@ -130,8 +132,8 @@ def test_ue8m0_mid_m_kernel_against_oracle(gpu, oracle, M, N, K):
 
 # the streaming decode kernel: one K range and several, the last range short (K blocks not a multiple of 8), one to four
 # bytes used in the last exponent word, token counts below and at the 16 rows of the MFMA tile (rows past M repeat the last token)
-DECODE = [(8, 256, 512), (4, 4352, 512), (5, 7168, 36864), (16, 7168, 36864), (5, 18432, 7168), (12, 18432, 7168), (9, 3072, 1536),
-          (6, 36864, 1280), (11, 16384, 2304), (15, 65536, 640), (16, 65536, 1152), (13, 7168, 18432), (8, 4352, 128)]
+DECODE = [(8, 256, 512), (4, 4352, 512), (5, 4096, 36864), (16, 4096, 36864), (13, 18432, 7168), (15, 18432, 7168), (9, 3072, 1536),
+          (14, 36864, 1280), (14, 16384, 2304), (15, 65536, 640), (16, 65536, 1152), (13, 4096, 18432), (8, 4352, 128)]
 
 
 def test_decode_shapes_reach_the_streaming_kernel():
@@ -184,7 +186,7 @@ def test_ue8m0_mid_m_exact_integers(gpu, oracle, M, N, K):
     _exact_integer_case(gpu, oracle, M, N, K)  # split and unsplit mid-M plans
 
 
-@pytest.mark.parametrize("M,N,K", [(8, 4352, 512), (5, 18432, 7168), (16, 2048, 7168), (11, 16384, 2304), (5, 7168, 36864)])
+@pytest.mark.parametrize("M,N,K", [(8, 4352, 512), (13, 18432, 7168), (16, 2048, 7168), (14, 16384, 2304), (5, 4096, 36864)])
 def test_ue8m0_decode_exact_integers(gpu, oracle, M, N, K):
     from sglang_amd import _lib
 

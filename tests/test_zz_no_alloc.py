@@ -40,8 +40,8 @@ def test_noalloc_matches_workspace_entry_point_twice_in_a_row(gpu, oracle):
     from sglang_amd import _lib
 
     L = _lib.lib()
-    # split-K decode (18 splits, 4.1 MB of partials), then a smaller split problem, then mid-M split, then one without split
-    shapes = [(8, 7168, 18432), (12, 2048, 7168), (48, 7168, 18432), (300, 1024, 512)]
+    # split-K decode (18 splits, 2.4 MB of partials), then a smaller split problem, then mid-M split, then one without split
+    shapes = [(8, 4096, 18432), (12, 2048, 7168), (48, 7168, 18432), (300, 1024, 512)]
     plans = [_lib.gemm_plan("fp8", *s) for s in shapes]
     assert plans[0]["splits"] > 1 and plans[1]["splits"] > 1 and plans[2]["splits"] > 1 and plans[3]["splits"] == 1
     problems = [_problem(*s, seed=i + 1, gpu=gpu) for i, s in enumerate(shapes)]
