@@ -246,7 +246,8 @@ int mi355_int8_scaled_mm(const void* a, const void* b, const float* sa, const fl
  * here the choice is observable so that tests can prove every kernel variant is reached.
  *   aligned  nonzero if both operand base pointers and row strides are multiples of 16 bytes (rows are assumed dense)
  *   buf      receives a NUL-terminated "key=value ..." line:
- *            kernel=decode|dma3|pingpong|pipelined|generic bm= bn= splits= kb_per_split= groups_per_wg= aligned=
+ *            kernel=decode|decode_wavesplit|dma3|pingpong|pingpong128|pipelined|generic bm= bn= splits= kb_per_split=
+ *            groups_per_wg= aligned= stages=   (stages: LDS stages of the mid-M kernel's pipeline, 0 for the other kernels)
  * Launches nothing and touches no device state.
  */
 int mi355_fp8_blockwise_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len);

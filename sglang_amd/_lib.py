@@ -164,7 +164,7 @@ def lib() -> ctypes.CDLL:
 
 def gemm_plan(kind: str, M: int, N: int, K: int, aligned: bool = True) -> dict:
     """Kernel and tiling the library would use for an FP8 (`kind` "fp8") or INT8 ("int8") GEMM of this shape:
-    {"kernel": str, "bm": int, "bn": int, "splits": int, "kb_per_split": int, "groups_per_wg": int, "aligned": int}."""
+    {"kernel": str, "bm": int, "bn": int, "splits": int, "kb_per_split": int, "groups_per_wg": int, "aligned": int, "stages": int}."""
     fn = {"fp8": lib().mi355_fp8_blockwise_mm_plan, "int8": lib().mi355_int8_scaled_mm_plan}[kind]
     buf = ctypes.create_string_buffer(256)
     check(fn(M, N, K, int(aligned), buf, len(buf)))

@@ -190,6 +190,7 @@ struct Dma3Plan {
   double time_us;     // modelled duration of the chosen plan
 };
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8 = false);
+int dma3_stages(int bm, int bn, int64_t workgroups);  // LDS stages the FP8 kernel runs such a launch with (3, 4 or 6)
 int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);  // bm: 64 or 128, bn: 128, 192 or 256, from dma3_plan()
 // The same for packed UE8M0 scales on both operands (p.sa / p.sb point to the words, p.sa_sk / p.sb_sn / p.sb_sk are word
 // strides; token words M-major with a pitch that is a multiple of four words), applied by the MFMA.

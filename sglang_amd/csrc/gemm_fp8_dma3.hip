@@ -1,5 +1,5 @@
 // Blockwise-scaled FP8 GEMM for gfx950 with short token tiles: (64 or 128) x (256, 192 or 128) macro tile, 8 waves (two per SIMD),
-// THREE LDS stages.
+// THREE LDS stages (six for 64 x 128 tiles and four for 64 x 192 / 128 x 128 when a workgroup has a CU to itself).
 //
 // For 16 < M <= 1024 a linear layer is between weight streaming and MFMA-bound; prefill shapes with few output channels
 // (M = 4096, N = 576 or 1536) do not give 256 x 256 tiles enough workgroups.  Both take this kernel.  The tile is short in the token dimension
@@ -170,22 +170,22 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
   }
 }
 
-// Everything but the youngest block's loads has landed; then the workgroup barrier.  Instructions, see the file comment.
+// Everything but the YOUNGER youngest loads has landed; then the workgroup barrier.  Instructions, see the file comment.
 template <int YOUNGER>
 __device__ __forceinline__ void wait_and_barrier() {
-  static_assert(YOUNGER >= 4 && YOUNGER <= 7, "LOADS + 1 = (BM + BN) / 64 + 1");
-  if constexpr (YOUNGER == 7) asm volatile("s_waitcnt vmcnt(7)\n\ts_barrier" ::: "memory");
-  else if constexpr (YOUNGER == 6) asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
-  else if constexpr (YOUNGER == 5) asm volatile("s_waitcnt vmcnt(5)\n\ts_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
+  static_assert(YOUNGER >= 4 && YOUNGER <= 28, "(stages - 2) x (LOADS + 1), LOADS + 1 = (BM + BN) / 64 + 1");
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(YOUNGER) : "memory");
 }
 
 // One BM x 256 output tile at (m0, n0), K blocks of split `split`, by the whole workgroup.
 // UE8M0: p.sa / p.sb point to packed exponent words (int32): token word (m, kw) at sa[kw * sa_sk + m], channel word (n, kw)
 // at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb; the MFMA applies them.
-template <int BM, bool SPLIT, int BN = T_BN, bool UE8M0 = false>
+// S: LDS stages (S - 1 K blocks in flight).  Three everywhere; more where the tile is small enough for them to fit and the
+// launch has at most one workgroup per CU, so that nothing else would use the LDS.
+template <int BM, bool SPLIT, int BN = T_BN, bool UE8M0 = false, int S = 3>
 __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, int split) {
   static_assert(BN == 128 || BN == 192 || BN == 256, "channel tile");
+  static_assert(S >= 3 && S * ((BM + BN) * KSTEP + BM * 4) <= 160 * 1024, "the stages must fit the CU's LDS");
   constexpr int WM = BM / 2, MT = WM / 16, T_WN = BN / 4, T_NT = T_WN / 16, LOADS = Dma3State<BM, BN>::LOADS;
   constexpr bool INTERLEAVED = Dma3State<BM, BN>::INTERLEAVED;
   constexpr int SB = Dma3State<BM, BN>::SB;
@@ -234,14 +234,11 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   }
   s.sb_sk = p.sb_sk;
 
-  // three stages: tiles (rows 0..BM-1 tokens, BM.. channels) and the tile's BM token scales, sized per tile shape: a
-  // 64 x 128 tile takes 73.5 KB, so two such workgroups share a CU's 160 KB
-  __shared__ __attribute__((aligned(1024))) uint8_t t_stage0[(BM + BN) * KSTEP];
-  __shared__ __attribute__((aligned(1024))) uint8_t t_stage1[(BM + BN) * KSTEP];
-  __shared__ __attribute__((aligned(1024))) uint8_t t_stage2[(BM + BN) * KSTEP];
-  __shared__ __attribute__((aligned(256))) float t_scale0[BM];
-  __shared__ __attribute__((aligned(256))) float t_scale1[BM];
-  __shared__ __attribute__((aligned(256))) float t_scale2[BM];
+  // the stages: tiles (rows 0..BM-1 tokens, BM.. channels) and the tile's BM token scales, sized per tile shape: three
+  // stages of a 64 x 128 tile take 73.5 KB, so two such workgroups share a CU's 160 KB
+  __shared__ __attribute__((aligned(1024))) uint8_t t_stage[S][(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(256))) float t_scale[S][BM];
+  constexpr int YOUNGER = (S - 2) * (LOADS + 1);  // loads that may still be in flight when the next block is due
 
   float acc[T_NT][MT][4];
 #pragma unroll
@@ -251,40 +248,39 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
 
-  // ---- prologue: blocks 0 and 1 (clamped) into stages 0 and 1
+  // ---- prologue: blocks 0 .. S-2 (clamped) into stages 0 .. S-2
 #pragma unroll
-  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN, UE8M0>(s, i, t_stage0, t_scale0, kb_begin);
+  for (int b = 0; b < S - 1; ++b)
 #pragma unroll
-  for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN, UE8M0>(s, i, t_stage1, t_scale1, kb_begin + 1);
-  wait_and_barrier<LOADS + 1>();  // block 0 has landed everywhere
+    for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN, UE8M0>(s, i, t_stage[b], t_scale[b], kb_begin + b);
+  wait_and_barrier<YOUNGER>();  // block 0 has landed everywhere
 
-  // ---- three blocks per trip over the three stages; iteration k multiplies block k, requests block k + 2
+  // ---- S blocks per trip over the S stages; iteration k multiplies block k and requests block k + S - 1 into the stage
+  //      that iteration k - 1 read
   auto sb_of = [&](int kb, float (&v)[SB]) {
 #pragma unroll
     for (int b = 0; b < SB; ++b) v[b] = s.sb_ptr[b][(int64_t)(UE8M0 ? kb >> 2 : kb) * s.sb_sk];
   };
   int k = 0;
-  for (; k + 2 < nkb; k += 3) {
-    float sb0[SB], sb1[SB], sb2[SB];
-    sb_of(kb_begin + k, sb0);
-    sb_of(kb_begin + k + 1, sb1);
-    sb_of(kb_begin + k + 2, sb2);
-    k_block<BM, BN, UE8M0>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2, kb_begin + k);
-    wait_and_barrier<LOADS + 1>();
-    k_block<BM, BN, UE8M0>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3, kb_begin + k + 1);
-    wait_and_barrier<LOADS + 1>();
-    k_block<BM, BN, UE8M0>(s, t_stage2, t_scale2, sb2, acc, t_stage1, t_scale1, kb_begin + k + 4, kb_begin + k + 2);
-    wait_and_barrier<LOADS + 1>();
+  for (; k + S - 1 < nkb; k += S) {
+    float sbv[S][SB];
+#pragma unroll
+    for (int u = 0; u < S; ++u) sb_of(kb_begin + k + u, sbv[u]);
+#pragma unroll
+    for (int u = 0; u < S; ++u) {
+      k_block<BM, BN, UE8M0>(s, t_stage[u], t_scale[u], sbv[u], acc, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S],
+                             kb_begin + k + u + S - 1, kb_begin + k + u);
+      wait_and_barrier<YOUNGER>();
+    }
   }
-  if (k < nkb) {  // one or two blocks left, in stages 0 and 1
-    float sb0[SB];
-    sb_of(kb_begin + k, sb0);
-    k_block<BM, BN, UE8M0>(s, t_stage0, t_scale0, sb0, acc, t_stage2, t_scale2, kb_begin + k + 2, kb_begin + k);
-    wait_and_barrier<LOADS + 1>();
-    if (k + 1 < nkb) {
-      float sb1[SB];
-      sb_of(kb_begin + k + 1, sb1);
-      k_block<BM, BN, UE8M0>(s, t_stage1, t_scale1, sb1, acc, t_stage0, t_scale0, kb_begin + k + 3, kb_begin + k + 1);
+#pragma unroll
+  for (int u = 0; u < S - 1; ++u) {  // up to S - 1 blocks left, in stages 0 ..
+    if (k + u < nkb) {
+      float sbl[SB];
+      sb_of(kb_begin + k + u, sbl);
+      k_block<BM, BN, UE8M0>(s, t_stage[u], t_scale[u], sbl, acc, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S],
+                             kb_begin + k + u + S - 1, kb_begin + k + u);
+      if (k + u + 1 < nkb) wait_and_barrier<YOUNGER>();
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
@@ -313,10 +309,10 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   }
 }
 
-template <int BM, bool SPLIT, int BN, bool UE8M0 = false>
+template <int BM, bool SPLIT, int BN, bool UE8M0 = false, int S = 3>
 __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmParams p) {
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
-  dma3_tile<BM, SPLIT, BN, UE8M0>(p, tc.tile_m * BM, tc.tile_n * BN, tc.split);
+  dma3_tile<BM, SPLIT, BN, UE8M0, S>(p, tc.tile_m * BM, tc.tile_n * BN, tc.split);
 }
 
 // Grouped problems (see GroupedParams): the workgroup's token tile comes from the table the plan kernel wrote, the
@@ -329,15 +325,29 @@ __global__ __launch_bounds__(T_THREADS) void fp8_grouped_dma3_kernel(const Group
   dma3_tile<BM, false>(p, m0, tile_n * T_BN, 0);
 }
 
+// More than three stages pay only where a workgroup has its CU to itself (otherwise two workgroups of three stages keep as
+// many blocks in flight).  Measured, us, three stages / more: K=7168 -> N=576 at M=2048 29.0 / 27.0, K=4096 -> N=14336 at
+// M=48 24.5 / 23.1, K=7168 -> N=4096 at M=512 25.8 / 24.6, K=18432 -> N=7168 at M=32 33.7 / 32.8, at M=64 37.9 / 37.3;
+// no change (within 0.3 us) for ten other shapes: these tiles are bound by the step's own chain of LDS reads, MFMAs and the
+// barrier more than by the latency of the loads.
+bool dma3_deep_pipeline(int64_t workgroups) { return workgroups <= NUM_CUS; }
+constexpr int deep_stages(int bm, int bn) { return bm + bn == 192 ? 6 : bm + bn == 256 ? 4 : 3; }  // 6 x 24 KB, 4 x 32 KB
+
 template <int BM, int BN, bool UE8M0 = false>
 int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits));
-  if (p.splits > 1)
-    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
-  else
-    hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
+  // more stages where they fit and each workgroup has a CU to itself
+  constexpr int DEEP = deep_stages(BM, BN);
+  const bool deep = DEEP > 3 && dma3_deep_pipeline((int64_t)p.tiles_m * p.tiles_n * p.splits);
+  if (p.splits > 1) {
+    if (deep) hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0, DEEP>), grid, dim3(T_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
+  } else {
+    if (deep) hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0, DEEP>), grid, dim3(T_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
+  }
   return check_launch(what);
 }
 
@@ -395,6 +405,8 @@ double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int bn, int
   return t;
 }
 }  // namespace
+
+int dma3_stages(int bm, int bn, int64_t workgroups) { return dma3_deep_pipeline(workgroups) ? deep_stages(bm, bn) : 3; }
 
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8) {
   Dma3Plan pl;

@@ -627,14 +627,22 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
     "wavesplit_two_tile_long_k_blocks", "wavesplit_two_tile_max_tokens", "wavesplit_long_k_max_tokens",
     "fused_quant_long_k_blocks", "fused_quant_short_k_blocks", "fused_quant_short_k_max_tokens"};
 
+// LDS stages of the mid-M kernel's pipeline for this plan (0 for the other kernels, whose depth is fixed).
+int route_stages(bool is_fp8, const Route& r, int64_t M, int64_t N) {
+  if (r.kernel != RK_DMA3) return 0;
+  const int64_t workgroups = ((M + r.bm - 1) / r.bm) * ((N + r.bn - 1) / r.bn) * r.splits;
+  return is_fp8 ? dma3_stages(r.bm, r.bn, workgroups) : 3;
+}
+
 int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len, const char* what) {
   clear_error();
   MI355_REQUIRE(buf != nullptr && buf_len > 0, MI355_ERR_INVALID_ARGUMENT, "%s: no buffer", what);
   MI355_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31),
                 MI355_ERR_INVALID_ARGUMENT, "%s: shape out of range", what);
   const Route r = choose_route(is_fp8, M, N, K, K, K, aligned != 0 && K % 16 == 0);
-  const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d",
-                         ROUTE_NAMES[r.kernel], r.bm, r.bn, r.splits, r.kb_per_split, r.groups_per_wg, (int)r.aligned);
+  const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d stages=%d",
+                         ROUTE_NAMES[r.kernel], r.bm, r.bn, r.splits, r.kb_per_split, r.groups_per_wg, (int)r.aligned,
+                         route_stages(is_fp8, r, M, N));
   MI355_REQUIRE(n > 0 && (size_t)n < buf_len, MI355_ERR_INVALID_ARGUMENT, "%s: buffer of %zu bytes is too small", what,
                 buf_len);
   return MI355_OK;
@@ -1029,9 +1037,9 @@ extern "C" int mi355_fp8_block_linear_plan(int64_t M, int64_t N, int64_t K, char
                 MI355_ERR_INVALID_ARGUMENT, "%s: shape out of range (K must be a multiple of 128)", what);
   const bool fused = choose_route(true, M, N, K, K, K, true, true).kernel == RK_DECODE && fused_quant_preferred(M, N, K, K);
   const Route r = choose_route(true, M, N, K, K, K, true, fused);
-  const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d quantizer=%s",
+  const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d stages=%d quantizer=%s",
                          ROUTE_NAMES[r.kernel], r.bm, r.bn, r.splits, r.kb_per_split, r.groups_per_wg, (int)r.aligned,
-                         fused ? "fused" : "launch");
+                         route_stages(true, r, M, N), fused ? "fused" : "launch");
   MI355_REQUIRE(n > 0 && (size_t)n < buf_len, MI355_ERR_INVALID_ARGUMENT, "%s: buffer of %zu bytes is too small", what, buf_len);
   return MI355_OK;
 }
