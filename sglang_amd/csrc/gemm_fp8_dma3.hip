@@ -238,7 +238,13 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   // stages of a 64 x 128 tile take 73.5 KB, so two such workgroups share a CU's 160 KB
   __shared__ __attribute__((aligned(1024))) uint8_t t_stage[S][(BM + BN) * KSTEP];
   __shared__ __attribute__((aligned(256))) float t_scale[S][BM];
-  constexpr int YOUNGER = (S - 2) * (LOADS + 1);  // loads that may still be in flight when the next block is due
+  // PAIRED (six stages): one barrier per TWO K blocks (1-4 % over a barrier per block: K=7168 -> N=576 at M=2048 27.0 ->
+  // 26.3 us, K=7168 -> N=4096 at M=512 25.2 -> 24.3, K=7168 -> N=1536 at M=128 16.9 -> 16.5; never slower).  Iteration k requests block k + S - 2 into the stage that iteration
+  // k - 2 read, so the barrier after every odd iteration separates all reads of a stage from the next loads into it, and the
+  // wait in front of it covers the two blocks of the next pair: the S - 4 blocks requested after them may be in flight.
+  constexpr bool PAIRED = S == 6;
+  constexpr int AHEAD = PAIRED ? S - 2 : S - 1;                                 // blocks requested ahead of the one multiplied
+  constexpr int YOUNGER = (PAIRED ? S - 4 : S - 2) * (LOADS + 1);              // loads that may be in flight at a barrier
 
   float acc[T_NT][MT][4];
 #pragma unroll
@@ -248,15 +254,15 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
 
-  // ---- prologue: blocks 0 .. S-2 (clamped) into stages 0 .. S-2
+  // ---- prologue: blocks 0 .. AHEAD-1 (clamped) into stages 0 .. AHEAD-1
 #pragma unroll
-  for (int b = 0; b < S - 1; ++b)
+  for (int b = 0; b < AHEAD; ++b)
 #pragma unroll
     for (int i = 0; i <= LOADS; ++i) issue_one<BM, BN, UE8M0>(s, i, t_stage[b], t_scale[b], kb_begin + b);
-  wait_and_barrier<YOUNGER>();  // block 0 has landed everywhere
+  wait_and_barrier<YOUNGER>();  // block 0 (PAIRED: and block 1) has landed everywhere
 
-  // ---- S blocks per trip over the S stages; iteration k multiplies block k and requests block k + S - 1 into the stage
-  //      that iteration k - 1 read
+  // ---- S blocks per trip over the S stages; iteration k multiplies block k and requests block k + AHEAD into the stage
+  //      that iteration k - 1 (PAIRED: k - 2) read
   auto sb_of = [&](int kb, float (&v)[SB]) {
 #pragma unroll
     for (int b = 0; b < SB; ++b) v[b] = s.sb_ptr[b][(int64_t)(UE8M0 ? kb >> 2 : kb) * s.sb_sk];
@@ -268,9 +274,9 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
     for (int u = 0; u < S; ++u) sb_of(kb_begin + k + u, sbv[u]);
 #pragma unroll
     for (int u = 0; u < S; ++u) {
-      k_block<BM, BN, UE8M0>(s, t_stage[u], t_scale[u], sbv[u], acc, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S],
-                             kb_begin + k + u + S - 1, kb_begin + k + u);
-      wait_and_barrier<YOUNGER>();
+      k_block<BM, BN, UE8M0>(s, t_stage[u], t_scale[u], sbv[u], acc, t_stage[(u + AHEAD) % S], t_scale[(u + AHEAD) % S],
+                             kb_begin + k + u + AHEAD, kb_begin + k + u);
+      if (!PAIRED || (u & 1)) wait_and_barrier<YOUNGER>();
     }
   }
 #pragma unroll
@@ -278,9 +284,9 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
     if (k + u < nkb) {
       float sbl[SB];
       sb_of(kb_begin + k + u, sbl);
-      k_block<BM, BN, UE8M0>(s, t_stage[u], t_scale[u], sbl, acc, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S],
-                             kb_begin + k + u + S - 1, kb_begin + k + u);
-      if (k + u + 1 < nkb) wait_and_barrier<YOUNGER>();
+      k_block<BM, BN, UE8M0>(s, t_stage[u], t_scale[u], sbl, acc, t_stage[(u + AHEAD) % S], t_scale[(u + AHEAD) % S],
+                             kb_begin + k + u + AHEAD, kb_begin + k + u);
+      if ((!PAIRED || (u & 1)) && k + u + 1 < nkb) wait_and_barrier<YOUNGER>();
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
