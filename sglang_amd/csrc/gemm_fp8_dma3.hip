@@ -1,5 +1,6 @@
 // Blockwise-scaled FP8 GEMM for gfx950 with short token tiles: (64 or 128) x (256, 192 or 128) macro tile, 8 waves (two per SIMD),
-// THREE LDS stages (six for 64 x 128 tiles and four for 64 x 192 / 128 x 128 when a workgroup has a CU to itself).
+// THREE LDS stages (four for 64 x 192 and 128 x 128 tiles, six for 64 x 128 tiles when a workgroup has a CU to itself); the 128-token
+// tiles run with two extra loader waves (dma3_tile_lw).
 //
 // For 16 < M <= 1024 a linear layer is between weight streaming and MFMA-bound; prefill shapes with few output channels
 // (M = 4096, N = 576 or 1536) do not give 256 x 256 tiles enough workgroups.  Both take this kernel.  The tile is short in the token dimension
@@ -95,7 +96,7 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM, BN>& s, int i, uin
 // One K block out of `cur`; the loads of block kb_next go out over the first LOADS + 1 steps into `nxt`.
 // UE8M0: the scale stage holds the tokens' packed exponent words and sbv the weight blocks' (as bits); the byte of block
 // `kb` goes to the MFMA, which applies both scales and accumulates in place: no promotion FMAs.
-template <int BM, int BN, bool UE8M0 = false>
+template <int BM, int BN, bool UE8M0 = false, bool ISSUE = true>
 __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_t* cur, const float* sc_cur,
                                         const float (&sbv)[Dma3State<BM, BN>::SB], float (&acc)[BN / 64][BM / 32][4], uint8_t* nxt,
                                         float* sc_nxt, int kb_next, int kb = 0) {
@@ -159,7 +160,7 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
         else scb[(j + 1) & 1][b] = scp[(j + 1) * 16] * sbv[b];
       }
     }
-    if (t <= LOADS) issue_one<BM, BN, UE8M0>(s, t, nxt, sc_nxt, kb_next);
+    if (ISSUE && t <= LOADS) issue_one<BM, BN, UE8M0>(s, t, nxt, sc_nxt, kb_next);
     __builtin_amdgcn_sched_barrier(0);
   }
   if constexpr (!UE8M0) {
@@ -315,6 +316,196 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   }
 }
 
+// ---- The same tile with LOADER WAVES: waves 0..7 only read LDS and multiply, LW more waves only issue the direct-to-LDS
+// loads.  In the kernel above every wave's loads sit in the same in-order instruction stream as its LDS reads and MFMAs,
+// and with 128-token tiles the cost of the loads ADDS to the step's own time instead of hiding under it.  Here a loader
+// wave owns every LW-th group of 8 tile rows (one load instruction each) plus a copy of the tile's token-scale load, keeps
+// S - 1 blocks in flight, waits until the block due next has landed (a constant vmcnt, as above) and meets the compute
+// waves at the barrier that ends each K block; compute waves have nothing in vmcnt and only take the barrier.
+constexpr int T_LW = 2;  // loader waves
+template <int BM, int BN>
+struct LoaderState {
+  static constexpr int NG = (BM + BN) / 8 / T_LW;  // row groups per loader wave and K block
+  static_assert((BM + BN) / 8 % T_LW == 0, "row groups divide among the loader waves");
+  const uint8_t* a_base;
+  const uint8_t* b_base;
+  uint32_t goff[NG];  // lane's byte offset from the matrix base for row group lw + j * T_LW (rows clamped)
+  const float* sa_base;
+  uint32_t sa_off;
+  int64_t sa_sk;
+  int lw, kb_last;
+};
+template <int BM, int BN, bool UE8M0>
+__device__ __forceinline__ void loader_issue_block(const LoaderState<BM, BN>& L, uint8_t* stage, float* scale, int kb) {
+  constexpr int NG = LoaderState<BM, BN>::NG;
+  kb = min(kb, L.kb_last);
+#pragma unroll
+  for (int j = 0; j < NG; ++j) {
+    const int g = L.lw + j * T_LW;  // wave-uniform
+    const uint8_t* base = (g < BM / 8 ? L.a_base : L.b_base) + (uint64_t)kb * KSTEP;
+    asm volatile("" : "+s"(base));
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)(stage + g * 8 * KSTEP);
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(L.goff[j]), "s"(base), "s"(lds_addr) : "memory");
+  }
+  // the tile's BM token scales: BM / 4 lanes fetch 16 bytes each (every loader wave issues it, so that all count alike)
+  const float* sbase = L.sa_base + (int64_t)(UE8M0 ? kb >> 2 : kb) * L.sa_sk;
+  asm volatile("" : "+s"(sbase));
+  const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)scale;
+  uint64_t saved;
+  if constexpr (BM == 128)
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffffffff\n\ts_mov_b32 m0, %3\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved) : "v"(L.sa_off), "s"(sbase), "s"(lds_addr) : "memory");
+  else
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 0xffff\n\ts_mov_b32 m0, %3\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved) : "v"(L.sa_off), "s"(sbase), "s"(lds_addr) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void loader_wait_and_barrier() {
+  static_assert(N >= 1 && N <= 63, "vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <int BM, bool SPLIT, int BN, bool UE8M0, int S>
+__device__ __forceinline__ void dma3_tile_lw(const GemmParams& p, int m0, int n0, int split) {
+  static_assert(BN == 128 || BN == 192 || BN == 256, "channel tile");
+  static_assert(S >= 3 && S * ((BM + BN) * KSTEP + BM * 4) <= 160 * 1024, "the stages must fit the CU's LDS");
+  constexpr int WM = BM / 2, MT = WM / 16, T_WN = BN / 4, T_NT = T_WN / 16;
+  constexpr bool INTERLEAVED = Dma3State<BM, BN>::INTERLEAVED;
+  constexpr int SB = Dma3State<BM, BN>::SB;
+  constexpr int LPB = LoaderState<BM, BN>::NG + 1;  // loads per loader wave and K block
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kb_begin = split * p.kb_per_split;
+  const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
+  const int nkb = kb_end - kb_begin;
+
+  __shared__ __attribute__((aligned(1024))) uint8_t t_stage[S][(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(256))) float t_scale[S][BM];
+
+  if (wave >= 8) {
+    // ================= loader wave =================
+    LoaderState<BM, BN> L;
+    L.lw = wave - 8;
+    L.kb_last = kb_end - 1;
+    L.a_base = p.a, L.b_base = p.b;
+    const int lrow = lane >> 3;
+    const int chunk_byte = ((lane & 7) ^ lrow) * 16;  // lands swizzled by (row & 7)
+#pragma unroll
+    for (int j = 0; j < LoaderState<BM, BN>::NG; ++j) {
+      const int row = (L.lw + j * T_LW) * 8 + lrow;
+      if (row < BM) L.goff[j] = (uint32_t)((int64_t)min(m0 + row, p.M - 1) * p.lda + chunk_byte);
+      else L.goff[j] = (uint32_t)((int64_t)min(n0 + row - BM, p.N - 1) * p.ldb + chunk_byte);
+    }
+    L.sa_base = p.sa, L.sa_sk = p.sa_sk;
+    L.sa_off = (uint32_t)min(m0 + (lane & (BM / 4 - 1)) * 4, (p.M - 1) & ~3) * 4u;
+#pragma unroll
+    for (int b = 0; b < S - 1; ++b) loader_issue_block<BM, BN, UE8M0>(L, t_stage[b], t_scale[b], kb_begin + b);
+    loader_wait_and_barrier<(S - 2) * LPB>();  // block 0 has landed
+    int k = 0;
+    for (; k + S - 1 < nkb; k += S) {
+#pragma unroll
+      for (int u = 0; u < S; ++u) {
+        loader_issue_block<BM, BN, UE8M0>(L, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S], kb_begin + k + u + S - 1);
+        loader_wait_and_barrier<(S - 2) * LPB>();  // block k + u + 1 has landed
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < S - 1; ++u) {
+      if (k + u < nkb) {
+        loader_issue_block<BM, BN, UE8M0>(L, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S], kb_begin + k + u + S - 1);
+        if (k + u + 1 < nkb) loader_wait_and_barrier<(S - 2) * LPB>();
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no refetch may outlive the workgroup's LDS
+    return;
+  }
+
+  // ================= compute wave =================
+  const int wave_m = wave >> 2, wave_n = wave & 3;
+  const int l16 = lane & 15, q = lane >> 4;
+  Dma3State<BM, BN> s;
+  s.wave = wave;
+  s.kb_last = kb_end - 1;
+  {
+    const int trow = wave_m * WM + l16, crow = BM + wave_n * (INTERLEAVED ? 16 : T_WN) + l16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      s.tok_off[h] = trow * KSTEP + (((q + 4 * h) ^ (trow & 7)) << 4);
+      s.ch_off[h] = crow * KSTEP + (((q + 4 * h) ^ (crow & 7)) << 4);
+    }
+    s.sc_off = (wave_m * WM + l16) * 4;
+  }
+#pragma unroll
+  for (int b = 0; b < SB; ++b) {
+    const int first = INTERLEAVED ? n0 + 64 * b : n0 + wave_n * T_WN;
+    s.sb_ptr[b] = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(UE8M0 ? min(first, p.N - 1) : min(first, p.N - 1) / 128) * p.sb_sn);
+  }
+  s.sb_sk = p.sb_sk;
+
+  float acc[T_NT][MT][4];
+#pragma unroll
+  for (int i = 0; i < T_NT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+  auto sb_of = [&](int kb, float (&v)[SB]) {
+#pragma unroll
+    for (int b = 0; b < SB; ++b) v[b] = s.sb_ptr[b][(int64_t)(UE8M0 ? kb >> 2 : kb) * s.sb_sk];
+  };
+  asm volatile("s_barrier" ::: "memory");  // block 0 has landed (the loaders waited for it)
+  int k = 0;
+  for (; k + S - 1 < nkb; k += S) {
+    float sbv[S][SB];
+#pragma unroll
+    for (int u = 0; u < S; ++u) sb_of(kb_begin + k + u, sbv[u]);
+#pragma unroll
+    for (int u = 0; u < S; ++u) {
+      k_block<BM, BN, UE8M0, false>(s, t_stage[u], t_scale[u], sbv[u], acc, nullptr, nullptr, 0, kb_begin + k + u);
+      asm volatile("s_barrier" ::: "memory");
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < S - 1; ++u) {
+    if (k + u < nkb) {
+      float sbl[SB];
+      sb_of(kb_begin + k + u, sbl);
+      k_block<BM, BN, UE8M0, false>(s, t_stage[u], t_scale[u], sbl, acc, nullptr, nullptr, 0, kb_begin + k + u);
+      if (k + u + 1 < nkb) asm volatile("s_barrier" ::: "memory");
+    }
+  }
+
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = m0 + wave_m * WM + j * 16 + l16;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int i = 0; i < T_NT; ++i) {
+      const int n = n0 + (INTERLEAVED ? i * 64 + wave_n * 16 : wave_n * T_WN + i * 16) + 4 * q;
+      if (n >= p.N) continue;
+      const int nvalid = min(4, p.N - n);
+      if constexpr (SPLIT) {
+        float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)split * p.M + m) * p.N + n;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (v < nvalid) wsp[v] = acc[i][j][v];
+      } else {
+        fp8_channel_epilogue(p, n, acc[i][j]);
+        store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
+      }
+    }
+  }
+}
+
+template <int BM, bool SPLIT, int BN, bool UE8M0, int S>
+__global__ __launch_bounds__(T_THREADS + 64 * T_LW) void fp8_gemm_dma3_lw_kernel(const GemmParams p) {
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
+  dma3_tile_lw<BM, SPLIT, BN, UE8M0, S>(p, tc.tile_m * BM, tc.tile_n * BN, tc.split);
+}
+
 template <int BM, bool SPLIT, int BN, bool UE8M0 = false, int S = 3>
 __global__ __launch_bounds__(T_THREADS) void fp8_gemm_dma3_kernel(const GemmParams p) {
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
@@ -331,28 +522,34 @@ __global__ __launch_bounds__(T_THREADS) void fp8_grouped_dma3_kernel(const Group
   dma3_tile<BM, false>(p, m0, tile_n * T_BN, 0);
 }
 
-// More than three stages pay only where a workgroup has its CU to itself (otherwise two workgroups of three stages keep as
-// many blocks in flight).  Measured, us, three stages / more: K=7168 -> N=576 at M=2048 29.0 / 27.0, K=4096 -> N=14336 at
-// M=48 24.5 / 23.1, K=7168 -> N=4096 at M=512 25.8 / 24.6, K=18432 -> N=7168 at M=32 33.7 / 32.8, at M=64 37.9 / 37.3;
-// no change (within 0.3 us) for ten other shapes: these tiles are bound by the step's own chain of LDS reads, MFMAs and the
-// barrier more than by the latency of the loads.
-bool dma3_deep_pipeline(int64_t workgroups) { return workgroups <= NUM_CUS; }
-constexpr int deep_stages(int bm, int bn) { return bm + bn == 192 ? 6 : bm + bn == 256 ? 4 : 3; }  // 6 x 24 KB, 4 x 32 KB
+// Stages per tile shape.  A 64 x 128 tile's three stages take 73.5 KB, so two such workgroups share a CU and keep four blocks
+// in flight between them; where a launch has at most one workgroup per CU it runs six stages instead (one barrier per two
+// blocks).  64 x 192 and 128 x 128 tiles (32 KB a stage) have the CU to themselves either way: four stages.  Measured, us,
+// three stages / more: K=7168 -> N=576 at M=2048 29.0 / 26.3, K=4096 -> N=14336 at M=48 24.5 / 23.1, K=7168 -> N=4096 at
+// M=512 25.8 / 24.3, K=18432 -> N=7168 at M=32 33.7 / 32.8, at M=64 37.9 / 37.3; no change (within 0.3 us) for ten other
+// shapes: these tiles are bound by the step's own chain of LDS reads, MFMAs and the barrier more than by load latency.
+constexpr int stages_of(int bm, int bn, bool own_cu) { return bm + bn == 192 ? (own_cu ? 6 : 3) : bm + bn == 256 ? 4 : 3; }
 
 template <int BM, int BN, bool UE8M0 = false>
 int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits));
-  // more stages where they fit and each workgroup has a CU to itself
-  constexpr int DEEP = deep_stages(BM, BN);
-  const bool deep = DEEP > 3 && dma3_deep_pipeline((int64_t)p.tiles_m * p.tiles_n * p.splits);
-  if (p.splits > 1) {
-    if (deep) hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0, DEEP>), grid, dim3(T_THREADS), 0, stream, p);
-    else hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
+  if constexpr (BM == 128) {
+    // 128-token tiles: compute waves + loader waves (1-5 % over every wave loading for itself, on all sixteen shapes
+    // measured: K=7168 -> N=36864 at M=128 65.5 -> 62.6 us, K=7168 -> N=4096 at M=1024 39.1 -> 37.2, K=7168 -> N=16384 at
+    // M=300 59.8 -> 57.4, K=18432 -> N=7168 at M=300 75.5 -> 72.8)
+    constexpr int S = stages_of(BM, BN, true);
+    if (p.splits > 1) hipLaunchKernelGGL((fp8_gemm_dma3_lw_kernel<BM, true, BN, UE8M0, S>), grid, dim3(T_THREADS + 64 * T_LW), 0, stream, p);
+    else hipLaunchKernelGGL((fp8_gemm_dma3_lw_kernel<BM, false, BN, UE8M0, S>), grid, dim3(T_THREADS + 64 * T_LW), 0, stream, p);
+  } else if (BM + BN == 192 && (int64_t)p.tiles_m * p.tiles_n * p.splits > NUM_CUS) {
+    constexpr int S = stages_of(BM, BN, false);
+    if (p.splits > 1) hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0, S>), grid, dim3(T_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0, S>), grid, dim3(T_THREADS), 0, stream, p);
   } else {
-    if (deep) hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0, DEEP>), grid, dim3(T_THREADS), 0, stream, p);
-    else hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0>), grid, dim3(T_THREADS), 0, stream, p);
+    constexpr int S = stages_of(BM, BN, true);
+    if (p.splits > 1) hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, true, BN, UE8M0, S>), grid, dim3(T_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((fp8_gemm_dma3_kernel<BM, false, BN, UE8M0, S>), grid, dim3(T_THREADS), 0, stream, p);
   }
   return check_launch(what);
 }
@@ -412,7 +609,7 @@ double dma3_model_us(int64_t M, int64_t N, int64_t kb_total, int bm, int bn, int
 }
 }  // namespace
 
-int dma3_stages(int bm, int bn, int64_t workgroups) { return dma3_deep_pipeline(workgroups) ? deep_stages(bm, bn) : 3; }
+int dma3_stages(int bm, int bn, int64_t workgroups) { return stages_of(bm, bn, workgroups <= NUM_CUS); }
 
 Dma3Plan dma3_plan(int64_t M, int64_t N, int64_t K, bool is_int8) {
   Dma3Plan pl;

@@ -30,9 +30,8 @@ FP8_ROUTE_SHAPES = [
     # the same kernel with 256-channel tiles and a K split (long K, many channels), and with 128-channel tiles
     (65, 7168, 18432), (24, 36864, 14336), (100, 36864, 640), (40, 4096, 7168), (300, 4096, 7168), (1000, 4096, 2048),
     (400, 4096, 16384), (100, 65536, 512), (130, 4096, 7168),
-    # small tiles with more workgroups than CUs keep three LDS stages (the others above run four or six): 64 x 192 and
-    # 128 x 128, whole-K and split
-    (135, 49152, 1024), (198, 36864, 1024), (129, 22528, 10240), (193, 17408, 12288),
+    # small tiles with more workgroups than CUs: 64 x 192 and 128 x 128
+    (135, 49152, 1024), (198, 36864, 1024),
     # 192-channel tiles (a wave's three channel tiles are 64 channels apart): whole-K and split, a ragged last tile
     (100, 36864, 512), (20, 36864, 1024), (130, 3072, 7168), (300, 3072, 14336), (130, 1000, 896),
     # 256 x 256 two-phase and 256 x 128 pipelined kernels, K a multiple of 128 and not
@@ -55,10 +54,11 @@ FP8_REQUIRED_VARIANTS = {
     ("decode_wavesplit", "w4", "one_round", "two_tiles"), ("decode_wavesplit", "w4", "rounds", "two_tiles"),
     ("decode_wavesplit", "w8", "one_round", "two_tiles"), ("decode_wavesplit", "w8", "rounds", "two_tiles"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("dma3", 128, "whole"), ("dma3", 128, "split"),
-    # 64 x 128 tiles are only planned where the launch has at most one workgroup per CU: always the six-stage pipeline
+    # "deep" = more than three LDS stages: always for 64 x 192 and 128 x 128 tiles; for 64 x 128 tiles where the launch has at
+    # most one workgroup per CU, which is the only place the plan puts them
     ("dma3", 64, "whole", "bn128", "deep"), ("dma3", 64, "split", "bn128", "deep"),
-    ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"), ("dma3", 128, "whole", "bn128", "deep"), ("dma3", 128, "split", "bn128", "deep"),
-    ("dma3", 64, "whole", "bn192"), ("dma3", 64, "split", "bn192"), ("dma3", 64, "whole", "bn192", "deep"), ("dma3", 64, "split", "bn192", "deep"),
+    ("dma3", 128, "whole", "bn128", "deep"), ("dma3", 128, "split", "bn128", "deep"),
+    ("dma3", 64, "whole", "bn192", "deep"), ("dma3", 64, "split", "bn192", "deep"),
     ("dma3", 128, "whole", "bn192"), ("dma3", 128, "split", "bn192"),
     ("pingpong", "kfull"), ("pingpong", "ktail"), ("pipelined", "kfull"), ("pipelined", "ktail"),
     ("generic", 16, "aligned", "whole"), ("generic", 16, "aligned", "split"), ("generic", 16, "bytes", "split"),
