@@ -362,7 +362,7 @@ size_t workspace_bytes(int64_t M, int64_t N, int64_t K, bool is_fp8) {
     const size_t dneed = ds > 1 ? (size_t)ds * (size_t)M * (size_t)N * 4u : 0;
     if (dneed > need) need = dneed;
   }
-  if (is_fp8 && M > 16) need += scale_relayout_bytes(M, K);  // the direct-to-LDS kernels may have to re-lay the token scales out
+  if (is_fp8 && (M > 16 || (double)M >= route_constants().decode_dma3_min_tokens)) need += scale_relayout_bytes(M, K);  // the direct-to-LDS kernels may have to re-lay the token scales out
   return need;
 }
 
@@ -432,7 +432,28 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   r.aligned = aligned;
   const bool small_b = N * ldb < (1ll << 32);                 // kernels that address rows by 32-bit byte offsets
   const bool small_offsets = M * lda < (1ll << 32) && small_b;
-  if (!fused_quant && wavesplit_supported(M, N, K) && aligned && small_b && wavesplit_preferred(is_fp8, M, N, K)) {
+  const bool to_wavesplit = !fused_quant && wavesplit_supported(M, N, K) && aligned && small_b && wavesplit_preferred(is_fp8, M, N, K);
+  if (is_fp8 && !fused_quant && M <= 16 && K % KSTEP == 0 && aligned && small_offsets) {
+    // decode sizes on the mid-M kernel (one 64-token tile, K unsplit) where that fills the chip in one round: instead of the
+    // streaming kernel whenever that one would split K, instead of the wave-split kernel with 192-channel tiles
+    const RouteConstants& rc = route_constants();
+    if ((double)M >= rc.decode_dma3_min_tokens) {
+      // the channel tile: the one that gives the most workgroups in one round
+      int bn = 0;
+      int64_t most = 0;
+      for (int c = 256; c >= 128; c -= 64) {
+        const int64_t tiles = (N + c - 1) / c;
+        if ((double)tiles >= rc.decode_dma3_min_workgroups && tiles <= NUM_CUS && tiles > most) most = tiles, bn = c;
+      }
+      const bool instead = to_wavesplit ? (bn == 192 && (double)(K / KSTEP) > rc.decode_dma3_wavesplit_min_kblocks)
+                                        : (decode_supported(M, N, K) && decode_splits(M, N, K) > 1);
+      if (instead && bn != 0) {
+        r.kernel = RK_DMA3, r.bm = 64, r.bn = bn, r.splits = 1, r.kb_per_split = (int)(K / KSTEP);
+        return r;
+      }
+    }
+  }
+  if (to_wavesplit) {
     const WavesplitShape ws = wavesplit_shape(K);
     r.kernel = RK_WAVESPLIT, r.bm = 16, r.bn = wavesplit_two_tiles(is_fp8, M, N, K) ? 32 : 16, r.splits = 1;
     r.kb_per_split = (int)((K + KSTEP - 1) / KSTEP);
@@ -625,6 +646,7 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
     "dma3_small_tile_factor", "wavesplit_min_kblocks", "wavesplit_small_weight_bytes", "wavesplit_small_weight_max_tokens",
     "wavesplit_large_weight_max_tokens", "wavesplit_two_tile_min_workgroups", "wavesplit_two_tile_min_tokens",
     "wavesplit_two_tile_long_k_blocks", "wavesplit_two_tile_max_tokens", "wavesplit_long_k_max_tokens",
+    "decode_dma3_min_tokens", "decode_dma3_wavesplit_min_kblocks", "decode_dma3_min_workgroups",
     "fused_quant_long_k_blocks", "fused_quant_short_k_blocks", "fused_quant_short_k_max_tokens"};
 
 // LDS stages of the mid-M kernel's pipeline for this plan (0 for the other kernels, whose depth is fixed).
@@ -966,7 +988,9 @@ size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 // plus the kernel the GEMM alone would take?  Always where that kernel is the streaming one (a launch saved, nothing else
 // changes); against the wave-split kernel by measurement.
 bool fused_quant_preferred(int64_t M, int64_t N, int64_t K, int64_t ldw) {
-  if (choose_route(true, M, N, K, K, ldw, true).kernel != RK_WAVESPLIT) return true;
+  const int plain = choose_route(true, M, N, K, K, ldw, true).kernel;
+  if (plain == RK_DMA3) return false;  // the mid-M kernel at decode sizes beats the streaming kernel by more than a launch
+  if (plain != RK_WAVESPLIT) return true;
   const RouteConstants& rc = route_constants();
   const double kb = (double)(K / KSTEP);
   if (kb > rc.fused_quant_long_k_blocks) return false;

@@ -60,6 +60,20 @@ struct RouteConstants {
   double wavesplit_two_tile_long_k_blocks = 64.0;    // ... or at any token count once K has more blocks than this (four-wave workgroups)
   double wavesplit_two_tile_max_tokens = 12.0;       // FP8, larger weights, two tiles: up to here against the streaming kernel,
   double wavesplit_long_k_max_tokens = 16.0;         // ... and up to here beyond wavesplit_two_tile_long_k_blocks
+  // ---- the mid-M kernel at decode sizes (FP8, 4 .. 16 tokens padded to one 64-token tile, K unsplit): where unsplit tiles fill
+  //      most of the CUs in one round it streams the weight in one launch with 8-row x 128-byte loads.  Median launch, us,
+  //      mid-M kernel (token scales M-major with an aligned pitch; 3.5-4 us more when they have to be re-laid out first) /
+  //      streaming kernel + reduce at M = 16: 7168->36864 50.1 / 59.9, 7168->24576 36.4 / 43.2, 4096->28672 30.5 / 34.2,
+  //      2048->32768 16.6 / 20.2, 1536->24576 10.7 / 14.3; 7168->18432 (144 workgroups) 33.3 / 33.9; and where the streaming
+  //      kernel needs no split: 1024->65536 17.9 / 16.9, 512->32768 9.0 / 9.0.  Against the wave-split kernel (two tiles) at
+  //      M = 4 / 8 / 12: 7168->36864 (192-channel tiles) 49.6 / 49.9 / 50.2 against 52.0 / 54.6 / 57.7; with 128-channel tiles
+  //      7168->24576 35.8 / 36.0 / 36.2 against 34.3 / 36.1 / 38.3, 4096->28672 30.5 against 27.1 at M = 6, 2048->32768 16.6
+  //      against 14.8: so only the 192-channel tiling replaces the wave-split kernel.
+  double decode_dma3_min_tokens = 4.0;        // below, its token-scale quads do not exist and the wave-split kernel is as fast
+  double decode_dma3_wavesplit_min_kblocks = 44.0;  // ... and replaces the wave-split kernel only for K of more blocks than this
+                                                    // (M = 8: 7168->33280 47.2 against 53.6, 7168->49152 62.5 against 66.4, but
+                                                    // 4096->33280 36.0 against 31.4: one turn of the wave-split ring covers K = 4096)
+  double decode_dma3_min_workgroups = 170.0;  // unsplit tiles (of the channel width that gives most), at most one per CU: 192 and more measured, 144 not enough
   // ---- one-call linear at decode sizes: the streaming kernel with the quantizer in its prologue (one launch) against a
   //      quantizer launch + the wave-split kernel, where that is the GEMM's plan.  FP8, median call, us, fused / two launches:
   //      7168->36864: M=1 52.0/52.3, 4 54.6/56.2, 8 58.3/58.6;  18432->7168: M=1 30.8/30.1, 4 32.1/30.4, 8 33.6/31.6, 16 36.6/34.8;

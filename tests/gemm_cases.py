@@ -12,7 +12,7 @@ whether the workgroup owns one 16-channel tile or two, for the large-M kernels w
 FP8_ROUTE_SHAPES = [
     # decode kernel (M <= 16, K % 128 == 0, N % 128 == 0): whole-K and split, 1 / 2 / 3+ channel groups per workgroup,
     # an uneven last workgroup (16640 = 130 groups), short last K ranges (4480 = 35 blocks, 2176 = 17 blocks)
-    (1, 128, 128), (3, 256, 512), (16, 2048, 7168), (13, 18432, 7168), (13, 36864, 7168), (16, 16640, 4480), (15, 33280, 2176),
+    (1, 128, 128), (3, 256, 512), (16, 2048, 7168), (13, 18432, 7168), (13, 66560, 1152), (16, 16640, 4480), (15, 33280, 2176),
     (5, 66048, 512), (2, 133120, 384),
     # wave-split decode kernel (few tokens or a small weight, K of at least 8 blocks; N % 16 == 0 is enough): 8 waves with one
     # round (K = 4096) and two (K = 7168, 4480 = 35 blocks: a ragged second round), 4 waves with many rounds (K = 18432) and
@@ -20,7 +20,7 @@ FP8_ROUTE_SHAPES = [
     (1, 512, 4096), (4, 1536, 7168), (2, 7168, 2048), (2, 36864, 7168), (1, 512, 18432), (12, 48, 1152), (1, 512, 7168), (1, 16640, 4480),
     # ... and two channel tiles per workgroup (N / 32 >= 200 and three tokens or more, or K beyond 64 blocks): both wave counts,
     # one round and several, an uneven split of the K blocks over the waves (2176 = 17 blocks), N % 32 == 0 but N % 128 != 0
-    (16, 7168, 2048), (9, 33280, 2176), (7, 33280, 4096), (12, 36864, 7168), (6, 16640, 4480), (1, 7168, 18432), (16, 7168, 18432),
+    (16, 7168, 2048), (9, 33280, 2176), (7, 16640, 4096), (7, 33280, 4096), (3, 36864, 7168), (6, 16640, 4480), (1, 7168, 18432), (16, 7168, 18432),
     (5, 6432, 1280),
     (5, 48, 128), (16, 16, 256),  # a single K block (three of the four waves have nothing to add), a single workgroup
     # three-stage mid-M kernel: 64 / 128 token tiles x 256 / 192 / 128 channel tiles, whole-K and split, ragged M, K blocks per
@@ -30,6 +30,9 @@ FP8_ROUTE_SHAPES = [
     # the same kernel with 256-channel tiles and a K split (long K, many channels), and with 128-channel tiles
     (65, 7168, 18432), (24, 36864, 14336), (100, 36864, 640), (40, 4096, 7168), (300, 4096, 7168), (1000, 4096, 2048),
     (400, 4096, 16384), (100, 65536, 512), (130, 4096, 7168),
+    # decode sizes on the mid-M kernel (4 .. 16 tokens, one round of unsplit tiles): instead of the wave-split kernel with
+    # 192-channel tiles, instead of the split streaming kernel with 128- and 256-channel tiles
+    (4, 36864, 7168), (13, 36864, 7168), (16, 24576, 1536), (14, 32768, 2048), (16, 49152, 2048),
     # small tiles with more workgroups than CUs: 64 x 192 and 128 x 128
     (135, 49152, 1024), (198, 36864, 1024),
     # 192-channel tiles (a wave's three channel tiles are 64 channels apart): whole-K and split, a ragged last tile

@@ -91,7 +91,7 @@ def test_perturbed_plan_query():
 
     L = _lib.lib()
     n = L.mi355_route_constant_count()
-    assert n == 46 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
+    assert n == 49 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
     assert _lib.route_constants()["pp_fp8_us_per_kblock"] == 1.39
     buf = ctypes.create_string_buffer(256)
     assert L.mi355_gemm_plan_perturbed(1, 128, 7168, 18432, 1, n, 1.1, buf, len(buf)) == 1
@@ -113,11 +113,13 @@ def test_plan_query_rejects_bad_arguments():
     assert L.mi355_fp8_blockwise_mm_plan(16, 128, 128, 1, buf, len(buf)) == 1 and b"too small" in L.mi355_last_error()
     assert L.mi355_int8_scaled_mm_plan(0, 128, 128, 1, buf, len(buf)) == 1
     assert L.mi355_fp8_blockwise_mm_plan(16, 128, 128, 1, None, 0) == 1
-    p = _lib.gemm_plan("fp8", 13, 36864, 7168)
+    p = _lib.gemm_plan("fp8", 13, 18432, 7168)
     assert p["kernel"] == "decode" and p["splits"] == 7
+    p = _lib.gemm_plan("fp8", 13, 36864, 7168)  # one round of unsplit 64 x 192 tiles beats the split streaming kernel
+    assert (p["kernel"], p["bm"], p["bn"], p["splits"]) == ("dma3", 64, 192, 1)
     p = _lib.gemm_plan("fp8", 1, 36864, 7168)
     assert p["kernel"] == "decode_wavesplit" and p["splits"] == 1 and p["bn"] == 16
-    p = _lib.gemm_plan("fp8", 8, 36864, 7168)  # two channel tiles per workgroup from three tokens on
+    p = _lib.gemm_plan("fp8", 3, 36864, 7168)  # two channel tiles per workgroup from three tokens on
     assert p["kernel"] == "decode_wavesplit" and p["bn"] == 32
 
 
@@ -128,7 +130,7 @@ def test_block_linear_plan():
 
     from sglang_amd import _lib
 
-    for shape, want in (((1, 36864, 7168), ("fused", "decode")), ((8, 36864, 7168), ("fused", "decode")),
+    for shape, want in (((1, 36864, 7168), ("fused", "decode")), ((3, 36864, 7168), ("fused", "decode")), ((8, 36864, 7168), ("launch", "dma3")),
                         ((16, 2048, 7168), ("fused", "decode")), ((8, 7168, 2048), ("fused", "decode")),
                         ((4, 7168, 18432), ("launch", "decode_wavesplit")), ((16, 7168, 2048), ("launch", "decode_wavesplit")),
                         ((128, 7168, 2048), ("launch", "dma3")), ((4, 1000, 1024), ("launch", "generic"))):

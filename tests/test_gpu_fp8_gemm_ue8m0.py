@@ -104,7 +104,8 @@ def test_ue8m0_gemm_exact_integers(gpu, oracle, M, N, K):
 # in the MFMA too; 50 x 3000 has a ragged last channel tile, 33 x 16384 x 2176 a last exponent word with one byte used
 MID_M = [(48, 16384, 2048), (33, 16384, 2176), (40, 4096, 7168), (50, 3000, 4224), (24, 36864, 14336), (130, 3072, 7168), (40, 65536, 512),
          (130, 4096, 7168), (100, 32768, 640), (65, 7168, 18432), (100, 36864, 640), (300, 3072, 14336), (100, 65536, 512),
-         (400, 4096, 16384)]
+         (400, 4096, 16384),
+         (14, 36864, 1280), (16, 65536, 1152), (8, 36864, 7168), (16, 24576, 1536)]  # decode sizes on one round of unsplit 64-token tiles
 
 
 def test_mid_m_shapes_reach_every_tile_and_split():
@@ -133,7 +134,7 @@ def test_ue8m0_mid_m_kernel_against_oracle(gpu, oracle, M, N, K):
 # the streaming decode kernel: one K range and several, the last range short (K blocks not a multiple of 8), one to four
 # bytes used in the last exponent word, token counts below and at the 16 rows of the MFMA tile (rows past M repeat the last token)
 DECODE = [(8, 256, 512), (4, 4352, 512), (5, 4096, 36864), (16, 4096, 36864), (13, 18432, 7168), (15, 18432, 7168), (9, 3072, 1536),
-          (14, 36864, 1280), (14, 16384, 2304), (15, 65536, 640), (16, 65536, 1152), (13, 4096, 18432), (8, 4352, 128)]
+          (14, 70656, 1280), (14, 16384, 2304), (15, 65536, 640), (16, 66560, 1152), (13, 4096, 18432), (8, 4352, 128)]
 
 
 def test_decode_shapes_reach_the_streaming_kernel():
