@@ -433,20 +433,23 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
   const bool small_b = N * ldb < (1ll << 32);                 // kernels that address rows by 32-bit byte offsets
   const bool small_offsets = M * lda < (1ll << 32) && small_b;
   const bool to_wavesplit = !fused_quant && wavesplit_supported(M, N, K) && aligned && small_b && wavesplit_preferred(is_fp8, M, N, K);
-  if (is_fp8 && !fused_quant && M <= 16 && K % KSTEP == 0 && aligned && small_offsets) {
-    // decode sizes on the mid-M kernel (one 64-token tile, K unsplit) where that fills the chip in one round: instead of the
-    // streaming kernel whenever that one would split K, instead of the wave-split kernel with 192-channel tiles
+  if (!fused_quant && M <= 16 && K % KSTEP == 0 && aligned && small_offsets) {
+    // decode sizes on the mid-M kernel (one 64-token tile, K unsplit) where that fills the chip in one round.  FP8: instead
+    // of the streaming kernel whenever that one would split K, instead of the wave-split kernel with 192-channel tiles and
+    // long K.  INT8: from a dozen tokens on.
     const RouteConstants& rc = route_constants();
-    if ((double)M >= rc.decode_dma3_min_tokens) {
+    if ((double)M >= (is_fp8 ? rc.decode_dma3_min_tokens : rc.decode_dma3_int8_min_tokens)) {
       // the channel tile: the one that gives the most workgroups in one round
+      const double min_workgroups = is_fp8 ? rc.decode_dma3_min_workgroups : rc.decode_dma3_int8_min_workgroups;
       int bn = 0;
       int64_t most = 0;
-      for (int c = 256; c >= 128; c -= 64) {
+      for (int c = 256; c >= 128; c -= is_fp8 ? 64 : 128) {
         const int64_t tiles = (N + c - 1) / c;
-        if ((double)tiles >= rc.decode_dma3_min_workgroups && tiles <= NUM_CUS && tiles > most) most = tiles, bn = c;
+        if ((double)tiles >= min_workgroups && tiles <= NUM_CUS && tiles > most) most = tiles, bn = c;
       }
-      const bool instead = to_wavesplit ? (bn == 192 && (double)(K / KSTEP) > rc.decode_dma3_wavesplit_min_kblocks)
-                                        : (decode_supported(M, N, K) && decode_splits(M, N, K) > 1);
+      const bool instead = !is_fp8 ? true
+                           : to_wavesplit ? (bn == 192 && (double)(K / KSTEP) > rc.decode_dma3_wavesplit_min_kblocks)
+                                          : (decode_supported(M, N, K) && decode_splits(M, N, K) > 1);
       if (instead && bn != 0) {
         r.kernel = RK_DMA3, r.bm = 64, r.bn = bn, r.splits = 1, r.kb_per_split = (int)(K / KSTEP);
         return r;
@@ -646,7 +649,8 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
     "dma3_small_tile_factor", "wavesplit_min_kblocks", "wavesplit_small_weight_bytes", "wavesplit_small_weight_max_tokens",
     "wavesplit_large_weight_max_tokens", "wavesplit_two_tile_min_workgroups", "wavesplit_two_tile_min_tokens",
     "wavesplit_two_tile_long_k_blocks", "wavesplit_two_tile_max_tokens", "wavesplit_long_k_max_tokens",
-    "decode_dma3_min_tokens", "decode_dma3_wavesplit_min_kblocks", "decode_dma3_min_workgroups",
+    "decode_dma3_min_tokens", "decode_dma3_wavesplit_min_kblocks", "decode_dma3_int8_min_tokens", "decode_dma3_int8_min_workgroups",
+    "decode_dma3_min_workgroups",
     "fused_quant_long_k_blocks", "fused_quant_short_k_blocks", "fused_quant_short_k_max_tokens"};
 
 // LDS stages of the mid-M kernel's pipeline for this plan (0 for the other kernels, whose depth is fixed).

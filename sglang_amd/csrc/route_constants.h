@@ -73,6 +73,12 @@ struct RouteConstants {
   double decode_dma3_wavesplit_min_kblocks = 44.0;  // ... and replaces the wave-split kernel only for K of more blocks than this
                                                     // (M = 8: 7168->33280 47.2 against 53.6, 7168->49152 62.5 against 66.4, but
                                                     // 4096->33280 36.0 against 31.4: one turn of the wave-split ring covers K = 4096)
+  // INT8 (the wave-split kernel has one channel tile per workgroup there, so its time grows faster with the tokens), median
+  // launch, us, wave-split / mid-M kernel at M = 4 / 8 / 16: 7168->24576 37.6 / 42.2 / 50.5 against 37.9 / 37.6 / 38.3,
+  // 2048->32768 16.2 / 18.1 / 21.1 against 17.4 / 17.4 / 17.8, 7168->36864 (144 tiles of 256 channels) 54.3 / 61.8 / 74.6
+  // against 58.3 / 58.5 / 59.6, 4096->28672 25.5 / 27.3 / 33.0 against 31.9 / 31.9 / 32.1
+  double decode_dma3_int8_min_tokens = 12.0;
+  double decode_dma3_int8_min_workgroups = 130.0;
   double decode_dma3_min_workgroups = 170.0;  // unsplit tiles (of the channel width that gives most), at most one per CU: 192 and more measured, 144 not enough
   // ---- one-call linear at decode sizes: the streaming kernel with the quantizer in its prologue (one launch) against a
   //      quantizer launch + the wave-split kernel, where that is the GEMM's plan.  FP8, median call, us, fused / two launches:
