@@ -57,7 +57,8 @@ def _rand_fp8(shape, g):
 # (+ 192-channel tiles of the mid-M kernel, whole-K and split: the channel-scale epilogue follows their interleaved tiles)
 SHAPES = [(1, 512, 1024), (16, 2048, 7168), (48, 16384, 2048), (130, 8192, 7168), (300, 1088, 512), (128, 16, 512),
           (1024, 1024, 4096), (4096, 4352, 512), (4000, 576, 1024), (100, 36864, 512), (130, 3072, 7168),
-          (3990, 4304, 512)]  # two-phase kernel with a ragged last token tile (6 of 16 rows) and a ragged last channel tile
+          (3990, 4304, 512),  # two-phase kernel with a ragged last token tile (6 of 16 rows) and a ragged last channel tile
+          (8, 36864, 5760), (13, 24576, 1536)]  # decode sizes on one round of unsplit mid-M tiles (the token scales are re-laid out first)
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
