@@ -178,6 +178,36 @@ __device__ __forceinline__ void wait_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(YOUNGER) : "memory");
 }
 
+// Epilogue of a compute wave: the lane holds channels n .. n+3 of token m for each of its MFMA tiles; raw partial sums to the
+// workspace (SPLIT) or channel epilogue, conversion and store.
+template <int BM, bool SPLIT, int BN>
+__device__ __forceinline__ void store_tile(const GemmParams& p, float (&acc)[BN / 64][BM / 32][4], int m0, int n0, int split, int wave_m,
+                                           int wave_n, int l16, int q) {
+  constexpr int WM = BM / 2, MT = WM / 16, T_WN = BN / 4, T_NT = T_WN / 16;
+  constexpr bool INTERLEAVED = Dma3State<BM, BN>::INTERLEAVED;
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int m = m0 + wave_m * WM + j * 16 + l16;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int i = 0; i < T_NT; ++i) {
+      const int n = n0 + (INTERLEAVED ? i * 64 + wave_n * 16 : wave_n * T_WN + i * 16) + 4 * q;
+      if (n >= p.N) continue;
+      const int nvalid = min(4, p.N - n);
+      if constexpr (SPLIT) {
+        float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)split * p.M + m) * p.N + n;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          if (v < nvalid) wsp[v] = acc[i][j][v];
+      } else {
+        fp8_channel_epilogue(p, n, acc[i][j]);
+        store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
+      }
+    }
+  }
+}
+
 // One BM x 256 output tile at (m0, n0), K blocks of split `split`, by the whole workgroup.
 // UE8M0: p.sa / p.sb point to packed exponent words (int32): token word (m, kw) at sa[kw * sa_sk + m], channel word (n, kw)
 // at sb[kw * sb_sk + n * sb_sn], byte kb & 3 of word kb >> 2 belongs to K block kb; the MFMA applies them.
@@ -292,28 +322,7 @@ __device__ __forceinline__ void dma3_tile(const GemmParams& p, int m0, int n0, i
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
 
-  // ---- epilogue: lane holds channels n .. n+3 of token m
-  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-#pragma unroll
-  for (int j = 0; j < MT; ++j) {
-    const int m = m0 + wave_m * WM + j * 16 + l16;
-    if (m >= p.M) continue;
-#pragma unroll
-    for (int i = 0; i < T_NT; ++i) {
-      const int n = n0 + (INTERLEAVED ? i * 64 + wave_n * 16 : wave_n * T_WN + i * 16) + 4 * q;
-      if (n >= p.N) continue;
-      const int nvalid = min(4, p.N - n);
-      if constexpr (SPLIT) {
-        float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)split * p.M + m) * p.N + n;
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          if (v < nvalid) wsp[v] = acc[i][j][v];
-      } else {
-        fp8_channel_epilogue(p, n, acc[i][j]);
-        store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
-      }
-    }
-  }
+  store_tile<BM, SPLIT, BN>(p, acc, m0, n0, split, wave_m, wave_n, l16, q);
 }
 
 // ---- The same tile with LOADER WAVES: waves 0..7 only read LDS and multiply, LW more waves only issue the direct-to-LDS
@@ -477,27 +486,7 @@ __device__ __forceinline__ void dma3_tile_lw(const GemmParams& p, int m0, int n0
     }
   }
 
-  const bool vec_ok = ((p.ldo & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-#pragma unroll
-  for (int j = 0; j < MT; ++j) {
-    const int m = m0 + wave_m * WM + j * 16 + l16;
-    if (m >= p.M) continue;
-#pragma unroll
-    for (int i = 0; i < T_NT; ++i) {
-      const int n = n0 + (INTERLEAVED ? i * 64 + wave_n * 16 : wave_n * T_WN + i * 16) + 4 * q;
-      if (n >= p.N) continue;
-      const int nvalid = min(4, p.N - n);
-      if constexpr (SPLIT) {
-        float* wsp = reinterpret_cast<float*>(p.ws) + ((int64_t)split * p.M + m) * p.N + n;
-#pragma unroll
-        for (int v = 0; v < 4; ++v)
-          if (v < nvalid) wsp[v] = acc[i][j][v];
-      } else {
-        fp8_channel_epilogue(p, n, acc[i][j]);
-        store_out4(p.out, p.out_dtype, (int64_t)m * p.ldo + n, acc[i][j], nvalid, vec_ok);
-      }
-    }
-  }
+  store_tile<BM, SPLIT, BN>(p, acc, m0, n0, split, wave_m, wave_n, l16, q);
 }
 
 template <int BM, bool SPLIT, int BN, bool UE8M0, int S>
