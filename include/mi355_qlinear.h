@@ -369,8 +369,9 @@ int mi355_fp8_scaled_mm(const void* a, const void* b, const float* sa, const flo
  *          GEMM and `output += bias`.  The activation is quantized with q = x / s (s = max(amax, 1e-10) / 448) into the
  *          workspace, with M-major scales, and the bias is added in fp32 in the GEMM epilogue (the reference adds it
  *          after rounding the GEMM result to the output type).  At decode sizes (M <= 16, 16-bit x, N % 128 == 0) there
- *          is no quantizer launch where that is the faster way: the GEMM kernel quantizes the tokens of its K range in its
- *          prologue, with the same arithmetic, and the result is bit-identical to the two-step sequence.
+ *          is no quantizer launch where that is the faster way: the GEMM kernel quantizes the tokens itself (the streaming
+ *          kernel in its prologue, the mid-M kernel by producer waves), with the same arithmetic, and the result is
+ *          bit-identical to the two-step sequence.
  *          mi355_fp8_block_linear_plan (host only, dense 16-byte aligned operands assumed) writes the GEMM's plan in the
  *          format of mi355_fp8_blockwise_mm_plan followed by quantizer=fused|launch.
  *   x [M, K] contiguous F32/F16/BF16, K % 128 == 0; w [N, K] e4m3fn row stride ldw; w_scale element (nb, kb) at

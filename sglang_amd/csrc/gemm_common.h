@@ -52,6 +52,52 @@ __device__ __forceinline__ int in_vgpr(int x) {
   return x;
 }
 
+// ---- 1 x 128 group quantization inside a GEMM kernel (the one-call linear at decode sizes): 16 lanes hold a group, 8
+// elements each, with the arithmetic of the group quantizer's reference path (amax floored at 1e-10, s = amax / 448,
+// q = e4m3fn(clamp(x / s)), group_quant.hip).
+// max over the 16 lanes of a DPP row
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
+  return v;
+}
+// x / s, correctly rounded, given r = RN(1 / s): two Markstein steps, as in the group quantizer (group_quant.hip), where
+// the conditions under which this equals the `/` operator are stated and checked.
+__device__ __forceinline__ float div_by_shared(float x, float s, float r) {
+  float q = x * r;
+  q = fmaf(fmaf(-q, s, x), r, q);
+  q = fmaf(fmaf(-q, s, x), r, q);
+  return q;
+}
+// The lane's eight 16-bit elements (raw) of a group spread over its DPP row -> their eight e4m3fn codes and the group's scale
+// (the same value in all 16 lanes).  Every lane of the row must be active.
+__device__ __forceinline__ u32x2 quantize_group_lane(const u32x4& raw, int x_dtype, float& scale) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = x_dtype == MI355_BF16 ? __uint_as_float(w[i] << 16) : f16_bits_to_f32(w[i] & 0xffffu);
+    v[2 * i + 1] = x_dtype == MI355_BF16 ? __uint_as_float(w[i] & 0xffff0000u) : f16_bits_to_f32(w[i] >> 16);
+  }
+  float amax = 1e-10f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
+  amax = row16_max(amax);
+  const float sc = amax / 448.0f;
+  const float rcp = 1.0f / sc;
+  float t[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) t[e] = fminf(fmaxf(div_by_shared(v[e], sc, rcp), -448.0f), 448.0f);
+  int c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
+  c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c0, true);
+  int c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], 0, false);
+  c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], c1, true);
+  scale = sc;
+  return u32x2{(uint32_t)c0, (uint32_t)c1};
+}
+
 __device__ __forceinline__ void store_out4(void* out, int out_dtype, int64_t off, const float* r, int nvalid,
                                            bool vec_ok) {
   if (out_dtype == MI355_F32) {
@@ -195,6 +241,8 @@ int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const cha
 // The same for packed UE8M0 scales on both operands (p.sa / p.sb point to the words, p.sa_sk / p.sb_sn / p.sb_sk are word
 // strides; token words M-major with a pitch that is a multiple of four words), applied by the MFMA.
 int launch_fp8_dma3_ue8m0(GemmParams& p, int bm, int bn, hipStream_t stream, const char* what);
+// One-call linear at decode sizes on this kernel: a producer wave quantizes the unquantized tokens (p.x16, M <= 16) block by block.
+int launch_fp8_dma3_quant(GemmParams& p, int bn, hipStream_t stream, const char* what);
 
 // Grouped problems on the tile bodies of the dense kernels: token rows of all experts stacked in one matrix, one weight
 // matrix per expert.  `g` describes expert 0 (a, out, b, sb, and sa = the re-laid-out token scales: M-major, every

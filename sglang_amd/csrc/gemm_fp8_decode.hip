@@ -149,15 +149,6 @@ __device__ __forceinline__ void consume(const DecodeState& s, const uint8_t* sta
   }
 }
 
-// max over the 16 lanes of a DPP row
-__device__ __forceinline__ float row16_max(float v) {
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
-  return v;
-}
-
 // QUANT (FP8 only): the tokens come unquantized (p.x16, bf16 or fp16) and the workgroup quantizes the 16 x KB_PER groups of
 // its K range itself, straight into the token stage, with the arithmetic of the group quantizer's reference path
 // (amax floored at 1e-10, s = amax / 448, q = e4m3fn(clamp(x / s)), group_quant.hip) - so a linear layer at decode sizes
@@ -176,14 +167,6 @@ __device__ __forceinline__ void load_raw_tokens(const GemmParams& p, int kb_begi
                                                (int64_t)min(kb_begin + d, p.kb_total - 1) * KSTEP + gl * 8);
   }
 }
-// x / s, correctly rounded, given r = RN(1 / s): two Markstein steps, as in the group quantizer (group_quant.hip), where
-// the conditions under which this equals the `/` operator are stated and checked.
-__device__ __forceinline__ float div_by_shared(float x, float s, float r) {
-  float q = x * r;
-  q = fmaf(fmaf(-q, s, x), r, q);
-  q = fmaf(fmaf(-q, s, x), r, q);
-  return q;
-}
 template <int KBP>
 __device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begin, const u32x4 (&raw)[KBP], uint8_t* tok,
                                                 float* sa_lds) {
@@ -192,29 +175,11 @@ __device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begi
   for (int j = 0; j < KBP; ++j) {
     const int pair = r + 16 * j, m = pair / KBP, d = pair % KBP;
     if (m >= p.M) break;  // uniform over the 16-lane row, which is all the DPP reduction below involves
-    const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
-    float v[8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[2 * i] = p.x_dtype == MI355_BF16 ? __uint_as_float(w[i] << 16) : f16_bits_to_f32(w[i] & 0xffffu);
-      v[2 * i + 1] = p.x_dtype == MI355_BF16 ? __uint_as_float(w[i] & 0xffff0000u) : f16_bits_to_f32(w[i] >> 16);
-    }
-    float amax = 1e-10f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
-    amax = row16_max(amax);
-    const float sc = amax / 448.0f;
-    const float rcp = 1.0f / sc;
-    float t[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) t[e] = fminf(fmaxf(div_by_shared(v[e], sc, rcp), -448.0f), 448.0f);
-    int c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
-    c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c0, true);
-    int c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], 0, false);
-    c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[6], t[7], c1, true);
+    float sc;
+    const u32x2 codes = quantize_group_lane(raw[j], p.x_dtype, sc);
     const bool valid = kb_begin + d < p.kb_total;  // blocks past the end of K: zero tokens, zero scale
     *reinterpret_cast<u32x2*>(tok + d * TOK_BLOCK + m * KSTEP + (((gl >> 1) ^ (m & 7)) << 4) + (gl & 1) * 8) =
-        valid ? u32x2{(uint32_t)c0, (uint32_t)c1} : u32x2{0u, 0u};
+        valid ? codes : u32x2{0u, 0u};
     if (gl < WAVES) sa_lds[gl * (SLICE / 4) + d * 16 + m] = valid ? sc : 0.f;  // one copy per wave slice (all 16 lanes hold sc)
   }
 }

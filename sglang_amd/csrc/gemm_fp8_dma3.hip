@@ -96,7 +96,9 @@ __device__ __forceinline__ void issue_one(const Dma3State<BM, BN>& s, int i, uin
 // One K block out of `cur`; the loads of block kb_next go out over the first LOADS + 1 steps into `nxt`.
 // UE8M0: the scale stage holds the tokens' packed exponent words and sbv the weight blocks' (as bits); the byte of block
 // `kb` goes to the MFMA, which applies both scales and accumulates in place: no promotion FMAs.
-template <int BM, int BN, bool UE8M0 = false, bool ISSUE = true>
+// ISSUE: 1 = the wave issues its share of every load of block kb_next (tile rows and token scales), 2 = of the weight rows
+// only (a producer wave writes the tokens), 0 = none (loader waves do).
+template <int BM, int BN, bool UE8M0 = false, int ISSUE = 1>
 __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_t* cur, const float* sc_cur,
                                         const float (&sbv)[Dma3State<BM, BN>::SB], float (&acc)[BN / 64][BM / 32][4], uint8_t* nxt,
                                         float* sc_nxt, int kb_next, int kb = 0) {
@@ -160,7 +162,8 @@ __device__ __forceinline__ void k_block(const Dma3State<BM, BN>& s, const uint8_
         else scb[(j + 1) & 1][b] = scp[(j + 1) * 16] * sbv[b];
       }
     }
-    if (ISSUE && t <= LOADS) issue_one<BM, BN, UE8M0>(s, t, nxt, sc_nxt, kb_next);
+    if (ISSUE == 1 && t <= LOADS) issue_one<BM, BN, UE8M0>(s, t, nxt, sc_nxt, kb_next);
+    if (ISSUE == 2 && t >= BM / 64 && t < LOADS) issue_one<BM, BN, UE8M0>(s, t, nxt, sc_nxt, kb_next);
     __builtin_amdgcn_sched_barrier(0);
   }
   if constexpr (!UE8M0) {
@@ -472,7 +475,7 @@ __device__ __forceinline__ void dma3_tile_lw(const GemmParams& p, int m0, int n0
     for (int u = 0; u < S; ++u) sb_of(kb_begin + k + u, sbv[u]);
 #pragma unroll
     for (int u = 0; u < S; ++u) {
-      k_block<BM, BN, UE8M0, false>(s, t_stage[u], t_scale[u], sbv[u], acc, nullptr, nullptr, 0, kb_begin + k + u);
+      k_block<BM, BN, UE8M0, 0>(s, t_stage[u], t_scale[u], sbv[u], acc, nullptr, nullptr, 0, kb_begin + k + u);
       asm volatile("s_barrier" ::: "memory");
     }
   }
@@ -481,7 +484,7 @@ __device__ __forceinline__ void dma3_tile_lw(const GemmParams& p, int m0, int n0
     if (k + u < nkb) {
       float sbl[SB];
       sb_of(kb_begin + k + u, sbl);
-      k_block<BM, BN, UE8M0, false>(s, t_stage[u], t_scale[u], sbl, acc, nullptr, nullptr, 0, kb_begin + k + u);
+      k_block<BM, BN, UE8M0, 0>(s, t_stage[u], t_scale[u], sbl, acc, nullptr, nullptr, 0, kb_begin + k + u);
       if (k + u + 1 < nkb) asm volatile("s_barrier" ::: "memory");
     }
   }
@@ -493,6 +496,163 @@ template <int BM, bool SPLIT, int BN, bool UE8M0, int S>
 __global__ __launch_bounds__(T_THREADS + 64 * T_LW) void fp8_gemm_dma3_lw_kernel(const GemmParams p) {
   const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n);
   dma3_tile_lw<BM, SPLIT, BN, UE8M0, S>(p, tc.tile_m * BM, tc.tile_n * BN, tc.split);
+}
+
+// ---- The 64-token tile for the one-call linear at decode sizes (M <= 16, K unsplit): the tokens arrive unquantized
+// (p.x16, bf16 or fp16) and four more waves, the PRODUCERS, quantize the 16 x 128 values of a K block into the stage's token rows
+// and scale slots - the arithmetic of the group quantizer's reference path (quantize_group_lane), so the result equals
+// quantizer launch + GEMM bit for bit - while waves 0..7 load the weight rows and multiply as above.  A producer requests
+// the raw tokens four blocks ahead of the one it quantizes (one 16-byte load per lane and block, its own vmcnt), writes S - 1 blocks ahead of
+// the one being multiplied, and meets the others at every block's barrier.  Token rows 16..63 of a stage are never written:
+// what they hold only reaches accumulators of rows that are not stored.
+constexpr int T_PW = 4;  // producer waves of the fused quantizer
+template <int BN, int S>
+__device__ __forceinline__ void dma3_tile_q(const GemmParams& p, int n0) {
+  constexpr int BM = 64;
+  static_assert(S >= 3 && S * ((BM + BN) * KSTEP + BM * 4) <= 160 * 1024, "the stages must fit the CU's LDS");
+  constexpr int LOADS = Dma3State<BM, BN>::LOADS, LOADS_W = LOADS - BM / 64;  // weight-row loads per wave and block
+  constexpr bool INTERLEAVED = Dma3State<BM, BN>::INTERLEAVED;
+  constexpr int SB = Dma3State<BM, BN>::SB, WM = BM / 2, MT = WM / 16, T_WN = BN / 4, T_NT = T_WN / 16;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nkb = p.kb_total, kb_last = p.kb_total - 1;
+
+  __shared__ __attribute__((aligned(1024))) uint8_t t_stage[S][(BM + BN) * KSTEP];
+  __shared__ __attribute__((aligned(256))) float t_scale[S][BM];
+
+  if (wave >= 8) {
+    // ================= producer wave pw: tokens 4 pw .. 4 pw + 3 =================
+    // (one wave quantizing all sixteen tokens of a block takes ~1.3 us of dependent arithmetic per block, more than the block's
+    // multiplication: 78 against 50 us on K=7168 -> N=36864; four waves take a quarter each)
+    const int pw = wave - 8;
+    const int gl = lane & 15, r4 = lane >> 4;  // 16 lanes per (token, block) group; four tokens per wave
+    const int m = pw * 4 + r4;                 // the stage row this lane's group goes to; rows past M repeat the last token
+    const bool active = pw * 4 < p.M;          // a wave whose tokens all lie past M only keeps the barriers
+    const uint16_t* xrow = reinterpret_cast<const uint16_t*>(p.x16) + (int64_t)min(m, p.M - 1) * p.ldx + gl * 8;
+    auto request = [&](int kb, u32x4& raw) {
+      const uint16_t* src = xrow + (int64_t)min(kb, kb_last) * KSTEP;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(raw) : "v"(src) : "memory");
+    };
+    auto produce = [&](int stage, const u32x4& raw) {
+      float sc;
+      const u32x2 codes = quantize_group_lane(raw, p.x_dtype, sc);
+      *reinterpret_cast<u32x2*>(&t_stage[stage][m * KSTEP + (((gl >> 1) ^ (m & 7)) << 4) + (gl & 1) * 8]) = codes;
+      if (gl == 0) t_scale[stage][m] = sc;
+    };
+    // A ring of R registers keeps the raw tokens of the next R blocks in flight: one is quantized into its stage, then
+    // requested again for the block R further on (a register that a load is still writing cannot be copied, so the loop is
+    // unrolled over the ring).  Step b produces block b into stage b % S; from step S - 2 on (blocks 0 .. S-2 are in LDS) every
+    // step ends at a barrier: the first is the one the other waves pass before block 0, the j-th after it ends their block j - 1,
+    // so block b is written after the barrier that ends block b - S, the last reader of its stage.
+    constexpr int R = 4;
+    static_assert(R == 4, "the wait below is written for a ring of four loads");
+    u32x4 ring[R];
+    if (active) {
+#pragma unroll
+      for (int u = 0; u < R; ++u) request(u, ring[u]);
+    }
+    const int steps = nkb + S - 2;
+    int st = 0;
+    for (int b = 0; b < steps; b += R) {
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        if (b + u < steps) {
+          if (active) {
+            asm volatile("s_waitcnt vmcnt(3)" : "+v"(ring[u])::"memory");  // the oldest of the R loads in flight
+            produce(st, ring[u]);
+            st = st + 1 == S ? 0 : st + 1;
+            request(b + u + R, ring[u]);
+          }
+          if (b + u >= S - 2) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        }
+      }
+    }
+    if (nkb % S == 0) asm volatile("s_barrier" ::: "memory");  // the other waves' barrier after the last block of a whole trip
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
+
+  // ================= waves 0..7: weight loads and arithmetic =================
+  const int wave_m = wave >> 2, wave_n = wave & 3;
+  const int l16 = lane & 15, q = lane >> 4;
+  Dma3State<BM, BN> s;
+  s.wave = wave;
+  s.kb_last = kb_last;
+  s.a_base = p.b;  // (token rows are not loaded; a valid address all the same)
+  s.b_base = p.b;
+  {
+    const int lrow = lane >> 3;
+    const int chunk_byte = ((lane & 7) ^ lrow) * 16;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int row = i * 64 + wave * 8 + lrow;
+      s.goff[i] = row < BM ? 0u : (uint32_t)((int64_t)min(n0 + row - BM, p.N - 1) * p.ldb + chunk_byte);
+    }
+    const int trow = wave_m * WM + l16, crow = BM + wave_n * (INTERLEAVED ? 16 : T_WN) + l16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      s.tok_off[h] = trow * KSTEP + (((q + 4 * h) ^ (trow & 7)) << 4);
+      s.ch_off[h] = crow * KSTEP + (((q + 4 * h) ^ (crow & 7)) << 4);
+    }
+    s.sc_off = (wave_m * WM + l16) * 4;
+  }
+  s.sa_base = p.sb, s.sa_off = 0, s.sa_sk = 0;  // (token scales are not loaded)
+#pragma unroll
+  for (int b = 0; b < SB; ++b) {
+    const int first = INTERLEAVED ? n0 + 64 * b : n0 + wave_n * T_WN;
+    s.sb_ptr[b] = (cfloat_ptr)(p.sb + (int64_t)__builtin_amdgcn_readfirstlane(min(first, p.N - 1) / 128) * p.sb_sn);
+  }
+  s.sb_sk = p.sb_sk;
+  constexpr int YOUNGER = (S - 2) * LOADS_W;
+
+  float acc[T_NT][MT][4];
+#pragma unroll
+  for (int i = 0; i < T_NT; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+#pragma unroll
+  for (int b = 0; b < S - 1; ++b)
+#pragma unroll
+    for (int i = BM / 64; i < LOADS; ++i) issue_one<BM, BN, false>(s, i, t_stage[b], t_scale[b], b);
+  wait_and_barrier<YOUNGER>();  // the weight rows of block 0 have landed; the producer has written blocks 0 .. S-2
+
+  auto sb_of = [&](int kb, float (&v)[SB]) {
+#pragma unroll
+    for (int b = 0; b < SB; ++b) v[b] = s.sb_ptr[b][(int64_t)kb * s.sb_sk];
+  };
+  int k = 0;
+  for (; k + S - 1 < nkb; k += S) {
+    float sbv[S][SB];
+#pragma unroll
+    for (int u = 0; u < S; ++u) sb_of(k + u, sbv[u]);
+#pragma unroll
+    for (int u = 0; u < S; ++u) {
+      k_block<BM, BN, false, 2>(s, t_stage[u], t_scale[u], sbv[u], acc, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S], k + u + S - 1, k + u);
+      wait_and_barrier<YOUNGER>();  // unconditional (a condition here makes the compiler sink arithmetic across blocks): when K
+                                    // is a whole number of trips this is one barrier past the last block, which the producers match
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < S - 1; ++u) {
+    if (k + u < nkb) {
+      float sbl[SB];
+      sb_of(k + u, sbl);
+      k_block<BM, BN, false, 2>(s, t_stage[u], t_scale[u], sbl, acc, t_stage[(u + S - 1) % S], t_scale[(u + S - 1) % S], k + u + S - 1, k + u);
+      if (k + u + 1 < nkb) wait_and_barrier<YOUNGER>();
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
+  store_tile<BM, false, BN>(p, acc, 0, n0, 0, wave_m, wave_n, l16, q);
+}
+
+template <int BN, int S>
+__global__ __launch_bounds__(T_THREADS + 64 * T_PW) void fp8_gemm_dma3_q_kernel(const GemmParams p) {
+  const TileCoord tc = tile_of_block(blockIdx.x, gridDim.x, 1, p.tiles_n);
+  dma3_tile_q<BN, S>(p, tc.tile_n * BN);
 }
 
 template <int BM, bool SPLIT, int BN, bool UE8M0 = false, int S = 3>
@@ -648,6 +808,22 @@ int launch_fp8_dma3(GemmParams& p, int bm, int bn, hipStream_t stream, const cha
   if (bn == 128) return bm == 64 ? launch_bm<64, 128>(p, stream, what) : launch_bm<128, 128>(p, stream, what);
   if (bn == 192) return bm == 64 ? launch_bm<64, 192>(p, stream, what) : launch_bm<128, 192>(p, stream, what);
   return bm == 64 ? launch_bm<64, 256>(p, stream, what) : launch_bm<128, 256>(p, stream, what);
+}
+
+// One-call linear at decode sizes: p.x16 / p.ldx / p.x_dtype describe the unquantized tokens (M <= 16, 16-byte aligned rows),
+// K unsplit, one 64-token tile per workgroup; p.a and p.sa are not read.
+int launch_fp8_dma3_quant(GemmParams& p, int bn, hipStream_t stream, const char* what) {
+  if (p.M > 16 || p.x16 == nullptr || p.splits != 1) {
+    set_error("%s: the fused quantizer of the mid-M kernel takes up to 16 unquantized tokens and an unsplit K", what);
+    return MI355_ERR_UNSUPPORTED;
+  }
+  p.tiles_m = 1;
+  p.tiles_n = (p.N + bn - 1) / bn;
+  const dim3 grid((unsigned)p.tiles_n), block(T_THREADS + 64 * T_PW);
+  if (bn == 128) hipLaunchKernelGGL((fp8_gemm_dma3_q_kernel<128, 6>), grid, block, 0, stream, p);
+  else if (bn == 192) hipLaunchKernelGGL((fp8_gemm_dma3_q_kernel<192, 4>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((fp8_gemm_dma3_q_kernel<256, 3>), grid, block, 0, stream, p);
+  return check_launch(what);
 }
 
 // The same kernels for packed power-of-two (UE8M0) scales on both operands, applied by the MFMA (see dma3_tile).

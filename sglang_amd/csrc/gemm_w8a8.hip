@@ -1035,6 +1035,19 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
   // Decode sizes: the GEMM kernel quantizes the tokens of each K range itself (same arithmetic), no quantizer launch -
   // except where a quantizer launch in front of the wave-split kernel is measured faster (route_constants.h).
   const bool ptr_ok = x_dtype != MI355_F32 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && ldw % 16 == 0;
+  if (ptr_ok && M <= 16) {
+    const Route plain = choose_route(true, M, N, K, K, ldw, true);
+    if (plain.kernel == RK_DMA3) {  // one round of unsplit 64-token tiles: a producer wave of that kernel quantizes the tokens
+      GemmParams p;
+      bool empty;
+      const int rc = fp8_mm_params(what, x, w, w_scale, w_scale, out, out_dtype, M, N, K, K, ldw, 1, (M + 3) & ~3ll, ws_sn, ws_sk, ldo, p, empty);
+      if (rc != MI355_OK || empty) return rc;
+      p.bias = bias;
+      p.x16 = x, p.ldx = K, p.x_dtype = x_dtype;
+      p.kb_total = K / KSTEP, p.splits = 1, p.kb_per_split = p.kb_total;
+      return launch_fp8_dma3_quant(p, plain.bn, static_cast<hipStream_t>(stream), what);
+    }
+  }
   if (ptr_ok && choose_route(true, M, N, K, K, ldw, true, true).kernel == RK_DECODE && fused_quant_preferred(M, N, K, ldw)) {
     GemmParams p;
     bool empty;
@@ -1063,8 +1076,10 @@ extern "C" int mi355_fp8_block_linear_plan(int64_t M, int64_t N, int64_t K, char
   MI355_REQUIRE(buf != nullptr && buf_len > 0, MI355_ERR_INVALID_ARGUMENT, "%s: no buffer", what);
   MI355_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && K % KSTEP == 0,
                 MI355_ERR_INVALID_ARGUMENT, "%s: shape out of range (K must be a multiple of 128)", what);
-  const bool fused = choose_route(true, M, N, K, K, K, true, true).kernel == RK_DECODE && fused_quant_preferred(M, N, K, K);
-  const Route r = choose_route(true, M, N, K, K, K, true, fused);
+  const Route plain = choose_route(true, M, N, K, K, K, true);
+  const bool producer = M <= 16 && plain.kernel == RK_DMA3;  // the mid-M kernel's producer wave quantizes
+  const bool fused = producer || (choose_route(true, M, N, K, K, K, true, true).kernel == RK_DECODE && fused_quant_preferred(M, N, K, K));
+  const Route r = producer ? plain : choose_route(true, M, N, K, K, K, true, fused);
   const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d stages=%d quantizer=%s",
                          ROUTE_NAMES[r.kernel], r.bm, r.bn, r.splits, r.kb_per_split, r.groups_per_wg, (int)r.aligned,
                          route_stages(true, r, M, N), fused ? "fused" : "launch");

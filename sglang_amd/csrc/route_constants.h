@@ -80,7 +80,10 @@ struct RouteConstants {
   double decode_dma3_int8_min_tokens = 12.0;
   double decode_dma3_int8_min_workgroups = 130.0;
   double decode_dma3_min_workgroups = 170.0;  // unsplit tiles (of the channel width that gives most), at most one per CU: 192 and more measured, 144 not enough
-  // ---- one-call linear at decode sizes: the streaming kernel with the quantizer in its prologue (one launch) against a
+  // ---- one-call linear at decode sizes.  Where the GEMM's plan is the mid-M kernel (above), that kernel's producer waves
+  //      quantize the tokens: fused / quantizer launch + GEMM, us: 7168->36864 M=8 50.7 / 53.6, 16 51.5 / 54.0; 1536->24576 M=16
+  //      13.7 / 15.1; 4096->28672 33.6 / 35.0; 1152->53248 17.8 / 20.7.  Otherwise:
+  //      the streaming kernel with the quantizer in its prologue (one launch) against a
   //      quantizer launch + the wave-split kernel, where that is the GEMM's plan.  FP8, median call, us, fused / two launches:
   //      7168->36864: M=1 52.0/52.3, 4 54.6/56.2, 8 58.3/58.6;  18432->7168: M=1 30.8/30.1, 4 32.1/30.4, 8 33.6/31.6, 16 36.6/34.8;
   //      1536->24576: M=1 13.5/15.5, 4 14.0/15.7, 8 15.1/16.3;  7168->4096: M=1 11.9/13.7, 8 13.5/14.5, 16 16.0/15.9;

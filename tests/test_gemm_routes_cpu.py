@@ -130,7 +130,7 @@ def test_block_linear_plan():
 
     from sglang_amd import _lib
 
-    for shape, want in (((1, 36864, 7168), ("fused", "decode")), ((3, 36864, 7168), ("fused", "decode")), ((8, 36864, 7168), ("launch", "dma3")),
+    for shape, want in (((1, 36864, 7168), ("fused", "decode")), ((3, 36864, 7168), ("fused", "decode")), ((8, 36864, 7168), ("fused", "dma3")),
                         ((16, 2048, 7168), ("fused", "decode")), ((8, 7168, 2048), ("fused", "decode")),
                         ((4, 7168, 18432), ("launch", "decode_wavesplit")), ((16, 7168, 2048), ("launch", "decode_wavesplit")),
                         ((128, 7168, 2048), ("launch", "dma3")), ((4, 1000, 1024), ("launch", "generic"))):

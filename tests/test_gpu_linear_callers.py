@@ -123,7 +123,8 @@ def test_fused_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (12, 2048, 7168), (14, 16640, 4480), (8, 4096, 18432), (16, 512, 512), (5, 66048, 512),
-                                   (9, 256, 128), (4, 7168, 18432), (16, 7168, 2048)])
+                                   (9, 256, 128), (4, 7168, 18432), (16, 7168, 2048),
+                                   (16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280)])
 def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype):
     """At decode sizes the one-call linear has no quantizer launch: the streaming decode kernel quantizes the tokens of
     each K range in its prologue.  Same arithmetic on the same codes and scales as quantizer + GEMM in two steps, so where
@@ -131,7 +132,9 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
     channel groups per workgroup, a short last K range, rows past M).  Where the two-step GEMM takes the wave-split decode
     kernel instead (M = 1 here) the sums are added in another order and both are held to the oracle.  The last two shapes
     (K of 144 blocks; K of 16 blocks with 16 tokens) are ones where the one-call linear itself launches the quantizer and
-    the wave-split kernel, being faster there: identical to the two steps again."""
+    the wave-split kernel, being faster there: identical to the two steps again.  The five after them take the mid-M kernel on
+    one round of unsplit 64-token tiles (128-, 192- and 256-channel tiles: six, four and three stages; K of 12, 45, 9, 9 and
+    10 blocks), whose producer wave quantizes the tokens: identical to quantizer + that kernel."""
     from sglang_amd import _lib
     from sglang_amd.fp8_kernel import per_token_group_quant_fp8
     from sglang_amd.fp8_utils import fused_w8a8_block_fp8_linear as w8a8_block_fp8_linear
@@ -139,9 +142,10 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
 
     kernel = _lib.gemm_plan("fp8", M, N, K)["kernel"]
     two_launches = (M, N, K) in ((4, 7168, 18432), (16, 7168, 2048))
-    assert kernel == ("decode_wavesplit" if M == 1 or two_launches else "decode")
+    producer = (M, N, K) in ((16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280))
+    assert kernel == ("dma3" if producer else "decode_wavesplit" if M == 1 or two_launches else "decode")
     lin = _lib.block_linear_plan(M, N, K)
-    assert (lin["quantizer"], lin["kernel"]) == (("launch", "decode_wavesplit") if two_launches else ("fused", "decode"))
+    assert (lin["quantizer"], lin["kernel"]) == (("fused", "dma3") if producer else ("launch", "decode_wavesplit") if two_launches else ("fused", "decode"))
     x = make_activation(M, K, seed=M + N, dtype=dtype)
     x[0, :128] = 0  # a group of zeros: scale 1e-10 / 448, codes 0
     w_q, w_s = make_fp8_weight(N, K, seed=K)
@@ -150,7 +154,7 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
     q, s = per_token_group_quant_fp8(xg, 128, column_major_scales=True)
     two_step = fp8_blockwise_scaled_mm(q, wg.t(), s, sg.t(), dtype)
     assert fused.dtype == dtype
-    if kernel == "decode" or two_launches:
+    if kernel in ("decode", "dma3") or two_launches:
         assert torch.equal(fused.view(torch.int16), two_step.view(torch.int16))
     xq, xs = oracle.group_quant(x, 128, mode="div")
     ref, mag = oracle.fp8_blockwise_mm(xq, w_q, xs, w_s, torch.float32, want_abs=True)
