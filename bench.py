@@ -874,6 +874,10 @@ def main():
                 for nm, (K, N) in DSV3_MLP.items():
                     also.append(bench_fp8_gemm(nm, M, K, N, S, W, False))
             also.append(bench_fp8_gemm("single_linear", 16, 7168, 2048, S, W, cpu, w8a16_cpu=cpu))
+            # the whole decode linear bf16 -> bf16 in one call (quantizer inside the GEMM kernel) on the gate_up / down shapes
+            for M in (1, 8):
+                for nm, (K, N) in DSV3_MLP.items():
+                    also.append(bench_fp8_linear(M, K, N, S, W, False))
             for M in (1, 256, 4096):
                 for nm, (K, N) in LLAMA3_8B.items():
                     also.append(bench_int8_gemm(nm, M, K, N, S, W, with_cpu=(cpu and M == 4096 and nm == "gate_up")))
