@@ -1,3 +1,4 @@
+#include <cstdlib>
 // Blockwise-scaled FP8 GEMM and per-token/per-channel INT8 GEMM for gfx950 (MI355X).
 //
 // One LDS-staged MFMA skeleton serves both:
@@ -424,6 +425,20 @@ bool wavesplit_preferred(bool is_fp8, int64_t M, int64_t N, int64_t K) {
   return (double)M <= ((double)(K / KSTEP) > rc.wavesplit_two_tile_long_k_blocks ? rc.wavesplit_long_k_max_tokens : rc.wavesplit_two_tile_max_tokens);
 }
 
+// The mid-M kernel at decode sizes: the channel tile that gives the most unsplit 64-token tiles in one round (at most one per
+// CU, at least the measured minimum), 0 if none does.
+int decode_dma3_channel_tile(bool is_fp8, int64_t N) {
+  const RouteConstants& rc = route_constants();
+  const double min_workgroups = is_fp8 ? rc.decode_dma3_min_workgroups : rc.decode_dma3_int8_min_workgroups;
+  int bn = 0;
+  int64_t most = 0;
+  for (int c = 256; c >= 128; c -= is_fp8 ? 64 : 128) {
+    const int64_t tiles = (N + c - 1) / c;
+    if ((double)tiles >= min_workgroups && tiles <= NUM_CUS && tiles > most) most = tiles, bn = c;
+  }
+  return bn;
+}
+
 // `aligned`: both operand base pointers and row strides are multiples of 16 bytes and K % 16 == 0.
 // `fused_quant`: the tokens arrive unquantized and the kernel is to quantize them itself, which only the streaming
 // decode kernel can.
@@ -439,14 +454,7 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
     // long K.  INT8: from a dozen tokens on.
     const RouteConstants& rc = route_constants();
     if ((double)M >= (is_fp8 ? rc.decode_dma3_min_tokens : rc.decode_dma3_int8_min_tokens)) {
-      // the channel tile: the one that gives the most workgroups in one round
-      const double min_workgroups = is_fp8 ? rc.decode_dma3_min_workgroups : rc.decode_dma3_int8_min_workgroups;
-      int bn = 0;
-      int64_t most = 0;
-      for (int c = 256; c >= 128; c -= is_fp8 ? 64 : 128) {
-        const int64_t tiles = (N + c - 1) / c;
-        if ((double)tiles >= min_workgroups && tiles <= NUM_CUS && tiles > most) most = tiles, bn = c;
-      }
+      const int bn = decode_dma3_channel_tile(is_fp8, N);
       const bool instead = !is_fp8 ? true
                            : to_wavesplit ? (bn == 192 && (double)(K / KSTEP) > rc.decode_dma3_wavesplit_min_kblocks)
                                           : (decode_supported(M, N, K) && decode_splits(M, N, K) > 1);
@@ -651,7 +659,7 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
     "wavesplit_two_tile_long_k_blocks", "wavesplit_two_tile_max_tokens", "wavesplit_long_k_max_tokens",
     "decode_dma3_min_tokens", "decode_dma3_wavesplit_min_kblocks", "decode_dma3_int8_min_tokens", "decode_dma3_int8_min_workgroups",
     "decode_dma3_min_workgroups",
-    "fused_quant_long_k_blocks", "fused_quant_short_k_blocks", "fused_quant_short_k_max_tokens"};
+    "linear_producer_min_decode_splits", "fused_quant_long_k_blocks", "fused_quant_short_k_blocks", "fused_quant_short_k_max_tokens"};
 
 // LDS stages of the mid-M kernel's pipeline for this plan (0 for the other kernels, whose depth is fixed).
 int route_stages(bool is_fp8, const Route& r, int64_t M, int64_t N) {
@@ -991,6 +999,23 @@ size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 // One-call linear where the streaming decode kernel can quantize the tokens itself: is that faster than a quantizer launch
 // plus the kernel the GEMM alone would take?  Always where that kernel is the streaming one (a launch saved, nothing else
 // changes); against the wave-split kernel by measurement.
+// One-call linear at decode sizes: the mid-M kernel with producer waves where the GEMM alone takes that kernel, and beyond:
+// for fewer tokens than the GEMM's own threshold on the same shape, and where the streaming kernel would split K into many
+// ranges (the alternatives here are the streaming kernel with the quantizer in its prologue or two launches, not the bare
+// wave-split kernel).  Returns the GEMM's plan otherwise.
+Route linear_producer_route(int64_t M, int64_t N, int64_t K, int64_t ldw) {
+  Route plain = choose_route(true, M, N, K, K, ldw, true);
+  if (plain.kernel == RK_DMA3 || M > 16 || K % KSTEP != 0 || N * ldw >= (1ll << 32)) return plain;
+  const RouteConstants& rc = route_constants();
+  const int bn = decode_dma3_channel_tile(true, N);
+  if (bn == 0) return plain;
+  const bool few_tokens = (double)M < rc.decode_dma3_min_tokens &&
+                          choose_route(true, (int64_t)rc.decode_dma3_min_tokens, N, K, K, ldw, true).kernel == RK_DMA3;
+  const bool many_ranges = decode_supported(M, N, K) && (double)decode_splits(M, N, K) >= rc.linear_producer_min_decode_splits;
+  if (few_tokens || many_ranges) plain.kernel = RK_DMA3, plain.bm = 64, plain.bn = bn, plain.splits = 1, plain.kb_per_split = (int)(K / KSTEP);
+  return plain;
+}
+
 bool fused_quant_preferred(int64_t M, int64_t N, int64_t K, int64_t ldw) {
   const int plain = choose_route(true, M, N, K, K, ldw, true).kernel;
   if (plain == RK_DMA3) return false;  // the mid-M kernel at decode sizes beats the streaming kernel by more than a launch
@@ -1036,8 +1061,8 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
   // except where a quantizer launch in front of the wave-split kernel is measured faster (route_constants.h).
   const bool ptr_ok = x_dtype != MI355_F32 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && ldw % 16 == 0;
   if (ptr_ok && M <= 16) {
-    const Route plain = choose_route(true, M, N, K, K, ldw, true);
-    if (plain.kernel == RK_DMA3) {  // one round of unsplit 64-token tiles: a producer wave of that kernel quantizes the tokens
+    const Route plain = linear_producer_route(M, N, K, ldw);
+    if (plain.kernel == RK_DMA3) {  // one round of unsplit 64-token tiles: producer waves of that kernel quantize the tokens
       GemmParams p;
       bool empty;
       const int rc = fp8_mm_params(what, x, w, w_scale, w_scale, out, out_dtype, M, N, K, K, ldw, 1, (M + 3) & ~3ll, ws_sn, ws_sk, ldo, p, empty);
@@ -1076,8 +1101,8 @@ extern "C" int mi355_fp8_block_linear_plan(int64_t M, int64_t N, int64_t K, char
   MI355_REQUIRE(buf != nullptr && buf_len > 0, MI355_ERR_INVALID_ARGUMENT, "%s: no buffer", what);
   MI355_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && K % KSTEP == 0,
                 MI355_ERR_INVALID_ARGUMENT, "%s: shape out of range (K must be a multiple of 128)", what);
-  const Route plain = choose_route(true, M, N, K, K, K, true);
-  const bool producer = M <= 16 && plain.kernel == RK_DMA3;  // the mid-M kernel's producer wave quantizes
+  const Route plain = linear_producer_route(M, N, K, K);
+  const bool producer = M <= 16 && plain.kernel == RK_DMA3;  // the mid-M kernel's producer waves quantize
   const bool fused = producer || (choose_route(true, M, N, K, K, K, true, true).kernel == RK_DECODE && fused_quant_preferred(M, N, K, K));
   const Route r = producer ? plain : choose_route(true, M, N, K, K, K, true, fused);
   const int n = snprintf(buf, buf_len, "kernel=%s bm=%d bn=%d splits=%d kb_per_split=%d groups_per_wg=%d aligned=%d stages=%d quantizer=%s",

@@ -88,6 +88,11 @@ struct RouteConstants {
   //      7168->36864: M=1 52.0/52.3, 4 54.6/56.2, 8 58.3/58.6;  18432->7168: M=1 30.8/30.1, 4 32.1/30.4, 8 33.6/31.6, 16 36.6/34.8;
   //      1536->24576: M=1 13.5/15.5, 4 14.0/15.7, 8 15.1/16.3;  7168->4096: M=1 11.9/13.7, 8 13.5/14.5, 16 16.0/15.9;
   //      7168->2048: M=1 10.3/13.2, 8 12.2/14.5;  2048->7168: M=1 10.5/11.5, 4 10.9/11.9, 8 12.2/12.0, 16 14.4/11.8.
+  //      Beyond the GEMM's own plan the producer-wave kernel also takes the linear for fewer tokens on the same shapes
+  //      (7168->36864 M=1 / 2 / 3: 50.2 / 50.2 / 50.3 against 52.0 / 53.4 / 54.7 on the fused streaming kernel) and where the
+  //      streaming kernel would cut K into many ranges (7168->24576, seven: M=1 / 8 / 12 36.5 / 37.2 / 37.8 against 37.9 / 42.3 /
+  //      44.4; not 4096->28672, four: M=1 32.3 against 29.6; two ranges: 1536->24576 13.1 against 13.5, 2048->32768 18.3 / 18.9)
+  double linear_producer_min_decode_splits = 5.0;
   double fused_quant_long_k_blocks = 64.0;       // beyond this many K blocks the two launches win
   double fused_quant_short_k_blocks = 16.0;      // up to this many K blocks they win too,
   double fused_quant_short_k_max_tokens = 8.0;   // ... above this many tokens

@@ -91,7 +91,7 @@ def test_perturbed_plan_query():
 
     L = _lib.lib()
     n = L.mi355_route_constant_count()
-    assert n == 51 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
+    assert n == 52 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
     assert _lib.route_constants()["pp_fp8_us_per_kblock"] == 1.39
     buf = ctypes.create_string_buffer(256)
     assert L.mi355_gemm_plan_perturbed(1, 128, 7168, 18432, 1, n, 1.1, buf, len(buf)) == 1
@@ -124,13 +124,16 @@ def test_plan_query_rejects_bad_arguments():
 
 
 def test_block_linear_plan():
-    """The one-call linear quantizes inside the streaming decode kernel, except where a quantizer launch in front of the
-    wave-split kernel was measured faster (long K; short K with more than eight tokens) and beyond decode sizes."""
+    """The one-call linear quantizes inside the GEMM kernel - the mid-M kernel's producer waves where one round of unsplit tiles
+    fills the chip (and K would make many ranges for the streaming kernel), else the streaming decode kernel's prologue -
+    except where a quantizer launch in front of the wave-split kernel was measured faster (long K; short K with more than
+    eight tokens) and beyond decode sizes."""
     import ctypes
 
     from sglang_amd import _lib
 
-    for shape, want in (((1, 36864, 7168), ("fused", "decode")), ((3, 36864, 7168), ("fused", "decode")), ((8, 36864, 7168), ("fused", "dma3")),
+    for shape, want in (((1, 36864, 7168), ("fused", "dma3")), ((3, 36864, 7168), ("fused", "dma3")), ((8, 36864, 7168), ("fused", "dma3")),
+                        ((1, 28672, 4096), ("fused", "decode")), ((8, 24576, 7168), ("fused", "dma3")),
                         ((16, 2048, 7168), ("fused", "decode")), ((8, 7168, 2048), ("fused", "decode")),
                         ((4, 7168, 18432), ("launch", "decode_wavesplit")), ((16, 7168, 2048), ("launch", "decode_wavesplit")),
                         ((128, 7168, 2048), ("launch", "dma3")), ((4, 1000, 1024), ("launch", "generic"))):

@@ -124,7 +124,8 @@ def test_fused_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (12, 2048, 7168), (14, 16640, 4480), (8, 4096, 18432), (16, 512, 512), (5, 66048, 512),
                                    (9, 256, 128), (4, 7168, 18432), (16, 7168, 2048),
-                                   (16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280)])
+                                   (16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280),
+                                   (2, 36864, 5760), (3, 24576, 5120)])
 def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype):
     """At decode sizes the one-call linear has no quantizer launch: the streaming decode kernel quantizes the tokens of
     each K range in its prologue.  Same arithmetic on the same codes and scales as quantizer + GEMM in two steps, so where
@@ -134,7 +135,8 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
     (K of 144 blocks; K of 16 blocks with 16 tokens) are ones where the one-call linear itself launches the quantizer and
     the wave-split kernel, being faster there: identical to the two steps again.  The five after them take the mid-M kernel on
     one round of unsplit 64-token tiles (128-, 192- and 256-channel tiles: six, four and three stages; K of 12, 45, 9, 9 and
-    10 blocks), whose producer wave quantizes the tokens: identical to quantizer + that kernel."""
+    10 blocks), whose producer waves quantize the tokens: identical to quantizer + that kernel; the last two take it for the linear only
+    (fewer tokens than the GEMM's own threshold; K of five ranges for the streaming kernel)."""
     from sglang_amd import _lib
     from sglang_amd.fp8_kernel import per_token_group_quant_fp8
     from sglang_amd.fp8_utils import fused_w8a8_block_fp8_linear as w8a8_block_fp8_linear
@@ -143,9 +145,10 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
     kernel = _lib.gemm_plan("fp8", M, N, K)["kernel"]
     two_launches = (M, N, K) in ((4, 7168, 18432), (16, 7168, 2048))
     producer = (M, N, K) in ((16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280))
-    assert kernel == ("dma3" if producer else "decode_wavesplit" if M == 1 or two_launches else "decode")
+    linear_only = (M, N, K) in ((2, 36864, 5760), (3, 24576, 5120))  # the GEMM alone takes the wave-split kernel, the linear the producers
+    assert kernel == ("dma3" if producer else "decode_wavesplit" if M == 1 or two_launches or linear_only else "decode")
     lin = _lib.block_linear_plan(M, N, K)
-    assert (lin["quantizer"], lin["kernel"]) == (("fused", "dma3") if producer else ("launch", "decode_wavesplit") if two_launches else ("fused", "decode"))
+    assert (lin["quantizer"], lin["kernel"]) == (("fused", "dma3") if producer or linear_only else ("launch", "decode_wavesplit") if two_launches else ("fused", "decode"))
     x = make_activation(M, K, seed=M + N, dtype=dtype)
     x[0, :128] = 0  # a group of zeros: scale 1e-10 / 448, codes 0
     w_q, w_s = make_fp8_weight(N, K, seed=K)
