@@ -1,4 +1,3 @@
-#include <cstdlib>
 // Blockwise-scaled FP8 GEMM and per-token/per-channel INT8 GEMM for gfx950 (MI355X).
 //
 // One LDS-staged MFMA skeleton serves both:
