@@ -73,16 +73,17 @@ __device__ __forceinline__ void k_step(const U8State<BM, BN>& s, const uint8_t* 
   }
 }
 
-template <int LOADS>
+// Everything but the YOUNGER youngest loads has landed; then the workgroup barrier.
+template <int YOUNGER>
 __device__ __forceinline__ void wait_and_barrier() {
-  static_assert(LOADS >= 3 && LOADS <= 6, "(BM + BN) / 64");
-  if constexpr (LOADS == 6) asm volatile("s_waitcnt vmcnt(6)\n\ts_barrier" ::: "memory");
-  else if constexpr (LOADS == 5) asm volatile("s_waitcnt vmcnt(5)\n\ts_barrier" ::: "memory");
-  else if constexpr (LOADS == 4) asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(3)\n\ts_barrier" ::: "memory");
+  static_assert(YOUNGER >= 3 && YOUNGER <= 24, "(stages - 2) x LOADS, LOADS = (BM + BN) / 64");
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(YOUNGER) : "memory");
 }
 
-template <int BM, bool SPLIT, int BN>
+// S: LDS stages.  Three; four for 128 x 128 tiles (32 KB a stage: the workgroup has the CU to itself either way); six for
+// 64 x 128 tiles where the launch has at most one workgroup per CU (otherwise two workgroups of three stages share the CU),
+// then with one barrier per two K blocks - as in the FP8 kernel of the same structure (gemm_fp8_dma3.hip).
+template <int BM, bool SPLIT, int BN, int S = 3>
 __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmParams p) {
   static_assert(BN == 128 || BN == 256, "channel tile");
   constexpr int WM = BM / 2, MT = WM / 16, U_WN = BN / 4, U_NT = U_WN / 16, LOADS = U8State<BM, BN>::LOADS;
@@ -98,11 +99,15 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
   const int kb_end = min(p.kb_total, kb_begin + p.kb_per_split);
   const int nkb = kb_end - kb_begin;
 
-  // three stages of (BM token rows + BN channel rows) x 128 bytes, sized per tile shape: a 64 x 128 tile takes 72 KB, so
-  // two such workgroups share a CU's 160 KB
-  __shared__ __attribute__((aligned(1024))) uint8_t u_stage0[(BM + BN) * KSTEP];
-  __shared__ __attribute__((aligned(1024))) uint8_t u_stage1[(BM + BN) * KSTEP];
-  __shared__ __attribute__((aligned(1024))) uint8_t u_stage2[(BM + BN) * KSTEP];
+  // S stages of (BM token rows + BN channel rows) x 128 bytes, sized per tile shape: three stages of a 64 x 128 tile take
+  // 72 KB, so two such workgroups share a CU's 160 KB
+  static_assert(S >= 3 && S * (BM + BN) * KSTEP <= 160 * 1024, "the stages must fit the CU's LDS");
+  __shared__ __attribute__((aligned(1024))) uint8_t u_stage[S][(BM + BN) * KSTEP];
+  // PAIRED (six stages): one barrier per two K blocks; iteration k requests block k + S - 2 into the stage that iteration
+  // k - 2 read, and the wait in front of the barrier covers the two blocks of the next pair
+  constexpr bool PAIRED = S == 6;
+  constexpr int AHEAD = PAIRED ? S - 2 : S - 1;
+  constexpr int YOUNGER = (PAIRED ? S - 4 : S - 2) * LOADS;
   U8State<BM, BN> s;
   s.wave = wave;
   s.kb_last = kb_end - 1;
@@ -136,24 +141,25 @@ __global__ __launch_bounds__(U_THREADS) void int8_gemm_dma3_kernel(const GemmPar
     for (int j = 0; j < MT; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
 #pragma unroll
-  for (int i = 0; i < LOADS; ++i) issue_one<BM, BN>(s, i, u_stage0, kb_begin);
+  for (int b = 0; b < AHEAD; ++b)
 #pragma unroll
-  for (int i = 0; i < LOADS; ++i) issue_one<BM, BN>(s, i, u_stage1, kb_begin + 1);
-  wait_and_barrier<LOADS>();
+    for (int i = 0; i < LOADS; ++i) issue_one<BM, BN>(s, i, u_stage[b], kb_begin + b);
+  wait_and_barrier<YOUNGER>();
 
   int k = 0;
-  for (; k + 2 < nkb; k += 3) {
-    k_step<BM, BN>(s, u_stage0, acc, u_stage2, kb_begin + k + 2);
-    wait_and_barrier<LOADS>();
-    k_step<BM, BN>(s, u_stage1, acc, u_stage0, kb_begin + k + 3);
-    wait_and_barrier<LOADS>();
-    k_step<BM, BN>(s, u_stage2, acc, u_stage1, kb_begin + k + 4);
-    wait_and_barrier<LOADS>();
+  for (; k + S - 1 < nkb; k += S) {
+#pragma unroll
+    for (int u = 0; u < S; ++u) {
+      k_step<BM, BN>(s, u_stage[u], acc, u_stage[(u + AHEAD) % S], kb_begin + k + u + AHEAD);
+      if (!PAIRED || (u & 1)) wait_and_barrier<YOUNGER>();
+    }
   }
-  if (k < nkb) {
-    k_step<BM, BN>(s, u_stage0, acc, u_stage2, kb_begin + k + 2);
-    wait_and_barrier<LOADS>();
-    if (k + 1 < nkb) k_step<BM, BN>(s, u_stage1, acc, u_stage0, kb_begin + k + 3);
+#pragma unroll
+  for (int u = 0; u < S - 1; ++u) {  // up to S - 1 blocks left, in stages 0 ..
+    if (k + u < nkb) {
+      k_step<BM, BN>(s, u_stage[u], acc, u_stage[(u + AHEAD) % S], kb_begin + k + u + AHEAD);
+      if ((!PAIRED || (u & 1)) && k + u + 1 < nkb) wait_and_barrier<YOUNGER>();
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // stray refetches must not outlive the workgroup's LDS
 
@@ -208,10 +214,14 @@ int launch_bm(GemmParams& p, hipStream_t stream, const char* what) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const dim3 grid((unsigned)(p.tiles_m * p.tiles_n * p.splits));
-  if (p.splits > 1)
-    hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, true, BN>), grid, dim3(U_THREADS), 0, stream, p);
-  else
-    hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, false, BN>), grid, dim3(U_THREADS), 0, stream, p);
+  if (BM + BN == 192 && (int64_t)p.tiles_m * p.tiles_n * p.splits > NUM_CUS) {
+    if (p.splits > 1) hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, true, BN, 3>), grid, dim3(U_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, false, BN, 3>), grid, dim3(U_THREADS), 0, stream, p);
+  } else {
+    constexpr int S = BM + BN == 192 ? 6 : BM + BN == 256 ? 4 : 3;
+    if (p.splits > 1) hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, true, BN, S>), grid, dim3(U_THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((int8_gemm_dma3_kernel<BM, false, BN, S>), grid, dim3(U_THREADS), 0, stream, p);
+  }
   return check_launch(what);
 }
 

@@ -664,7 +664,7 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
 int route_stages(bool is_fp8, const Route& r, int64_t M, int64_t N) {
   if (r.kernel != RK_DMA3) return 0;
   const int64_t workgroups = ((M + r.bm - 1) / r.bm) * ((N + r.bn - 1) / r.bn) * r.splits;
-  return is_fp8 ? dma3_stages(r.bm, r.bn, workgroups) : 3;
+  return dma3_stages(r.bm, r.bn, workgroups);  // the INT8 kernel of the same structure follows the same rule
 }
 
 int describe_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len, const char* what) {

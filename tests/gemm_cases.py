@@ -97,7 +97,9 @@ INT8_REQUIRED_VARIANTS = {
     ("decode_wavesplit", "w4", "one_round"), ("decode_wavesplit", "w4", "rounds"), ("decode_wavesplit", "w8", "one_round"),
     ("decode_wavesplit", "w8", "rounds"),
     ("dma3", 64, "whole"), ("dma3", 64, "split"), ("pingpong128", "whole"), ("pingpong128", "split"),
-    ("dma3", 64, "whole", "bn128"), ("dma3", 64, "split", "bn128"), ("dma3", 128, "whole", "bn128"), ("dma3", 128, "split", "bn128"),
+    # (the 128-channel tiles always run more than three stages: 128 x 128 four, 64 x 128 six - the plan puts 64 x 128 tiles only
+    # where the launch has at most one workgroup per CU)
+    ("dma3", 64, "whole", "bn128", "deep"), ("dma3", 64, "split", "bn128", "deep"), ("dma3", 128, "whole", "bn128", "deep"), ("dma3", 128, "split", "bn128", "deep"),
     ("pingpong", "kfull"),
     ("generic", 16, "aligned", "whole"), ("generic", 32, "aligned", "split"), ("generic", 64, "aligned", "whole"),
     ("generic", 128, "aligned", "whole"), ("generic", 128, "aligned", "split"), ("generic", 256, "aligned", "whole"),
