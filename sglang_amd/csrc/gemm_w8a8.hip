@@ -452,7 +452,8 @@ Route choose_route(bool is_fp8, int64_t M, int64_t N, int64_t K, int64_t lda, in
     // of the streaming kernel whenever that one would split K, instead of the wave-split kernel with 192-channel tiles and
     // long K.  INT8: from a dozen tokens on.
     const RouteConstants& rc = route_constants();
-    if ((double)M >= (is_fp8 ? rc.decode_dma3_min_tokens : rc.decode_dma3_int8_min_tokens)) {
+    const bool long_k = (double)(K / KSTEP) > rc.decode_dma3_wavesplit_min_kblocks;
+    if ((double)M >= (is_fp8 ? rc.decode_dma3_min_tokens : long_k ? rc.decode_dma3_int8_long_k_min_tokens : rc.decode_dma3_int8_min_tokens)) {
       const int bn = decode_dma3_channel_tile(is_fp8, N);
       const bool instead = !is_fp8 ? true
                            : to_wavesplit ? (bn == 192 && (double)(K / KSTEP) > rc.decode_dma3_wavesplit_min_kblocks)
@@ -656,7 +657,8 @@ const char* const ROUTE_CONSTANT_NAMES[ROUTE_CONSTANT_COUNT] = {
     "dma3_small_tile_factor", "wavesplit_min_kblocks", "wavesplit_small_weight_bytes", "wavesplit_small_weight_max_tokens",
     "wavesplit_large_weight_max_tokens", "wavesplit_two_tile_min_workgroups", "wavesplit_two_tile_min_tokens",
     "wavesplit_two_tile_long_k_blocks", "wavesplit_two_tile_max_tokens", "wavesplit_long_k_max_tokens",
-    "decode_dma3_min_tokens", "decode_dma3_wavesplit_min_kblocks", "decode_dma3_int8_min_tokens", "decode_dma3_int8_min_workgroups",
+    "decode_dma3_min_tokens", "decode_dma3_wavesplit_min_kblocks", "decode_dma3_int8_long_k_min_tokens", "decode_dma3_int8_min_tokens",
+    "decode_dma3_int8_min_workgroups",
     "decode_dma3_min_workgroups",
     "linear_producer_min_decode_splits", "fused_quant_long_k_blocks", "fused_quant_short_k_blocks", "fused_quant_short_k_max_tokens"};
 

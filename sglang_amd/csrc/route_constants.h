@@ -77,7 +77,9 @@ struct RouteConstants {
   // launch, us, wave-split / mid-M kernel at M = 4 / 8 / 16: 7168->24576 37.6 / 42.2 / 50.5 against 37.9 / 37.6 / 38.3,
   // 2048->32768 16.2 / 18.1 / 21.1 against 17.4 / 17.4 / 17.8, 7168->36864 (144 tiles of 256 channels) 54.3 / 61.8 / 74.6
   // against 58.3 / 58.5 / 59.6, 4096->28672 25.5 / 27.3 / 33.0 against 31.9 / 31.9 / 32.1
-  double decode_dma3_int8_min_tokens = 12.0;
+  // (with six stages for the 64 x 128 tile: 7168->24576 35.5 / 35.6 / 36.2, 7168->36864 58.5 / 58.6 / 59.5, 4096->28672 31.2 / 31.1 / 31.4)
+  double decode_dma3_int8_long_k_min_tokens = 8.0;  // ... from here on where K has more blocks than decode_dma3_wavesplit_min_kblocks,
+  double decode_dma3_int8_min_tokens = 12.0;        // ... from here on for any K
   double decode_dma3_int8_min_workgroups = 130.0;
   double decode_dma3_min_workgroups = 170.0;  // unsplit tiles (of the channel width that gives most), at most one per CU: 192 and more measured, 144 not enough
   // ---- one-call linear at decode sizes.  Where the GEMM's plan is the mid-M kernel (above), that kernel's producer waves

@@ -76,7 +76,7 @@ INT8_ROUTE_SHAPES = [
     (16, 128, 512), (1, 6144, 4096), (1, 16640, 4480), (9, 33280, 2176), (16, 7168, 18432), (7, 33280, 4096),
     (5, 66048, 512), (2, 133120, 384),
     # a dozen tokens or more on the mid-M kernel where one round of unsplit 64-token tiles fills the chip (128- and 256-channel tiles)
-    (16, 28672, 512), (13, 36864, 1024), (12, 24576, 2304),
+    (16, 28672, 512), (13, 36864, 1024), (12, 24576, 2304), (8, 24576, 5760),  # (eight tokens where K has more than 44 blocks)
     (20, 8192, 4096), (40, 65536, 512), (200, 16384, 2048), (200, 32768, 1024), (300, 4096, 14336), (130, 8192, 7168),
     (100, 16384, 3584), (500, 4096, 14336),
     # the mid-M kernel's 128-channel tiles (and 128 x 256 with a K split): ragged M, a ragged last channel tile

@@ -91,7 +91,7 @@ def test_perturbed_plan_query():
 
     L = _lib.lib()
     n = L.mi355_route_constant_count()
-    assert n == 52 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
+    assert n == 53 and L.mi355_route_constant_name(n) is None and L.mi355_route_constant_name(-1) is None
     assert _lib.route_constants()["pp_fp8_us_per_kblock"] == 1.39
     buf = ctypes.create_string_buffer(256)
     assert L.mi355_gemm_plan_perturbed(1, 128, 7168, 18432, 1, n, 1.1, buf, len(buf)) == 1
