@@ -125,7 +125,7 @@ def test_fused_block_fp8_linear(gpu, oracle, shape, N, K, with_bias):
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 7168), (12, 2048, 7168), (14, 16640, 4480), (8, 4096, 18432), (16, 512, 512), (5, 66048, 512),
                                    (9, 256, 128), (4, 7168, 18432), (16, 7168, 2048),
                                    (16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280),
-                                   (2, 36864, 5760), (3, 24576, 5120)])
+                                   (2, 36864, 5760), (3, 24576, 5120), (8, 36800, 5760)])
 def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype):
     """At decode sizes the one-call linear has no quantizer launch: the streaming decode kernel quantizes the tokens of
     each K range in its prologue.  Same arithmetic on the same codes and scales as quantizer + GEMM in two steps, so where
@@ -144,7 +144,8 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
 
     kernel = _lib.gemm_plan("fp8", M, N, K)["kernel"]
     two_launches = (M, N, K) in ((4, 7168, 18432), (16, 7168, 2048))
-    producer = (M, N, K) in ((16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280))
+    producer = (M, N, K) in ((16, 24576, 1536), (5, 36864, 5760), (13, 53248, 1152), (16, 32768, 1152), (13, 45056, 1280),
+                            (8, 36800, 5760))  # (the last with a ragged last channel tile: 128 of 192 channels)
     linear_only = (M, N, K) in ((2, 36864, 5760), (3, 24576, 5120))  # the GEMM alone takes the wave-split kernel, the linear the producers
     assert kernel == ("dma3" if producer else "decode_wavesplit" if M == 1 or two_launches or linear_only else "decode")
     lin = _lib.block_linear_plan(M, N, K)
