@@ -171,6 +171,29 @@ def test_decode_linear_quantizes_in_the_gemm_kernel(gpu, oracle, M, N, K, dtype)
         assert bool(((out.float().cpu() - ref).abs() <= 1e-2 * ref.abs() + FP8_MAG_TOL * mag).all())
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 53248, 1280), (16, 53248, 1408), (16, 45056, 1408), (16, 32768, 1664), (16, 32768, 1792),
+                                   (16, 32768, 2176)])
+def test_producer_wave_linear_every_tail_length(gpu, M, N, K):
+    """The producer waves and the other waves of the mid-M kernel must meet at the same number of barriers whatever is left of K
+    after whole trips over the stages: three stages with 1 and 2 blocks left, four with 3, six with 1, 2 and 5 (0 and the other
+    remainders are in the test above).  Bit-identical to quantizer + GEMM."""
+    from sglang_amd import _lib
+    from sglang_amd.fp8_kernel import per_token_group_quant_fp8
+    from sglang_amd.fp8_utils import fused_w8a8_block_fp8_linear
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    lin = _lib.block_linear_plan(M, N, K)
+    assert (lin["kernel"], lin["quantizer"]) == ("dma3", "fused") and (K // 128) % lin["stages"] != 0
+    print(f"case M={M} N={N} K={K}: {lin}", flush=True)
+    x = make_activation(M, K, seed=N + K)
+    w_q, w_s = make_fp8_weight(N, K, seed=K)
+    xg, wg, sg = x.to(gpu), w_q.to(gpu), w_s.to(gpu)
+    fused = fused_w8a8_block_fp8_linear(xg, wg, [128, 128], sg)
+    q, s = per_token_group_quant_fp8(xg, 128, column_major_scales=True)
+    two_step = fp8_blockwise_scaled_mm(q, wg.t(), s, sg.t(), torch.bfloat16)
+    assert torch.equal(fused.view(torch.int16), two_step.view(torch.int16))
+
+
 def test_block_fp8_linear_ragged_n_falls_back_to_the_triton_wrapper(gpu, oracle):
     """N not a multiple of 128: the CUTLASS-style wrapper hands over to the Triton-style one (fp8_utils.py:195-201),
     i.e. `x * (1 / s)` codes; K must be a multiple of the group size for either quantizer."""
