@@ -33,6 +33,9 @@ FP8_ROUTE_SHAPES = [
     # decode sizes on the mid-M kernel (4 .. 16 tokens, one round of unsplit tiles): instead of the wave-split kernel with
     # 192-channel tiles, instead of the split streaming kernel with 128- and 256-channel tiles
     (4, 36864, 7168), (13, 36864, 7168), (16, 24576, 1536), (14, 32768, 2048), (16, 49152, 2048),
+    # K blocks left over after whole trips over the stages that no shape above has: 64 x 192 (four stages) 3; 128 x 128 (four) 2 and
+    # 3; 128 x 192 and 128 x 256 (three; loader waves) 0
+    (20, 36864, 896), (100, 32768, 768), (100, 32768, 896), (100, 36864, 768), (300, 16384, 768),
     # small tiles with more workgroups than CUs: 64 x 192 and 128 x 128
     (135, 49152, 1024), (198, 36864, 1024),
     # 192-channel tiles (a wave's three channel tiles are 64 channels apart): whole-K and split, a ragged last tile
@@ -77,6 +80,7 @@ INT8_ROUTE_SHAPES = [
     (5, 66048, 512), (2, 133120, 384),
     # a dozen tokens or more on the mid-M kernel where one round of unsplit 64-token tiles fills the chip (128- and 256-channel tiles)
     (16, 28672, 512), (13, 36864, 1024), (12, 24576, 2304), (8, 24576, 5760),  # (eight tokens where K has more than 44 blocks)
+    (400, 6144, 896),  # 128 x 128 tiles (four stages) with three K blocks left after whole trips
     (20, 8192, 4096), (40, 65536, 512), (200, 16384, 2048), (200, 32768, 1024), (300, 4096, 14336), (130, 8192, 7168),
     (100, 16384, 3584), (500, 4096, 14336),
     # the mid-M kernel's 128-channel tiles (and 128 x 256 with a K split): ragged M, a ragged last channel tile
