@@ -382,6 +382,12 @@ size_t mi355_fp8_block_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w, const float* w_scale, int64_t ws_sn, int64_t ws_sk,
                            const void* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldw,
                            int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
+/* The same with the quantizer's arithmetic chosen: MI355_QUANT_DIV as above (fp8_utils.py:201-203, the M-major-scale path),
+ * MI355_QUANT_RCP for q = x * (1 / s), which is what triton_w8a8_block_fp8_linear's quantizer computes (fp8_utils.py:293-295,
+ * fp8_kernel.py:156-158).  Either way the result is bit-identical to that wrapper's quantizer followed by the blockwise GEMM. */
+int mi355_fp8_block_linear_mode(const void* x, int x_dtype, int quant_mode, const void* w, const float* w_scale, int64_t ws_sn,
+                                int64_t ws_sk, const void* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
 int mi355_fp8_block_linear_plan(int64_t M, int64_t N, int64_t K, char* buf, size_t buf_len);
 
 #ifdef __cplusplus

@@ -31,6 +31,7 @@ struct GemmParams {
   const void* x16;         // FP8 decode kernel only, optional: unquantized tokens [M, K] (x_dtype, row stride ldx elements);
   int64_t ldx;             // when set, the kernel quantizes them per 1 x 128 group itself and ignores a / sa
   int x_dtype;
+  int x_by_reciprocal;     // the fused quantizer computes q = x * (1 / s) instead of q = x / s
   void* out;
   void* ws;  // split-K partial tiles: [splits][M][N] fp32 or int32
   int M, N, K;
@@ -72,8 +73,9 @@ __device__ __forceinline__ float div_by_shared(float x, float s, float r) {
   return q;
 }
 // The lane's eight 16-bit elements (raw) of a group spread over its DPP row -> their eight e4m3fn codes and the group's scale
-// (the same value in all 16 lanes).  Every lane of the row must be active.
-__device__ __forceinline__ u32x2 quantize_group_lane(const u32x4& raw, int x_dtype, float& scale) {
+// (the same value in all 16 lanes).  Every lane of the row must be active.  by_reciprocal: q = x * (1 / s) as the
+// reference's row-major-scale quantizer computes it (fp8_kernel.py:156-158), else the true division of its M-major one.
+__device__ __forceinline__ u32x2 quantize_group_lane(const u32x4& raw, int x_dtype, bool by_reciprocal, float& scale) {
   const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
   float v[8];
 #pragma unroll
@@ -89,7 +91,7 @@ __device__ __forceinline__ u32x2 quantize_group_lane(const u32x4& raw, int x_dty
   const float rcp = 1.0f / sc;
   float t[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) t[e] = fminf(fmaxf(div_by_shared(v[e], sc, rcp), -448.0f), 448.0f);
+  for (int e = 0; e < 8; ++e) t[e] = fminf(fmaxf(by_reciprocal ? v[e] * rcp : div_by_shared(v[e], sc, rcp), -448.0f), 448.0f);
   int c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[0], t[1], 0, false);
   c0 = __builtin_amdgcn_cvt_pk_fp8_f32(t[2], t[3], c0, true);
   int c1 = __builtin_amdgcn_cvt_pk_fp8_f32(t[4], t[5], 0, false);

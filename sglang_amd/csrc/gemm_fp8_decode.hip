@@ -176,7 +176,7 @@ __device__ __forceinline__ void quantize_tokens(const GemmParams& p, int kb_begi
     const int pair = r + 16 * j, m = pair / KBP, d = pair % KBP;
     if (m >= p.M) break;  // uniform over the 16-lane row, which is all the DPP reduction below involves
     float sc;
-    const u32x2 codes = quantize_group_lane(raw[j], p.x_dtype, sc);
+    const u32x2 codes = quantize_group_lane(raw[j], p.x_dtype, p.x_by_reciprocal != 0, sc);
     const bool valid = kb_begin + d < p.kb_total;  // blocks past the end of K: zero tokens, zero scale
     *reinterpret_cast<u32x2*>(tok + d * TOK_BLOCK + m * KSTEP + (((gl >> 1) ^ (m & 7)) << 4) + (gl & 1) * 8) =
         valid ? codes : u32x2{0u, 0u};

@@ -536,7 +536,7 @@ __device__ __forceinline__ void dma3_tile_q(const GemmParams& p, int n0) {
     };
     auto produce = [&](int stage, const u32x4& raw) {
       float sc;
-      const u32x2 codes = quantize_group_lane(raw, p.x_dtype, sc);
+      const u32x2 codes = quantize_group_lane(raw, p.x_dtype, p.x_by_reciprocal != 0, sc);
       *reinterpret_cast<u32x2*>(&t_stage[stage][m * KSTEP + (((gl >> 1) ^ (m & 7)) << 4) + (gl & 1) * 8]) = codes;
       if (gl == 0) t_scale[stage][m] = sc;
     };

@@ -1034,12 +1034,13 @@ extern "C" size_t mi355_fp8_block_linear_workspace_bytes(int64_t M, int64_t N, i
   return align256((size_t)M * (size_t)K) + align256((size_t)((M + 3) & ~3ll) * kb * 4u) + workspace_bytes(M, N, K, true);
 }
 
-extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w, const float* w_scale, int64_t ws_sn,
-                                      int64_t ws_sk, const void* bias, void* out, int out_dtype, int64_t M, int64_t N,
-                                      int64_t K, int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes_given,
-                                      void* stream) {
-  const char* what = "mi355_fp8_block_linear";
+namespace {
+int block_linear(const char* what, const void* x, int x_dtype, int quant_mode, const void* w, const float* w_scale, int64_t ws_sn,
+                 int64_t ws_sk, const void* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldw,
+                 int64_t ldo, void* workspace, size_t workspace_bytes_given, void* stream) {
   clear_error();
+  MI355_REQUIRE(quant_mode == MI355_QUANT_DIV || quant_mode == MI355_QUANT_RCP, MI355_ERR_INVALID_ARGUMENT,
+                "%s: quant_mode must be MI355_QUANT_DIV or MI355_QUANT_RCP", what);
   MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
   MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16, MI355_ERR_INVALID_ARGUMENT,
                 "%s: out_dtype must be bfloat16 or float16", what);
@@ -1069,7 +1070,7 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
       const int rc = fp8_mm_params(what, x, w, w_scale, w_scale, out, out_dtype, M, N, K, K, ldw, 1, (M + 3) & ~3ll, ws_sn, ws_sk, ldo, p, empty);
       if (rc != MI355_OK || empty) return rc;
       p.bias = bias;
-      p.x16 = x, p.ldx = K, p.x_dtype = x_dtype;
+      p.x16 = x, p.ldx = K, p.x_dtype = x_dtype, p.x_by_reciprocal = quant_mode == MI355_QUANT_RCP;
       p.kb_total = K / KSTEP, p.splits = 1, p.kb_per_split = p.kb_total;
       return launch_fp8_dma3_quant(p, plain.bn, static_cast<hipStream_t>(stream), what);
     }
@@ -1081,11 +1082,12 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
     int rc = fp8_mm_params(what, x, w, w_scale, w_scale, out, out_dtype, M, N, K, K, ldw, 1, (M + 3) & ~3ll, ws_sn, ws_sk, ldo, p, empty);
     if (rc != MI355_OK || empty) return rc;
     p.bias = bias;
-    p.x16 = x, p.ldx = K, p.x_dtype = x_dtype;
+    p.x16 = x, p.ldx = K, p.x_dtype = x_dtype, p.x_by_reciprocal = quant_mode == MI355_QUANT_RCP;
     return run_gemm<true>(p, workspace, workspace_bytes_given, static_cast<hipStream_t>(stream), what);
   }
-  // quantize with q = x / s, the arithmetic of the reference's column-major path (fp8_kernel.py:164-212 via fp8_utils.py:201-203)
-  int rc = mi355_group_quant_8bit(x, x_dtype, q, MI355_FP8_E4M3FN, sa, M, K, KSTEP, 1e-10f, -448.0f, 448.0f, MI355_QUANT_DIV,
+  // quantize with q = x / s, the arithmetic of the reference's column-major path (fp8_kernel.py:164-212 via fp8_utils.py:201-203),
+  // or with q = x * (1 / s), that of its row-major path (fp8_kernel.py:156-158); the scale layout here is the library's own
+  int rc = mi355_group_quant_8bit(x, x_dtype, q, MI355_FP8_E4M3FN, sa, M, K, KSTEP, 1e-10f, -448.0f, 448.0f, quant_mode,
                                   MI355_SCALE_F32, 0.0f, 1, pitch, stream);
   if (rc != MI355_OK) return rc;
   GemmParams p;
@@ -1094,6 +1096,23 @@ extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w,
   if (rc != MI355_OK || empty) return rc;
   p.bias = bias;
   return run_gemm<true>(p, q + q_bytes + sa_bytes, workspace_bytes_given - q_bytes - sa_bytes, static_cast<hipStream_t>(stream), what);
+}
+}  // namespace
+
+extern "C" int mi355_fp8_block_linear(const void* x, int x_dtype, const void* w, const float* w_scale, int64_t ws_sn,
+                                      int64_t ws_sk, const void* bias, void* out, int out_dtype, int64_t M, int64_t N,
+                                      int64_t K, int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes_given,
+                                      void* stream) {
+  return block_linear("mi355_fp8_block_linear", x, x_dtype, MI355_QUANT_DIV, w, w_scale, ws_sn, ws_sk, bias, out, out_dtype, M, N,
+                      K, ldw, ldo, workspace, workspace_bytes_given, stream);
+}
+
+extern "C" int mi355_fp8_block_linear_mode(const void* x, int x_dtype, int quant_mode, const void* w, const float* w_scale,
+                                           int64_t ws_sn, int64_t ws_sk, const void* bias, void* out, int out_dtype, int64_t M,
+                                           int64_t N, int64_t K, int64_t ldw, int64_t ldo, void* workspace,
+                                           size_t workspace_bytes_given, void* stream) {
+  return block_linear("mi355_fp8_block_linear_mode", x, x_dtype, quant_mode, w, w_scale, ws_sn, ws_sk, bias, out, out_dtype, M, N,
+                      K, ldw, ldo, workspace, workspace_bytes_given, stream);
 }
 
 extern "C" int mi355_fp8_block_linear_plan(int64_t M, int64_t N, int64_t K, char* buf, size_t buf_len) {

@@ -365,10 +365,12 @@ def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[to
 
 
 def block_fp8_linear(x2d: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
-                     bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+                     bias: Optional[torch.Tensor], out_dtype: torch.dtype, by_reciprocal: bool = False) -> torch.Tensor:
     """One block-FP8 linear layer (1x128 activation groups, 128x128 weight blocks) in one C-ABI call: the activation is
     quantized into the workspace, multiplied, and the bias is added in the GEMM epilogue.  x2d [M, K] contiguous
-    bf16/fp16/fp32 with K % 128 == 0, weight [N, K] e4m3fn, weight_scale [ceil(N/128), K/128] (any strides)."""
+    bf16/fp16/fp32 with K % 128 == 0, weight [N, K] e4m3fn, weight_scale [ceil(N/128), K/128] (any strides).
+    by_reciprocal: the quantizer computes q = x * (1 / s) (the reference's row-major-scale path, fp8_kernel.py:156-158)
+    instead of q = x / s (its M-major-scale path)."""
     _require(x2d.is_cuda and weight.is_cuda, "block_fp8_linear: operands must be CUDA tensors")
     _require(x2d.dim() == 2 and x2d.is_contiguous(), "block_fp8_linear: x must be a contiguous 2-D tensor")
     _require(weight.dim() == 2 and weight.stride(1) == 1 and weight.dtype == torch.float8_e4m3fn,
@@ -388,10 +390,10 @@ def block_fp8_linear(x2d: torch.Tensor, weight: torch.Tensor, weight_scale: torc
     L = lib()
     ws_bytes = _workspace_bytes("mi355_fp8_block_linear_workspace_bytes", int(M), int(N), int(K))
     ws = _workspace(ws_bytes, x2d.device)
-    check(L.mi355_fp8_block_linear(x2d.data_ptr(), _DT[x2d.dtype], weight.data_ptr(), weight_scale.data_ptr(),
-                                   weight_scale.stride(0), weight_scale.stride(1),
-                                   bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype],
-                                   M, N, K, weight.stride(0), out.stride(0), ws.data_ptr(), ws_bytes, _stream()))
+    check(L.mi355_fp8_block_linear_mode(x2d.data_ptr(), _DT[x2d.dtype], 1 if by_reciprocal else 0, weight.data_ptr(),
+                                        weight_scale.data_ptr(), weight_scale.stride(0), weight_scale.stride(1),
+                                        bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype],
+                                        M, N, K, weight.stride(0), out.stride(0), ws.data_ptr(), ws_bytes, _stream()))
     return out
 
 

@@ -90,6 +90,13 @@ def test_newer_entry_points_validate_before_any_device_work():
     assert L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(0, 128, 128) == 0
     need = L.mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(4, 512, 1024)
     assert need > 0 and need % 256 == 0
+    # one-call linear with the quantizer's arithmetic chosen: a known mode, K whole groups, a workspace, empty problem
+    B = L.mi355_fp8_block_linear_mode
+    assert B(p, _lib.BF16, _lib.QUANT_MUL, p, p, 8, 1, None, p, _lib.BF16, 4, 128, 1024, 1024, 128, p, 1 << 20, None) == 1
+    assert b"quant_mode" in L.mi355_last_error()
+    assert B(p, _lib.BF16, _lib.QUANT_RCP, p, p, 8, 1, None, p, _lib.BF16, 4, 128, 1000, 1000, 128, p, 1 << 20, None) == 1
+    assert B(p, _lib.BF16, _lib.QUANT_RCP, p, p, 8, 1, None, p, _lib.BF16, 4, 128, 1024, 1024, 128, None, 0, None) == 4
+    assert B(None, _lib.BF16, _lib.QUANT_DIV, None, None, 8, 1, None, None, _lib.BF16, 0, 128, 1024, 1024, 128, None, 0, None) == 0
     # grouped GEMM: output dtype, K whole blocks, workspace present and large enough, empty problem; queries are pure
     G = L.mi355_fp8_blockwise_scaled_grouped_mm
     tail = (128, 128, 128 * 128, 1, 1, 1, 1, 1, 128)  # lda, ldb, expert stride, scale strides, ldo

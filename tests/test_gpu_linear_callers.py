@@ -18,7 +18,10 @@ def _bias_after_rounding(out_nobias: torch.Tensor, bias: torch.Tensor, oracle) -
 
 
 @pytest.mark.parametrize("shape,N,K", [((2, 5), 384, 512), ((16,), 2048, 7168), ((3, 7), 576, 1024), ((300,), 1088, 384),
-                                       ((1,), 7168, 2048), ((4100,), 1024, 256), ((40,), 200, 384)])
+                                       ((1,), 7168, 2048), ((4100,), 1024, 256), ((40,), 200, 384),
+                                       # decode sizes where the wrappers' one call quantizes inside the GEMM kernel: producer
+                                       # waves of the mid-M kernel, the streaming kernel's prologue (split, with a short last range)
+                                       ((13,), 53248, 1152), ((2, 4), 24576, 1536), ((14,), 16640, 4480), ((8,), 36800, 1280)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_block_fp8_linear_wrappers_follow_the_reference(gpu, oracle, shape, N, K, dtype):
     """The two block-FP8 wrappers of the reference are different computations (fp8_utils.py:184-214 vs :281-301):
