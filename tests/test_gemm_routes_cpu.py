@@ -141,6 +141,13 @@ def test_block_linear_plan():
         assert (p["quantizer"], p["kernel"]) == want, (shape, p)
         if p["quantizer"] == "launch":
             assert {k: v for k, v in p.items() if k != "quantizer"} == _lib.gemm_plan("fp8", *shape)
+    # the reference-named wrappers make the one call only where it multiplies with the GEMM entry point's kernel and tiling:
+    # any plan with a quantizer launch, and the fused plans whose kernel the GEMM entry point takes too
+    from sglang_amd.fp8_utils import _one_call_takes_the_same_gemm
+
+    for shape, want in (((8, 36864, 7168), True), ((16, 2048, 7168), True), ((4, 7168, 18432), True), ((4100, 1024, 256), True),
+                        ((40, 200, 384), True), ((1, 36864, 7168), False), ((8, 24576, 1536), False)):
+        assert _one_call_takes_the_same_gemm(*shape) == want, shape
     buf = ctypes.create_string_buffer(256)
     assert _lib.lib().mi355_fp8_block_linear_plan(4, 1024, 1000, buf, len(buf)) == 1  # K not a multiple of 128
     assert _lib.lib().mi355_fp8_block_linear_plan(4, 1024, 1024, buf, 8) == 1 and b"too small" in _lib.lib().mi355_last_error()
