@@ -390,6 +390,21 @@ int mi355_fp8_block_linear_mode(const void* x, int x_dtype, int quant_mode, cons
                                 int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
 int mi355_fp8_block_linear_plan(int64_t M, int64_t N, int64_t K, char* buf, size_t buf_len);
 
+/*
+ * One INT8 linear layer in one call:  out = int8_scaled_mm(per_token_quant_int8(x), w) with scales and bias in the GEMM epilogue.
+ * Replaces the call sequence of W8A8Int8LinearMethod.apply (python/sglang/srt/layers/quantization/w8a8_int8.py:387-417):
+ *          per_token_quant_int8 (int8_kernel.py:28-89), then int8_scaled_mm (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747).
+ *          The codes and token scales go to the workspace; the result is that of mi355_per_token_quant_int8 followed by
+ *          mi355_int8_scaled_mm, bit for bit (the same two kernels on the same data).
+ *   x [M, K] contiguous F32/F16/BF16, K * sizeof(x element) % 16 == 0; w [N, K] int8 row stride ldw (the reference's
+ *   column-major [K, N]); w_scale [N] fp32; bias NULL or [N] in the output dtype; out [M, N] BF16/F16 row stride ldo.
+ *   workspace: mi355_int8_linear_workspace_bytes(M, N, K) bytes, 256-byte aligned.
+ */
+size_t mi355_int8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_int8_linear(const void* x, int x_dtype, const void* w, const float* w_scale, const void* bias, void* out, int out_dtype,
+                      int64_t M, int64_t N, int64_t K, int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif

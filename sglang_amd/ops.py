@@ -542,6 +542,39 @@ def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[t
     return out
 
 
+def int8_linear(x2d: torch.Tensor, weight_kn: torch.Tensor, weight_scale: torch.Tensor, bias: Optional[torch.Tensor],
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """One INT8 linear layer in one C-ABI call: per-token quantization of x2d [M, K] (contiguous bf16/fp16/fp32) into the
+    workspace, then the INT8 GEMM with `weight_kn` [K, N] int8 column-major, per-channel `weight_scale` ([N] fp32) and bias in
+    its epilogue.  The result is that of `per_token_quant_int8` followed by `int8_scaled_mm`, bit for bit."""
+    _require(x2d.is_cuda and weight_kn.is_cuda, "int8_linear: operands must be CUDA tensors")
+    _require(x2d.dim() == 2 and x2d.is_contiguous(), "int8_linear: x must be a contiguous 2-D tensor")
+    _require(x2d.dtype in (torch.float32, torch.float16, torch.bfloat16), "int8_linear: unsupported input dtype")
+    _require(weight_kn.dim() == 2 and weight_kn.stride(0) == 1 and weight_kn.dtype == torch.int8,
+             "int8_linear: weight must be a column-major Int8 matrix [K, N]")
+    M, K = x2d.shape
+    N = weight_kn.size(1)
+    _require(weight_kn.size(0) == K, "int8_linear: x and weight shapes cannot be multiplied")
+    _require(K % 16 == 0, "int8_linear: K must be multiple of 16 for memory alignment")
+    _require(N % 8 == 0, "int8_linear: N must be multiple of 8 for memory alignment")
+    _require(weight_scale.numel() == N and weight_scale.is_contiguous() and weight_scale.dtype == torch.float32,
+             "int8_linear: weight_scale must be a contiguous Float32 tensor of N elements")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "int8_linear: out_dtype must be Half or BFloat16")
+    if bias is not None:
+        _require(bias.numel() == N and bias.is_contiguous() and bias.dtype == out_dtype,
+                 "int8_linear: bias must be a contiguous [N] tensor of the output dtype")
+    out = torch.empty((M, N), dtype=out_dtype, device=x2d.device)
+    if M == 0:
+        return out
+    L = lib()
+    ws_bytes = _workspace_bytes("mi355_int8_linear_workspace_bytes", int(M), int(N), int(K))
+    ws = _workspace(ws_bytes, x2d.device)
+    check(L.mi355_int8_linear(x2d.data_ptr(), _DT[x2d.dtype], weight_kn.data_ptr(), weight_scale.data_ptr(),
+                              bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype], M, N, K,
+                              weight_kn.stride(1), out.stride(0), ws.data_ptr(), ws_bytes, _stream()))
+    return out
+
+
 def _launch_int8_mm(mat_a, mat_b, scales_a, scales_b, bias, out):
     M, K = mat_a.shape
     N = mat_b.size(1)

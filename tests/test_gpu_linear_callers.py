@@ -212,19 +212,41 @@ def test_block_fp8_linear_ragged_n_falls_back_to_the_triton_wrapper(gpu, oracle)
     assert bool(((out.float().cpu() - ref).abs() <= 1e-2 * ref.abs() + FP8_MAG_TOL * mag).all())
 
 
-@pytest.mark.parametrize("shape,N,K", [((4, 3), 6144, 4096), ((1,), 4096, 14336), ((300,), 264, 512)])
-def test_int8_linear(gpu, oracle, shape, N, K):
+@pytest.mark.parametrize("shape,N,K", [((4, 3), 6144, 4096), ((1,), 4096, 14336), ((300,), 264, 512), ((256,), 4096, 14336),
+                                       ((16,), 28672, 4096), ((2, 64), 6144, 4096), ((5,), 4096, 4112)])
+@pytest.mark.parametrize("dtype,with_bias", [(torch.bfloat16, True), (torch.float16, False)])
+def test_int8_linear(gpu, oracle, shape, N, K, dtype, with_bias):
+    """The INT8 linear method's forward pass (w8a8_int8.py:387-417) is one C-ABI call: the oracle's codes, scales and
+    product bit for bit (integer arithmetic and one rounding), hence also the two operators called one after the other."""
+    from sglang_amd.int8_kernel import per_token_quant_int8
+    from sglang_amd.sgl_kernel import int8_scaled_mm
     from sglang_amd.w8a8_int8 import apply_w8a8_int8_linear
 
     M = 1
     for d in shape:
         M *= d
-    x = make_activation(M, K, seed=N, outlier_frac=0.0).view(*shape, K)
+    x = make_activation(M, K, seed=N, outlier_frac=0.0, dtype=dtype).view(*shape, K)
     w_q, w_s = make_int8_weight(N, K)
     g = torch.Generator().manual_seed(2)
-    bias = torch.randn(N, generator=g).to(torch.bfloat16)
-    out = apply_w8a8_int8_linear(x.to(gpu), w_q.to(gpu).t(), w_s.view(N, 1).to(gpu), bias.to(gpu))
-    assert tuple(out.shape) == (*shape, N) and out.dtype == torch.bfloat16
+    bias = torch.randn(N, generator=g).to(dtype) if with_bias else None
+    xg, wg, sg, bg = x.to(gpu), w_q.to(gpu).t(), w_s.view(N, 1).to(gpu), bias.to(gpu) if with_bias else None
+    out = apply_w8a8_int8_linear(xg, wg, sg, bg)
+    assert tuple(out.shape) == (*shape, N) and out.dtype == dtype
     xq, xs = oracle.per_token_quant_int8(x.view(M, K))
-    want = oracle.int8_scaled_mm(xq, w_q, xs, w_s, torch.bfloat16, bias)
+    want = oracle.int8_scaled_mm(xq, w_q, xs, w_s, dtype, bias)
     assert torch.equal(out.cpu().view(M, N).view(torch.int16), want.view(torch.int16))
+    q, s = per_token_quant_int8(xg.view(M, K))
+    two = int8_scaled_mm(q, wg, s, sg.view(-1), dtype, bg)
+    assert torch.equal(out.view(M, N).view(torch.int16), two.view(torch.int16))
+
+
+def test_int8_linear_leaves_unusual_operands_to_the_operators(gpu):
+    """Operands the one call does not take go through the two operators, which raise the reference's errors."""
+    from sglang_amd.w8a8_int8 import apply_w8a8_int8_linear
+
+    x = torch.randn(4, 512, device=gpu, dtype=torch.bfloat16)
+    w_row_major = torch.zeros(512, 256, device=gpu, dtype=torch.int8)  # [K, N] but not column-major
+    s = torch.ones(256, 1, device=gpu)
+    with pytest.raises(RuntimeError, match="column major"):
+        apply_w8a8_int8_linear(x, w_row_major, s)
+    assert tuple(apply_w8a8_int8_linear(x[:0], w_row_major.t().contiguous().t(), s).shape) == (0, 256)
