@@ -405,6 +405,20 @@ int mi355_int8_linear(const void* x, int x_dtype, const void* w, const float* w_
                       int64_t M, int64_t N, int64_t K, int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes,
                       void* stream);
 
+/*
+ * One per-token x per-channel FP8 linear layer in one call:  out = fp8_scaled_mm(per_token_quant_fp8(x), w).
+ * Replaces the dynamic per-token branch of apply_fp8_linear (python/sglang/srt/layers/quantization/fp8_utils.py:786-808):
+ *          sglang_per_token_quant_fp8 (fp8_kernel.py:573-589), then fp8_scaled_mm.  Codes and token scales go to the
+ *          workspace; the result is that of mi355_per_token_quant_fp8 followed by mi355_fp8_scaled_mm, bit for bit.
+ *   x [M, K] contiguous F32/F16/BF16, K * sizeof(x element) % 16 == 0; w [N, K] e4m3fn row stride ldw; w_scale [N] fp32;
+ *   bias NULL or [N] in the output dtype; out [M, N] BF16/F16 row stride ldo.
+ *   workspace: mi355_fp8_per_token_linear_workspace_bytes(M, N, K) bytes, 256-byte aligned.
+ */
+size_t mi355_fp8_per_token_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_fp8_per_token_linear(const void* x, int x_dtype, const void* w, const float* w_scale, const void* bias, void* out,
+                               int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldw, int64_t ldo, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

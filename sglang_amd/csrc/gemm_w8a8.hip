@@ -1204,6 +1204,39 @@ extern "C" int mi355_int8_linear(const void* x, int x_dtype, const void* w, cons
   return run_gemm<false>(p, q + q_bytes + sa_bytes, workspace_bytes_given - q_bytes - sa_bytes, static_cast<hipStream_t>(stream), what);
 }
 
+extern "C" size_t mi355_fp8_per_token_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  return align256((size_t)M * (size_t)K) + align256((size_t)M * 4u) + mi355_fp8_scaled_mm_workspace_bytes(M, N, K);
+}
+
+extern "C" int mi355_fp8_per_token_linear(const void* x, int x_dtype, const void* w, const float* w_scale, const void* bias,
+                                          void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldw, int64_t ldo,
+                                          void* workspace, size_t workspace_bytes_given, void* stream) {
+  const char* what = "mi355_fp8_per_token_linear";
+  clear_error();
+  MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
+  MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16, MI355_ERR_INVALID_ARGUMENT,
+                "%s: out_dtype must be bfloat16 or float16", what);
+  if (M == 0 || N == 0) return MI355_OK;
+  MI355_REQUIRE(K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), MI355_ERR_INVALID_ARGUMENT,
+                "%s: K must be positive and every dimension fit in 31 bits", what);
+  MI355_REQUIRE(x && w && w_scale && out, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  const size_t need = mi355_fp8_per_token_linear_workspace_bytes(M, N, K);
+  MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
+                "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
+  MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, MI355_ERR_WORKSPACE,
+                "%s: workspace must be 256-byte aligned", what);
+  // workspace: [codes M x K][token scales M][what the GEMM needs]
+  uint8_t* q = static_cast<uint8_t*>(workspace);
+  const size_t q_bytes = align256((size_t)M * (size_t)K);
+  float* sa = reinterpret_cast<float*>(q + q_bytes);
+  const size_t sa_bytes = align256((size_t)M * 4u);
+  const int rc = mi355_per_token_quant_fp8(x, x_dtype, q, sa, M, K, stream);
+  if (rc != MI355_OK) return rc;
+  return mi355_fp8_scaled_mm(q, w, sa, w_scale, bias, out, out_dtype, M, N, K, K, ldw, ldo, q + q_bytes + sa_bytes,
+                             workspace_bytes_given - q_bytes - sa_bytes, stream);
+}
+
 extern "C" int mi355_fp8_blockwise_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len) {
   return describe_route(true, M, N, K, aligned, buf, buf_len, "mi355_fp8_blockwise_mm_plan");
 }

@@ -364,6 +364,40 @@ def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[to
     return out
 
 
+def fp8_per_token_linear(x2d: torch.Tensor, weight_kn: torch.Tensor, weight_scale: torch.Tensor, bias: Optional[torch.Tensor],
+                         out_dtype: torch.dtype) -> torch.Tensor:
+    """One per-token x per-channel FP8 linear layer in one C-ABI call: per-token quantization of x2d [M, K] (contiguous
+    bf16/fp16/fp32) into the workspace, then the GEMM with `weight_kn` [K, N] e4m3fn column-major, per-channel `weight_scale`
+    ([N] fp32) and bias in its epilogue.  The result is that of `sgl_per_token_quant_fp8` followed by `fp8_scaled_mm`, bit
+    for bit."""
+    _require(x2d.is_cuda and weight_kn.is_cuda, "fp8_per_token_linear: operands must be CUDA tensors")
+    _require(x2d.dim() == 2 and x2d.is_contiguous(), "fp8_per_token_linear: x must be a contiguous 2-D tensor")
+    _require(x2d.dtype in (torch.float32, torch.float16, torch.bfloat16), "fp8_per_token_linear: unsupported input dtype")
+    _require(weight_kn.dim() == 2 and weight_kn.stride(0) == 1 and weight_kn.dtype == torch.float8_e4m3fn,
+             "fp8_per_token_linear: weight must be a column-major Float8_e4m3fn matrix [K, N]")
+    M, K = x2d.shape
+    N = weight_kn.size(1)
+    _require(weight_kn.size(0) == K, "fp8_per_token_linear: x and weight shapes cannot be multiplied")
+    _require(K % 16 == 0, "fp8_per_token_linear: K must be multiple of 16 bytes for memory alignment")
+    _require(weight_scale.numel() == N and weight_scale.is_contiguous() and weight_scale.dtype == torch.float32,
+             "fp8_per_token_linear: weight_scale must be a contiguous Float32 tensor of N elements")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "fp8_per_token_linear: out_dtype must be Half or BFloat16")
+    _require(N % 8 == 0, "fp8_per_token_linear: out must be multiple of 16 bytes for memory alignment")
+    if bias is not None:
+        _require(bias.numel() == N and bias.is_contiguous() and bias.dtype == out_dtype,
+                 "fp8_per_token_linear: bias must be a contiguous [N] tensor of the output dtype")
+    out = torch.empty((M, N), dtype=out_dtype, device=x2d.device)
+    if M == 0:
+        return out
+    L = lib()
+    ws_bytes = _workspace_bytes("mi355_fp8_per_token_linear_workspace_bytes", int(M), int(N), int(K))
+    ws = _workspace(ws_bytes, x2d.device)
+    check(L.mi355_fp8_per_token_linear(x2d.data_ptr(), _DT[x2d.dtype], weight_kn.data_ptr(), weight_scale.data_ptr(),
+                                       bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype], M, N, K,
+                                       weight_kn.stride(1), out.stride(0), ws.data_ptr(), ws_bytes, _stream()))
+    return out
+
+
 def block_fp8_linear(x2d: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
                      bias: Optional[torch.Tensor], out_dtype: torch.dtype, by_reciprocal: bool = False) -> torch.Tensor:
     """One block-FP8 linear layer (1x128 activation groups, 128x128 weight blocks) in one C-ABI call: the activation is

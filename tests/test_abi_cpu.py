@@ -105,6 +105,13 @@ def test_newer_entry_points_validate_before_any_device_work():
     assert I(p, _lib.BF16, p, p, None, p, _lib.BF16, 4, 128, 1024, 1024, 128, None, 0, None) == 4
     assert I(None, _lib.BF16, None, None, None, None, _lib.BF16, 0, 128, 1024, 1024, 128, None, 0, None) == 0
     assert L.mi355_int8_linear_workspace_bytes(0, 128, 1024) == 0 and L.mi355_int8_linear_workspace_bytes(4, 128, 1024) % 256 == 0
+    # one-call per-token FP8 linear: output dtype, workspace, empty problem
+    T = L.mi355_fp8_per_token_linear
+    assert T(p, _lib.BF16, p, p, None, p, _lib.F32, 4, 128, 1024, 1024, 128, p, 1 << 20, None) == 1
+    assert T(p, _lib.BF16, p, p, None, p, _lib.BF16, 4, 128, 1024, 1024, 128, None, 0, None) == 4
+    assert T(p, _lib.BF16, p, p, None, p, _lib.BF16, 4, 128, 1024, 1024, 128, p, 16, None) == 4
+    assert T(None, _lib.BF16, None, None, None, None, _lib.BF16, 0, 128, 1024, 1024, 128, None, 0, None) == 0
+    assert L.mi355_fp8_per_token_linear_workspace_bytes(4, 128, 1024) % 256 == 0
     # grouped GEMM: output dtype, K whole blocks, workspace present and large enough, empty problem; queries are pure
     G = L.mi355_fp8_blockwise_scaled_grouped_mm
     tail = (128, 128, 128 * 128, 1, 1, 1, 1, 1, 128)  # lda, ldb, expert stride, scale strides, ldo

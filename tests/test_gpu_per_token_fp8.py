@@ -107,10 +107,14 @@ def test_fp8_scaled_mm_exact_integers(gpu):
         assert torch.equal(out.cpu().double(), want.to(torch.bfloat16).double()), (M, N, K)
 
 
-@pytest.mark.parametrize("shape,N,K", [((2, 5), 384, 512), ((1,), 6144, 4096), ((700,), 1024, 2048)])
+@pytest.mark.parametrize("shape,N,K", [((2, 5), 384, 512), ((1,), 6144, 4096), ((700,), 1024, 2048), ((4096,), 1024, 1024),
+                                       ((16,), 18432, 7168), ((5,), 264, 400)])
 def test_apply_fp8_linear(gpu, oracle, shape, N, K):
-    """apply_fp8_linear: per-token quantization then fp8_scaled_mm, against the oracle's pipeline and the unquantized linear."""
+    """apply_fp8_linear: per-token quantization then fp8_scaled_mm (one C-ABI call for both), against the oracle's pipeline,
+    the unquantized linear, and the two operators called one after the other (bit for bit)."""
+    from sglang_amd.fp8_kernel import sglang_per_token_quant_fp8
     from sglang_amd.fp8_utils import apply_fp8_linear
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
 
     M = 1
     for d in shape:
@@ -129,3 +133,6 @@ def test_apply_fp8_linear(gpu, oracle, shape, N, K):
     check_fp8_gemm(out.view(M, N), ref, mag, "apply_fp8_linear")
     full = x.view(M, K).float() @ w.T + bias.float()
     assert float((out.float().cpu().view(M, N) - full).norm() / full.norm()) < 0.05
+    q, s = sglang_per_token_quant_fp8(x.to(gpu).view(M, K))
+    two = fp8_scaled_mm(q, w_q.to(gpu).t(), s, w_s.to(gpu), torch.bfloat16, bias.to(gpu))
+    assert torch.equal(out.view(M, N).view(torch.int16), two.view(torch.int16))
