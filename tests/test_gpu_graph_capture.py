@@ -172,3 +172,51 @@ def test_grouped_gemm_replays_with_new_routing(gpu, oracle):
                 if m:
                     ref, mag = oracle.fp8_blockwise_mm(a[r0:r0 + m], w[e], sa[r0:r0 + m], sw[e], torch.float32, want_abs=True)
                     check_fp8_gemm(got[r0:r0 + m], ref, mag, f"replay {e}")
+
+
+@pytest.mark.parametrize("M,N,K", [(4, 1024, 2048), (12, 1024, 2048), (13, 53248, 1152), (48, 1024, 2048)])
+def test_linear_methods_replay(gpu, M, N, K):
+    """The linear layers as the reference's methods call them - both block-FP8 wrappers (one C-ABI call each: the quantizer in the
+    streaming kernel's prologue, producer waves of the mid-M kernel, or a quantizer launch), the per-token FP8 linear and the INT8
+    linear - captured once and replayed with new inputs: every replay equals the eager result of the same input bit for bit."""
+    from sglang_amd import _lib
+    from sglang_amd.fp8_utils import apply_fp8_linear, cutlass_w8a8_block_fp8_linear_with_fallback, triton_w8a8_block_fp8_linear
+    from sglang_amd.w8a8_int8 import apply_w8a8_int8_linear
+
+    print(f"case M={M}: {_lib.block_linear_plan(M, N, K)}", flush=True)
+    N2 = 512
+    w_q, w_s = make_fp8_weight(N, K, seed=31)
+    wi_q, wi_s = make_int8_weight(N2, K, seed=32)
+    w_q, w_s, wi_q, wi_s = w_q.to(gpu), w_s.to(gpu), wi_q.to(gpu).t(), wi_s.to(gpu)
+    wc = w_q[:N2].t()  # [K, N2] column-major view for the per-token FP8 linear
+    sc = torch.rand(N2, device=gpu) * 1e-2 + 1e-4
+    bias = torch.randn(N2, device=gpu).to(torch.bfloat16)
+
+    def chain(x):
+        return (cutlass_w8a8_block_fp8_linear_with_fallback(x, w_q, [128, 128], w_s),
+                triton_w8a8_block_fp8_linear(x, w_q, [128, 128], w_s),
+                apply_fp8_linear(x, wc, sc, bias=bias),
+                apply_w8a8_int8_linear(x, wi_q, wi_s, bias))
+
+    inputs = [make_activation(M, K, seed=300 + i) for i in range(3)]
+    static_x = inputs[0].to(gpu).clone()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(2):
+            chain(static_x)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            static_out = chain(static_x)
+    torch.cuda.synchronize()
+    for i, x in enumerate(inputs[1:] + inputs[:1]):
+        static_x.copy_(x.to(gpu))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in static_out]
+        want = chain(x.to(gpu))
+        torch.cuda.synchronize()
+        for name, g_, w_ in zip(("cutlass-style", "triton-style", "per-token fp8", "int8"), got, want):
+            assert torch.equal(g_.view(torch.int16), w_.view(torch.int16)), (i, name)
+            assert bool(torch.isfinite(g_).all())
