@@ -419,6 +419,23 @@ int mi355_fp8_per_token_linear(const void* x, int x_dtype, const void* w, const 
                                int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldw, int64_t ldo, void* workspace,
                                size_t workspace_bytes, void* stream);
 
+/*
+ * One block-FP8 linear layer with packed power-of-two scales in one call:
+ *   out = mi355_fp8_blockwise_mm_ue8m0(quantize_1x128_ue8m0(x), w).
+ * Replaces the call sequence of deepgemm_w8a8_block_fp8_linear_with_fallback (python/sglang/srt/layers/quantization/
+ *          fp8_utils.py:217-255): sglang_per_token_group_quant_fp8(column_major_scales, scale_tma_aligned, scale_ue8m0)
+ *          (q = x * (448 / amax), scale rounded up to a power of two: per_token_group_quant_8bit_v2.cu:77-78), then the
+ *          GEMM.  Codes and packed token words go to the workspace; the result is that of mi355_group_quant_8bit with
+ *          those arguments followed by mi355_fp8_blockwise_mm_ue8m0, bit for bit.
+ *   x [M, K] contiguous F16/BF16, K % 128 == 0; w [N, K] e4m3fn row stride ldw; sb_words as for mi355_fp8_blockwise_mm_ue8m0;
+ *   bias NULL or [N] in the output dtype (added in the epilogue); out [M, N] BF16/F16 row stride ldo.
+ *   workspace: mi355_fp8_block_linear_ue8m0_workspace_bytes(M, N, K) bytes, 256-byte aligned.
+ */
+size_t mi355_fp8_block_linear_ue8m0_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mi355_fp8_block_linear_ue8m0(const void* x, int x_dtype, const void* w, const void* sb_words, int64_t sb_sn, int64_t sb_sk,
+                                 const void* bias, void* out, int out_dtype, int64_t M, int64_t N, int64_t K, int64_t ldw,
+                                 int64_t ldo, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -61,6 +61,8 @@ EXPORTS = (
     "mi355_int8_linear",
     "mi355_fp8_per_token_linear_workspace_bytes",
     "mi355_fp8_per_token_linear",
+    "mi355_fp8_block_linear_ue8m0_workspace_bytes",
+    "mi355_fp8_block_linear_ue8m0",
 )
 
 _lib = None
@@ -163,6 +165,10 @@ def lib() -> ctypes.CDLL:
     L.mi355_fp8_per_token_linear_workspace_bytes.restype = sz
     L.mi355_fp8_per_token_linear.argtypes = [vp, i32, vp, vp, vp, vp, i32] + [i64] * 5 + [vp, sz, vp]
     L.mi355_fp8_per_token_linear.restype = i32
+    L.mi355_fp8_block_linear_ue8m0_workspace_bytes.argtypes = [i64, i64, i64]
+    L.mi355_fp8_block_linear_ue8m0_workspace_bytes.restype = sz
+    L.mi355_fp8_block_linear_ue8m0.argtypes = [vp, i32, vp, vp, i64, i64, vp, vp, i32] + [i64] * 5 + [vp, sz, vp]
+    L.mi355_fp8_block_linear_ue8m0.restype = i32
     L.mi355_route_constant_count.restype = i32
     L.mi355_route_constant_name.argtypes = [i32]
     L.mi355_route_constant_name.restype = ctypes.c_char_p

@@ -1237,6 +1237,45 @@ extern "C" int mi355_fp8_per_token_linear(const void* x, int x_dtype, const void
                              workspace_bytes_given - q_bytes - sa_bytes, stream);
 }
 
+extern "C" size_t mi355_fp8_block_linear_ue8m0_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  const size_t words = (size_t)(((K + KSTEP - 1) / KSTEP + 3) / 4);
+  return align256((size_t)M * (size_t)K) + align256((size_t)((M + 3) & ~3ll) * words * 4u) +
+         mi355_fp8_blockwise_mm_ue8m0_workspace_bytes(M, N, K);
+}
+
+extern "C" int mi355_fp8_block_linear_ue8m0(const void* x, int x_dtype, const void* w, const void* sb_words, int64_t sb_sn,
+                                            int64_t sb_sk, const void* bias, void* out, int out_dtype, int64_t M, int64_t N,
+                                            int64_t K, int64_t ldw, int64_t ldo, void* workspace, size_t workspace_bytes_given,
+                                            void* stream) {
+  const char* what = "mi355_fp8_block_linear_ue8m0";
+  clear_error();
+  MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, MI355_ERR_INVALID_ARGUMENT, "%s: negative shape", what);
+  MI355_REQUIRE(out_dtype == MI355_BF16 || out_dtype == MI355_F16, MI355_ERR_INVALID_ARGUMENT,
+                "%s: out_dtype must be bfloat16 or float16", what);
+  if (M == 0 || N == 0) return MI355_OK;
+  MI355_REQUIRE(K > 0 && K % KSTEP == 0, MI355_ERR_INVALID_ARGUMENT,
+                "%s: K must be a positive multiple of the quantization group (128)", what);
+  MI355_REQUIRE(x && w && sb_words && out, MI355_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+  const size_t need = mi355_fp8_block_linear_ue8m0_workspace_bytes(M, N, K);
+  MI355_REQUIRE(workspace != nullptr && workspace_bytes_given >= need, MI355_ERR_WORKSPACE,
+                "%s: needs a workspace of %zu bytes, got %zu", what, need, workspace_bytes_given);
+  MI355_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, MI355_ERR_WORKSPACE,
+                "%s: workspace must be 256-byte aligned", what);
+  // workspace: [codes M x K][token scale words, packed along tokens, pitch align4(M)][what the GEMM needs]
+  uint8_t* q = static_cast<uint8_t*>(workspace);
+  const size_t q_bytes = align256((size_t)M * (size_t)K);
+  void* sa_words = q + q_bytes;
+  const int64_t pitch = (M + 3) & ~3ll;
+  const size_t sa_bytes = align256((size_t)pitch * (size_t)((K / KSTEP + 3) / 4) * 4u);
+  // q = x * (448 / amax) with the scale rounded up to a power of two: per_token_group_quant_8bit_v2.cu:77-78 with scale_ue8m0
+  const int rc = mi355_group_quant_8bit(x, x_dtype, q, MI355_FP8_E4M3FN, sa_words, M, K, KSTEP, 1e-10f, -448.0f, 448.0f,
+                                        MI355_QUANT_MUL, MI355_SCALE_UE8M0_PACKED, 0.0f, 1, pitch, stream);
+  if (rc != MI355_OK) return rc;
+  return mi355_fp8_blockwise_mm_ue8m0(q, w, sa_words, sb_words, bias, out, out_dtype, M, N, K, K, ldw, pitch, sb_sn, sb_sk, ldo,
+                                      q + q_bytes + sa_bytes, workspace_bytes_given - q_bytes - sa_bytes, stream);
+}
+
 extern "C" int mi355_fp8_blockwise_mm_plan(int64_t M, int64_t N, int64_t K, int aligned, char* buf, size_t buf_len) {
   return describe_route(true, M, N, K, aligned, buf, buf_len, "mi355_fp8_blockwise_mm_plan");
 }

@@ -364,6 +364,41 @@ def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias: Optional[to
     return out
 
 
+def block_fp8_linear_ue8m0(x2d: torch.Tensor, weight: torch.Tensor, weight_words: torch.Tensor, bias: Optional[torch.Tensor],
+                           out_dtype: torch.dtype) -> torch.Tensor:
+    """One block-FP8 linear layer with packed power-of-two scales in one C-ABI call: x2d [M, K] (contiguous bf16/fp16,
+    K % 128 == 0) is quantized per 1 x 128 group with UE8M0 scales into the workspace and multiplied with `weight` [N, K]
+    e4m3fn, whose packed scale words are `weight_words` int32 [N, ceil(K/512)] (fp8_utils.transform_scale_ue8m0).  The
+    result is that of the quantizer call of deepgemm_w8a8_block_fp8_linear_with_fallback followed by
+    `fp8_blockwise_mm_ue8m0`, bit for bit."""
+    _require(x2d.is_cuda and weight.is_cuda, "block_fp8_linear_ue8m0: operands must be CUDA tensors")
+    _require(x2d.dim() == 2 and x2d.is_contiguous() and x2d.dtype in (torch.bfloat16, torch.float16),
+             "block_fp8_linear_ue8m0: x must be a contiguous 2-D bf16/fp16 tensor")
+    _require(weight.dim() == 2 and weight.stride(1) == 1 and weight.dtype == torch.float8_e4m3fn,
+             "block_fp8_linear_ue8m0: weight must be a row-major Float8_e4m3fn matrix")
+    M, K = x2d.shape
+    N = weight.size(0)
+    _require(weight.size(1) == K and K % 128 == 0, "block_fp8_linear_ue8m0: K must match and be a multiple of 128")
+    kw = (K // 128 + 3) // 4
+    _require(weight_words.dtype == torch.int32 and weight_words.dim() == 2 and weight_words.size(0) == N and weight_words.size(1) >= kw,
+             f"block_fp8_linear_ue8m0: weight_words must be int32 [{N}, >= {kw}]")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "block_fp8_linear_ue8m0: out_dtype must be Half or BFloat16")
+    if bias is not None:
+        _require(bias.numel() == N and bias.is_contiguous() and bias.dtype == out_dtype,
+                 "block_fp8_linear_ue8m0: bias must be a contiguous [N] tensor of the output dtype")
+    out = torch.empty((M, N), dtype=out_dtype, device=x2d.device)
+    if M == 0 or N == 0:
+        return out
+    L = lib()
+    ws_bytes = _workspace_bytes("mi355_fp8_block_linear_ue8m0_workspace_bytes", int(M), int(N), int(K))
+    ws = _workspace(ws_bytes, x2d.device)
+    check(L.mi355_fp8_block_linear_ue8m0(x2d.data_ptr(), _DT[x2d.dtype], weight.data_ptr(), weight_words.data_ptr(),
+                                         weight_words.stride(0), weight_words.stride(1),
+                                         bias.data_ptr() if bias is not None else None, out.data_ptr(), _DT[out_dtype],
+                                         M, N, K, weight.stride(0), out.stride(0), ws.data_ptr(), ws_bytes, _stream()))
+    return out
+
+
 def fp8_per_token_linear(x2d: torch.Tensor, weight_kn: torch.Tensor, weight_scale: torch.Tensor, bias: Optional[torch.Tensor],
                          out_dtype: torch.dtype) -> torch.Tensor:
     """One per-token x per-channel FP8 linear layer in one C-ABI call: per-token quantization of x2d [M, K] (contiguous

@@ -112,6 +112,13 @@ def test_newer_entry_points_validate_before_any_device_work():
     assert T(p, _lib.BF16, p, p, None, p, _lib.BF16, 4, 128, 1024, 1024, 128, p, 16, None) == 4
     assert T(None, _lib.BF16, None, None, None, None, _lib.BF16, 0, 128, 1024, 1024, 128, None, 0, None) == 0
     assert L.mi355_fp8_per_token_linear_workspace_bytes(4, 128, 1024) % 256 == 0
+    # one-call block-FP8 linear with packed scales: output dtype, K whole groups, workspace, empty problem
+    U = L.mi355_fp8_block_linear_ue8m0
+    assert U(p, _lib.BF16, p, p, 1, 128, None, p, _lib.F32, 4, 128, 1024, 1024, 128, p, 1 << 20, None) == 1
+    assert U(p, _lib.BF16, p, p, 1, 128, None, p, _lib.BF16, 4, 128, 1000, 1000, 128, p, 1 << 20, None) == 1
+    assert U(p, _lib.BF16, p, p, 1, 128, None, p, _lib.BF16, 4, 128, 1024, 1024, 128, None, 0, None) == 4
+    assert U(None, _lib.BF16, None, None, 1, 128, None, None, _lib.BF16, 0, 128, 1024, 1024, 128, None, 0, None) == 0
+    assert L.mi355_fp8_block_linear_ue8m0_workspace_bytes(4, 128, 1024) % 256 == 0
     # grouped GEMM: output dtype, K whole blocks, workspace present and large enough, empty problem; queries are pure
     G = L.mi355_fp8_blockwise_scaled_grouped_mm
     tail = (128, 128, 128 * 128, 1, 1, 1, 1, 1, 128)  # lda, ldb, expert stride, scale strides, ldo

@@ -195,11 +195,11 @@ def test_ue8m0_decode_exact_integers(gpu, oracle, M, N, K):
     _exact_integer_case(gpu, oracle, M, N, K)
 
 
-@pytest.mark.parametrize("M", [8, 4096])
-def test_deepgemm_linear_wrapper(gpu, oracle, M):
+@pytest.mark.parametrize("M,N,K", [(8, 4352, 512), (4096, 4352, 512), (12, 2048, 7168), (200, 1024, 640), (8, 36864, 1152)])
+def test_deepgemm_linear_wrapper(gpu, oracle, M, N, K):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul_deepgemm
     from sglang_amd.fp8_utils import deepgemm_w8a8_block_fp8_linear_with_fallback, requant_weight_ue8m0
 
-    N, K = 4352, 512
     w_q, w_s = make_fp8_weight(N, K, seed=9)
     w2, sb_words = requant_weight_ue8m0(w_q.to(gpu), w_s.to(gpu), [128, 128])
     x = make_activation(M, K, seed=10)
@@ -210,10 +210,16 @@ def test_deepgemm_linear_wrapper(gpu, oracle, M):
     q_o, s_o = oracle.group_quant(v, 128, mode="mul", layout="ue8m0")
     sa = torch.exp2(oracle.unpack_ue8m0(s_o, K // 128).float() - 127.0)
     sb = torch.exp2(_unpack_bytes(sb_words, K // 128).float() - 127.0)[::128].contiguous()
-    rows = torch.arange(M) if M <= 64 else torch.tensor([0, 1, 255, 256, 4095])
+    rows = torch.arange(M) if M <= 64 else torch.tensor([0, 1, 255 % M, 256 % M, M - 1])
     ref, mag = oracle.fp8_blockwise_mm(q_o[rows].contiguous(), w2.cpu(), sa[rows].contiguous(), sb, torch.float32, want_abs=True)
     # the wrapper rounds the product to bf16 and then adds the bias (fp8_utils.py:250-254): up to half a unit in the last place of the product, 2^-8 of it
     check_fp8_gemm(out.reshape(M, N)[rows.to(gpu)], ref + bias.float()[None, :], mag, "deepgemm linear", extra=2.0 ** -8 * ref.abs())
+    # the wrapper's one C-ABI call against its two calls through the operator entry points: the same bits
+    plain = deepgemm_w8a8_block_fp8_linear_with_fallback(x.to(gpu), w2, [128, 128], sb_words)
+    q, s = sglang_per_token_group_quant_fp8(x.to(gpu), 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True,
+                                            enable_v2=True)
+    two = w8a8_block_fp8_matmul_deepgemm(q, w2, s, sb_words, [128, 128], torch.bfloat16)
+    assert torch.equal(plain.view(torch.int16), two.view(torch.int16))
     # an fp32 block scale tensor (a checkpoint that was not re-quantized) takes the ordinary block-FP8 linear
     out2 = deepgemm_w8a8_block_fp8_linear_with_fallback(x.to(gpu), w_q.to(gpu), [128, 128], w_s.to(gpu), None, None)
     assert tuple(out2.shape) == (M, N)
