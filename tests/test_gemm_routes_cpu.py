@@ -141,8 +141,8 @@ def test_block_linear_plan():
         assert (p["quantizer"], p["kernel"]) == want, (shape, p)
         if p["quantizer"] == "launch":
             assert {k: v for k, v in p.items() if k != "quantizer"} == _lib.gemm_plan("fp8", *shape)
-    # the reference-named wrappers make the one call only where it multiplies with the GEMM entry point's kernel and tiling:
-    # any plan with a quantizer launch, and the fused plans whose kernel the GEMM entry point takes too
+    # where the one call multiplies with the GEMM entry point's kernel and tiling (any plan with a quantizer launch, and the
+    # fused plans whose kernel the GEMM entry point takes too) the reference-named wrappers equal their two calls bit for bit
     from sglang_amd.fp8_utils import _one_call_takes_the_same_gemm
 
     for shape, want in (((8, 36864, 7168), True), ((16, 2048, 7168), True), ((4, 7168, 18432), True), ((4100, 1024, 256), True),
